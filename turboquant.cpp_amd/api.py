@@ -1,0 +1,114 @@
+"""The Python entry point, in the manner of the reference's ``quantcpp.Model``
+(/root/reference/bindings/python/quantcpp/__init__.py:220-683): a model is opened from a path with keyword
+options ``temperature``, ``top_p``, ``max_tokens``, ``context_length``, generates, and is closed or used as a
+context manager.  The reference's model takes text; this one takes and returns token ids (no tokenizer is
+part of the library).
+"""
+from __future__ import annotations
+
+import os
+from typing import Iterator, Sequence
+
+from .engine.generate import GenerationOptions, GenerationResult, generate
+from .engine.model import load_model, random_model
+from .engine.step import Engine
+
+
+class Model:
+    """A loaded model ready to generate.
+
+    ``path``: a folder with ``config.json`` and ``model.safetensors``.  ``dtype``: ``"bfloat16"`` (serving
+    kernels) or ``"float32"`` (everything in true 32-bit).  ``context_length``: positions per sequence the
+    cache is sized for (0: the model's ``max_position_embeddings``, at most 4096 as in the reference,
+    /root/reference/src/engine/tq_model.c:2951).  ``max_batch``: sequences that generate together.
+    """
+
+    def __init__(self, path: str, *, temperature: float = 0.7, top_p: float = 0.9, max_tokens: int = 256,
+                 context_length: int = 0, dtype: str = "bfloat16", seed: int = 42, rep_penalty: float = 1.1,
+                 max_batch: int = 8, device: str = "cuda:0", stop_tokens: Sequence[int] | None = None):
+        if not os.path.isdir(path):
+            raise FileNotFoundError(f"model folder not found: {path}")
+        self._path = path
+        self._model = load_model(path, act=dtype, device=device)
+        self._setup(temperature, top_p, max_tokens, context_length, seed, rep_penalty, max_batch, stop_tokens)
+
+    @classmethod
+    def from_random(cls, config_json: dict, seed: int, **kw) -> "Model":
+        """A model with random weights drawn in memory from a config.json dictionary and a seed."""
+        self = cls.__new__(cls)
+        self._path = "<random>"
+        opts = dict(temperature=0.7, top_p=0.9, max_tokens=256, context_length=0, dtype="bfloat16",
+                    gen_seed=42, rep_penalty=1.1, max_batch=8, device="cuda:0", stop_tokens=None, std=0.02, norm_std=0.0)
+        opts.update(kw)
+        self._model = random_model(config_json, seed, act=opts["dtype"], device=opts["device"], std=opts["std"],
+                                   norm_std=opts["norm_std"])
+        self._setup(opts["temperature"], opts["top_p"], opts["max_tokens"], opts["context_length"], opts["gen_seed"],
+                    opts["rep_penalty"], opts["max_batch"], opts["stop_tokens"])
+        return self
+
+    def _setup(self, temperature, top_p, max_tokens, context_length, seed, rep_penalty, max_batch, stop_tokens):
+        plan = self._model.plan
+        ctx = context_length if context_length > 0 else min(plan.max_positions, 4096)
+        ctx = min(ctx, plan.max_positions)
+        self.context_length = ctx
+        self.options = GenerationOptions(
+            max_tokens=max_tokens, temperature=temperature, top_p=top_p, seed=seed, rep_penalty=rep_penalty,
+            stop_tokens=tuple(stop_tokens) if stop_tokens is not None else tuple(plan.stop_tokens), max_batch=max_batch)
+        page = 64
+        per_seq = -(-ctx // page) * page
+        self._engine = Engine(self._model, max_tokens=per_seq * max_batch, page_size=page, max_slots=max_batch)
+
+    # ------------------------------------------------------------ generation
+    def generate(self, prompts, **overrides) -> list[list[int]]:
+        """Token ids in, token ids out.  ``prompts`` is one list of ids or a list of such lists."""
+        return [r.tokens for r in self.generate_detailed(prompts, **overrides)] if _is_batch(prompts) \
+            else self.generate_detailed([prompts], **overrides)[0].tokens
+
+    def generate_detailed(self, prompts, **overrides) -> list[GenerationResult]:
+        self._ensure_open()
+        opts = GenerationOptions(**{**self.options.__dict__, **overrides})
+        return generate(self._engine, [list(p) for p in prompts], opts)
+
+    def stream(self, prompt: Sequence[int], **overrides) -> Iterator[int]:
+        """Yields the tokens of one continuation (the reference's ``generate`` yields text pieces)."""
+        yield from self.generate(list(prompt), **overrides)
+
+    # ------------------------------------------------------------ lower level, for tests and tools
+    @property
+    def engine(self) -> Engine:
+        self._ensure_open()
+        return self._engine
+
+    @property
+    def path(self) -> str:
+        return self._path
+
+    @property
+    def config(self):
+        return self._model.config
+
+    def close(self) -> None:
+        self._engine = None
+        self._model = None
+
+    def _ensure_open(self) -> None:
+        if self._model is None:
+            raise ValueError("model has been closed")
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def __repr__(self):
+        return f"Model(path={self._path!r}, open={self._model is not None})"
+
+
+def _is_batch(prompts) -> bool:
+    return len(prompts) > 0 and isinstance(prompts[0], (list, tuple))
+
+
+def load(path: str, **kw) -> Model:
+    """Same as ``Model(path, **kw)`` (/root/reference/bindings/python/quantcpp/__init__.py:679-683)."""
+    return Model(path, **kw)

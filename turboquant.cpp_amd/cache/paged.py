@@ -1,0 +1,300 @@
+"""The cache: a slot for each live sequence, keys and values of every layer in pages, and state of
+fixed size per sequence.
+
+The reference keeps one run state per sequence with flat ``[layers][max_seq][kv_dim]`` arrays
+(/root/reference/src/engine/tq_transformer.c:208-281) and, beside them, recurrent state of fixed size
+(``delta_state``, ``conv_state``, tq_transformer.c:290-313); its block cache in ``src/cache`` hands out
+blocks on demand with create / append / seq_len / free calls and status checks
+(/root/reference/src/cache/tq_paged_cache.c:35-243).  This cache serves many sequences at once:
+
+* A *slot* stands for one live sequence: its length, its pages, its row of every state tensor.
+  Slots are opened when a batch starts, closed when its sequence ends, and handed out again.
+* Keys and values live in *pages* of ``page_size`` positions.  Layers whose needs agree (kv heads,
+  head size, window) form a *group* with storage of its own: one pool of pages, each page holding the
+  rows of all the group's layers for ``page_size`` positions of one sequence, laid out
+  ``[layer][kv head][row][head_dim]``.  A group that keeps a window gives back the pages that have
+  fallen out of every later token's window, so its sequences hold pages for the window only.
+* The page table of a group, ``[slot][logical page] -> page`` (-1: none), lives on the device and is
+  updated only when pages change hands; kernels find a token's rows through its slot.
+* A schedule entry that reads another entry's cache gets a view of that entry's storage and none
+  of its own.
+
+All bookkeeping is on the host and independent of the device, so it is tested without one.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+
+
+class CacheError(RuntimeError):
+    pass
+
+
+class CacheFull(CacheError):
+    """No page or slot is free for what was asked."""
+
+
+class PagePool:
+    """Free list of the pages of one group."""
+
+    def __init__(self, n_pages: int):
+        self.n_pages = n_pages
+        self._free = list(range(n_pages - 1, -1, -1))   # pop() hands out low numbers first
+        self._held = bytearray(n_pages)
+
+    @property
+    def n_free(self) -> int:
+        return len(self._free)
+
+    def take(self, n: int) -> list[int]:
+        if n > len(self._free):
+            raise CacheFull(f"cache needs {n} more pages, {len(self._free)} of {self.n_pages} are free")
+        pages = [self._free.pop() for _ in range(n)]
+        for p in pages:
+            self._held[p] = 1
+        return pages
+
+    def give_back(self, pages) -> None:
+        for p in pages:
+            if not 0 <= p < self.n_pages or not self._held[p]:
+                raise CacheError(f"page {p} is given back but is not held")
+            self._held[p] = 0
+            self._free.append(p)
+
+
+@dataclass(frozen=True)
+class GroupKey:
+    num_kv_heads: int
+    head_dim: int
+    window: int | None
+
+
+@dataclass
+class KVView:
+    """What a mixer needs to reach its keys and values."""
+    k_pages: torch.Tensor | None      # flat pool of the group
+    v_pages: torch.Tensor | None
+    table: torch.Tensor | None        # int32 [slots, logical pages]
+    layer_offset: int                 # offset of the layer's rows inside a page, in elements
+    page_size: int
+    page_stride: int                  # elements per page
+    window: int | None
+    owns: bool                        # False: this run reads another run's keys and values and writes none
+
+
+class CacheGroup:
+    def __init__(self, key: GroupKey, entries: list[int], n_pages: int, page_size: int, max_slots: int,
+                 max_pages_per_seq: int, dtype: torch.dtype, device):
+        self.key = key
+        self.entries = entries
+        self.page_size = page_size
+        self.layer_elems = key.num_kv_heads * page_size * key.head_dim
+        self.page_stride = len(entries) * self.layer_elems
+        self.pool = PagePool(n_pages)
+        self.max_pages_per_seq = max_pages_per_seq
+        self.host_table = np.full((max_slots, max_pages_per_seq), -1, dtype=np.int32)
+        self.dirty: set[int] = set()
+        self.device = device
+        if device is not None:
+            self.k_pages = torch.empty(n_pages * self.page_stride, dtype=dtype, device=device)
+            self.v_pages = torch.empty(n_pages * self.page_stride, dtype=dtype, device=device)
+            self.table = torch.full((max_slots, max_pages_per_seq), -1, dtype=torch.int32, device=device)
+        else:   # bookkeeping only
+            self.k_pages = self.v_pages = self.table = None
+
+    def offset_of(self, entry: int) -> int:
+        return self.entries.index(entry) * self.layer_elems
+
+    def first_needed_page(self, length: int) -> int:
+        """Lowest logical page that a token at position >= length can still attend to."""
+        if self.key.window is None:
+            return 0
+        return max(0, length - self.key.window + 1) // self.page_size
+
+    def sync(self) -> None:
+        """Sends the rows of the page table that changed to the device."""
+        if not self.dirty or self.table is None:
+            self.dirty.clear()
+            return
+        rows = sorted(self.dirty)
+        idx = torch.tensor(rows, dtype=torch.int64, device=self.device)
+        self.table[idx] = torch.from_numpy(self.host_table[rows]).to(self.device)
+        self.dirty.clear()
+
+
+@dataclass
+class Slot:
+    index: int
+    length: int = 0
+    live: bool = False
+    reserved: int = 0                 # positions reserved beyond length by the running step
+
+
+class PagedCache:
+    """Slots, page groups and per-sequence state for one model.
+
+    ``needs``: for every schedule entry ``(cache_need or None, state_need or None, cache_of or None)``.
+    ``max_tokens``: the most positions live sequences hold at once, each rounded up to whole pages.
+    """
+
+    def __init__(self, needs, max_tokens: int, dtype: torch.dtype, device, page_size: int = 64,
+                 max_slots: int | None = None, max_positions: int | None = None):
+        if page_size < 1 or max_tokens < 1:
+            raise CacheError("page_size and max_tokens must be positive")
+        self.page_size = page_size
+        self.n_pages = -(-max_tokens // page_size)
+        self.max_slots = min(self.n_pages, 4096) if max_slots is None else max_slots
+        per_seq = self.n_pages if max_positions is None else min(self.n_pages, -(-max_positions // page_size))
+        self.max_positions = per_seq * page_size
+        self.dtype, self.device = dtype, device
+        self.slots = [Slot(i) for i in range(self.max_slots)]
+        self._free_slots = list(range(self.max_slots - 1, -1, -1))
+
+        by_key: dict[GroupKey, list[int]] = {}
+        self._entry_group: dict[int, tuple[CacheGroup, int, bool]] = {}
+        self._needs = list(needs)
+        for e, (cache_need, _state, cache_of) in enumerate(self._needs):
+            if cache_need is not None and cache_of is None:
+                by_key.setdefault(GroupKey(cache_need.num_kv_heads, cache_need.head_dim, cache_need.window), []).append(e)
+        self.groups: list[CacheGroup] = [
+            CacheGroup(key, entries, self.n_pages, page_size, self.max_slots, per_seq, dtype, device)
+            for key, entries in by_key.items()]
+        for g in self.groups:
+            for e in g.entries:
+                self._entry_group[e] = (g, g.offset_of(e), True)
+        for e, (cache_need, _state, cache_of) in enumerate(self._needs):
+            if cache_need is not None and cache_of is not None:
+                if cache_of not in self._entry_group or not self._entry_group[cache_of][2]:
+                    raise CacheError(f"schedule entry {e} reads the cache of entry {cache_of}, which keeps none of its own")
+                g, off, _ = self._entry_group[cache_of]
+                src = self._needs[cache_of][0]
+                if (src.num_kv_heads, src.head_dim) != (cache_need.num_kv_heads, cache_need.head_dim):
+                    raise CacheError(f"schedule entry {e} reads the cache of entry {cache_of} but their head counts or sizes differ")
+                if src.window is not None and (cache_need.window is None or cache_need.window > src.window):
+                    raise CacheError(f"schedule entry {e} looks further back than entry {cache_of}, whose cache it reads, keeps")
+                self._entry_group[e] = (g, off, False)
+
+        self.states: dict[int, torch.Tensor] = {}
+        for e, (_cache, state_need, _of) in enumerate(self._needs):
+            if state_need is not None and device is not None:
+                self.states[e] = torch.zeros((self.max_slots, *state_need.shape), dtype=state_need.dtype, device=device)
+
+    # ------------------------------------------------------------ slots
+    @property
+    def n_live(self) -> int:
+        return self.max_slots - len(self._free_slots)
+
+    def open(self) -> int:
+        """A slot for a new sequence of length 0 with zeroed state."""
+        if not self._free_slots:
+            raise CacheFull(f"all {self.max_slots} slots hold live sequences")
+        i = self._free_slots.pop()
+        s = self.slots[i]
+        s.length, s.live, s.reserved = 0, True, 0
+        for st in self.states.values():
+            st[i].zero_()
+        return i
+
+    def close(self, slot: int) -> None:
+        """Ends a sequence: its pages and its slot go back."""
+        s = self._live(slot)
+        for g in self.groups:
+            row = g.host_table[slot]
+            held = row[row >= 0]
+            if held.size:
+                g.pool.give_back(held.tolist())
+                row[:] = -1
+                g.dirty.add(slot)
+        s.live, s.length, s.reserved = False, 0, 0
+        self._free_slots.append(slot)
+
+    def length(self, slot: int) -> int:
+        return self._live(slot).length
+
+    def _live(self, slot: int) -> Slot:
+        if not 0 <= slot < self.max_slots or not self.slots[slot].live:
+            raise CacheError(f"slot {slot} holds no live sequence")
+        return self.slots[slot]
+
+    # ------------------------------------------------------------ a step's positions
+    def reserve(self, slot: int, n_new: int) -> int:
+        """Makes room for positions length .. length+n_new-1 in every group; returns the first of them."""
+        s = self._live(slot)
+        if s.reserved:
+            raise CacheError(f"slot {slot} already has positions reserved for a running step")
+        end = s.length + n_new
+        if end > self.max_positions:
+            raise CacheFull(f"sequence in slot {slot} would reach {end} positions, the cache holds {self.max_positions} per sequence")
+        first_page, last_page = s.length // self.page_size, (end - 1) // self.page_size
+        for g in self.groups:
+            row = g.host_table[slot]
+            missing = [p for p in range(first_page, last_page + 1) if row[p] < 0]
+            if missing:
+                try:
+                    pages = g.pool.take(len(missing))
+                except CacheFull:
+                    self._undo_reserve(slot, g)
+                    raise
+                row[missing] = pages
+                g.dirty.add(slot)
+        s.reserved = n_new
+        return s.length
+
+    def _undo_reserve(self, slot: int, failed: CacheGroup) -> None:
+        s = self.slots[slot]
+        keep_upto = (s.length - 1) // self.page_size if s.length else -1
+        for g in self.groups:
+            if g is failed:
+                break
+            row = g.host_table[slot]
+            extra = [p for p in range(keep_upto + 1, g.max_pages_per_seq) if row[p] >= 0]
+            if extra:
+                g.pool.give_back(row[extra].tolist())
+                row[extra] = -1
+                g.dirty.add(slot)
+
+    def commit(self, slot: int) -> None:
+        """The step that reserved positions has run: they now count, and pages that no later token's
+        window reaches go back to their pool."""
+        s = self._live(slot)
+        s.length += s.reserved
+        s.reserved = 0
+        for g in self.groups:
+            first = g.first_needed_page(s.length)
+            if first > 0:
+                row = g.host_table[slot]
+                old = [p for p in range(first) if row[p] >= 0]
+                if old:
+                    g.pool.give_back(row[old].tolist())
+                    row[old] = -1
+                    g.dirty.add(slot)
+
+    def sync(self) -> None:
+        for g in self.groups:
+            g.sync()
+
+    # ------------------------------------------------------------ views
+    def kv(self, entry: int) -> KVView:
+        if entry not in self._entry_group:
+            raise CacheError(f"schedule entry {entry} keeps no keys and values")
+        g, off, owns = self._entry_group[entry]
+        return KVView(g.k_pages, g.v_pages, g.table, off, g.page_size, g.page_stride, self._needs[entry][0].window, owns)
+
+    def state(self, entry: int) -> torch.Tensor:
+        if entry not in self.states:
+            raise CacheError(f"schedule entry {entry} keeps no per-sequence state")
+        return self.states[entry]
+
+    def pages_held(self) -> dict[int, int]:
+        """Pages in use per group index."""
+        return {i: g.pool.n_pages - g.pool.n_free for i, g in enumerate(self.groups)}
+
+    def bytes(self) -> int:
+        n = 0
+        for g in self.groups:
+            if g.k_pages is not None:
+                n += 2 * g.k_pages.numel() * g.k_pages.element_size()
+        return n

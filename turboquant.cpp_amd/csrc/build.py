@@ -1,0 +1,150 @@
+"""Compiles the HIP sources of this folder for gfx950 into one shared library per activation type.
+
+The library lies in ``csrc/_build/`` next to the sources (or, where that folder cannot be written,
+in a per-user folder under the temporary directory) and carries a hash of its sources and flags in
+its name, so a library built from other sources is never loaded by mistake.
+"""
+from __future__ import annotations
+
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import time
+
+CSRC = os.path.dirname(os.path.abspath(__file__))
+
+# sources per activation type; the matrix-core kernels exist for bfloat16 only
+COMMON_SOURCES = ["elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "moe.hip", "sampling.hip"]
+SOURCES = {
+    "float32": COMMON_SOURCES,
+    "bfloat16": COMMON_SOURCES + ["gemm_mfma.hip", "attention_mfma.hip"],
+}
+HEADERS = ["common.h", "mfma.h"]
+DEFINES = {"float32": "-DTQ_ACT_F32", "bfloat16": "-DTQ_ACT_BF16"}
+FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-fno-gpu-rdc",
+         # keep the compiler from forming packed 32-bit float instructions
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+class BuildError(RuntimeError):
+    pass
+
+
+def _existing(names):
+    return [n for n in names if os.path.isfile(os.path.join(CSRC, n))]
+
+
+def _hash(dtype: str) -> str:
+    h = hashlib.sha256()
+    h.update(" ".join(FLAGS + [DEFINES[dtype]]).encode())
+    for name in _existing(SOURCES[dtype]) + _existing(HEADERS):
+        h.update(name.encode())
+        with open(os.path.join(CSRC, name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:12]
+
+
+def _build_dirs() -> list[str]:
+    return [os.path.join(CSRC, "_build"),
+            os.path.join(tempfile.gettempdir(), f"turboquant_cpp_amd_build_{os.getuid()}")]
+
+
+def library_name(dtype: str) -> str:
+    return f"libtq_{dtype}-{_hash(dtype)}.so"
+
+
+def find_library(dtype: str) -> str | None:
+    """The built library that matches the present sources, or None."""
+    name = library_name(dtype)
+    for d in _build_dirs():
+        p = os.path.join(d, name)
+        if os.path.isfile(p):
+            return p
+    return None
+
+
+def _hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.isfile(cand):
+            return cand
+    raise BuildError("hipcc not found (looked at $HIPCC, PATH and /opt/rocm/bin/hipcc): the gfx950 kernels cannot be built")
+
+
+def _writable_dir() -> str:
+    for d in _build_dirs():
+        try:
+            os.makedirs(d, exist_ok=True)
+            probe = os.path.join(d, f".probe{os.getpid()}")
+            with open(probe, "w"):
+                pass
+            os.remove(probe)
+            return d
+        except OSError:
+            continue
+    raise BuildError("no writable folder for the built library: tried " + ", ".join(_build_dirs()))
+
+
+def build(dtype: str, force: bool = False, verbose: bool = True) -> str:
+    """Compiles the library for one activation type and returns its path."""
+    if dtype not in SOURCES:
+        raise BuildError(f"unknown activation type {dtype!r}")
+    if not force:
+        found = find_library(dtype)
+        if found:
+            return found
+    hipcc = _hipcc()
+    out_dir = _writable_dir()
+    target = os.path.join(out_dir, library_name(dtype))
+    obj_dir = os.path.join(out_dir, f"obj_{dtype}_{os.getpid()}")
+    os.makedirs(obj_dir, exist_ok=True)
+    say = (lambda m: print(f"[turboquant] {m}", file=sys.stderr, flush=True)) if verbose else (lambda m: None)
+    sources = _existing(SOURCES[dtype])
+    say(f"compiling {len(sources)} HIP sources for gfx950 ({dtype}) into {target}")
+    t0 = time.time()
+    procs = []
+    for src in sources:
+        obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
+        cmd = [hipcc, *FLAGS, DEFINES[dtype], "-c", os.path.join(CSRC, src), "-o", obj]
+        procs.append((src, obj, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+    objs = []
+    pending = list(procs)
+    last = time.time()
+    while pending:
+        for item in list(pending):
+            src, obj, p = item
+            if p.poll() is None:
+                continue
+            out = p.stdout.read()
+            pending.remove(item)
+            if p.returncode != 0:
+                for _, _, q in pending:
+                    q.kill()
+                raise BuildError(f"hipcc failed on {src}:\n{out}")
+            say(f"  compiled {src} ({time.time() - t0:.0f}s)")
+            objs.append(obj)
+        if pending:
+            time.sleep(0.2)
+            if time.time() - last > 10:
+                say(f"  still compiling: {', '.join(s for s, _, _ in pending)} ({time.time() - t0:.0f}s)")
+                last = time.time()
+    tmp = target + f".tmp{os.getpid()}"
+    link = subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *sorted(objs), "-o", tmp],
+                          stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if link.returncode != 0:
+        raise BuildError(f"hipcc failed to link {target}:\n{link.stdout}")
+    os.replace(tmp, target)
+    shutil.rmtree(obj_dir, ignore_errors=True)
+    say(f"built {os.path.basename(target)} in {time.time() - t0:.0f}s")
+    return target
+
+
+def build_all(force: bool = True, verbose: bool = True) -> list[str]:
+    return [build(d, force=force, verbose=verbose) for d in SOURCES]
+
+
+if __name__ == "__main__":
+    for path in build_all():
+        print(path)

@@ -1,0 +1,171 @@
+// Row-wise kernels: embedding rows, residual sum + RMS norm, rotary position encoding with
+// the write of keys and values into cache pages, and the weighted sum of expert outputs.
+// All of them are bound by memory traffic; each fuses what would otherwise be a second pass.
+#include "common.h"
+
+// ---------------------------------------------------------------- embedding
+// x[t, :] = table[tokens[t], :] widened to float, no scaling
+// (/root/reference/src/engine/tq_transformer.c:2297-2329).
+template <class W>
+__global__ void embed_kernel(const int* __restrict__ tokens, const W* __restrict__ table,
+                             float* __restrict__ x, int H) {
+  const int t = blockIdx.x;
+  const W* row = table + (size_t)tokens[t] * H;
+  float* out = x + (size_t)t * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = to_f32(row[i]);
+}
+
+TQ_API int tq_embed(const int* tokens, const void* table, int wtype, float* x, int T, int H, hipStream_t st) {
+  if (T <= 0) return 0;
+  TQ_DISPATCH_W(wtype, { hipLaunchKernelGGL(embed_kernel<W>, dim3(T), dim3(256), 0, st, tokens, (const W*)table, x, H); });
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------- residual sum + RMS norm
+// For row r (token rows[r], or r itself when rows is null):
+//   v = x[row] + sum_s delta[s][row]            (the residual sum, in float, s ascending)
+//   x[row] = v                                  (only when rows is null)
+//   ss = sum v^2 / H + eps ; out = (v * (1/sqrt(ss))) * w
+// Formula and product order of /root/reference/src/engine/tq_ops.c:1373-1410.
+// The sum of squares is taken in a fixed order that does not depend on the number of rows.
+template <class W>
+__global__ void add_rmsnorm_kernel(float* __restrict__ x, const float* __restrict__ delta, int S,
+                                   size_t delta_stride, const W* __restrict__ w, float eps,
+                                   const int* __restrict__ rows, act_t* __restrict__ out,
+                                   float* __restrict__ out32, int H) {
+  extern __shared__ float v[];       // H floats, then one float per wave
+  float* red = v + H;
+  const int r = blockIdx.x;
+  const int row = rows ? rows[r] : r;
+  float* xr = x + (size_t)row * H;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float a = xr[i];
+    for (int s = 0; s < S; ++s) a += delta[s * delta_stride + (size_t)row * H + i];
+    v[i] = a;
+    if (!rows) xr[i] = a;
+    ss += a * a;
+  }
+  ss = block_sum(ss, red);
+  ss = ss / (float)H + eps;
+  const float rs = 1.0f / sqrtf(ss);
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const float o = v[i] * rs * to_f32(w[i]);
+    if (out) out[(size_t)r * H + i] = from_f32<act_t>(o);
+    if (out32) out32[(size_t)r * H + i] = o;
+  }
+}
+
+TQ_API int tq_add_rmsnorm(float* x, const float* delta, int S, int64_t delta_stride, const void* w, int wtype,
+                          float eps, const int* rows, int R, void* out, float* out32, int H, hipStream_t st) {
+  if (R <= 0) return 0;
+  const int threads = 256;
+  const size_t shmem = (size_t)(H + threads / TQ_WAVE) * sizeof(float);
+  if (shmem > 160 * 1024) return TQ_ERR_UNSUPPORTED;
+  TQ_DISPATCH_W(wtype, {
+    if (shmem > 48 * 1024)
+      hipFuncSetAttribute((const void*)add_rmsnorm_kernel<W>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+    hipLaunchKernelGGL(add_rmsnorm_kernel<W>, dim3(R), dim3(threads), shmem, st, x, delta, S, (size_t)delta_stride,
+                       (const W*)w, eps, rows, (act_t*)out, out32, H);
+  });
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------- rotary encoding + cache write
+// qkv[t] holds, in float, nh query heads, then nkv key heads, then nkv value heads of hd each.
+// Queries and keys are rotated by angle pos * inv_freq[i] (float) on the pair
+//   pairing 0 ("half"):        (x[i], x[i + rot/2])   (/root/reference/src/engine/tq_transformer.c:1263-1289)
+//   pairing 1 ("interleaved"): (x[2i], x[2i+1])        (/root/reference/src/engine/tq_ops.c:1418-1448)
+// as (a, b) <- (a cos - b sin, a sin + b cos); dimensions from rot on pass through.  Rotated queries
+// go to q_out; rotated keys and the values go into the page that holds position pos of the token's
+// sequence: page = block_table[seq][pos / page_size], row pos % page_size of kv head h, laid out
+// [page][kv head][row][hd] after the layer's own offset (already added to k_pool / v_pool).
+__global__ void rope_kv_write_kernel(const float* __restrict__ qkv, const int* __restrict__ positions,
+                                     const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
+                                     int bt_stride, const float* __restrict__ inv_freq, int pairing, int rot,
+                                     act_t* __restrict__ q_out, act_t* __restrict__ k_pool,
+                                     act_t* __restrict__ v_pool, int page_size, int64_t page_stride, int nh,
+                                     int nkv, int hd, int write_kv) {
+  const int t = blockIdx.x;
+  const int slot = blockIdx.y;          // 0..nh-1 query heads, then key heads, then value heads
+  const int pos = positions[t];
+  const float* src = qkv + ((size_t)t * (nh + 2 * nkv) + slot) * hd;
+  act_t* dst;
+  bool rotate = true;
+  if (slot < nh) {
+    dst = q_out + ((size_t)t * nh + slot) * hd;
+  } else {
+    if (!write_kv) return;
+    const int kvh = (slot - nh) % nkv;
+    const bool is_v = slot >= nh + nkv;
+    const int page = block_table[(size_t)seq_of_token[t] * bt_stride + pos / page_size];
+    act_t* pool = is_v ? v_pool : k_pool;
+    dst = pool + (size_t)page * page_stride + ((size_t)kvh * page_size + pos % page_size) * hd;
+    rotate = !is_v;
+  }
+  if (!rotate) {
+    for (int i = threadIdx.x; i < hd; i += blockDim.x) dst[i] = from_f32<act_t>(src[i]);
+    return;
+  }
+  const int half = rot / 2;
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    const float theta = (float)pos * inv_freq[i];
+    float sn, cs;
+    sincosf(theta, &sn, &cs);
+    const int ia = pairing == 0 ? i : 2 * i;
+    const int ib = pairing == 0 ? i + half : 2 * i + 1;
+    const float a = src[ia], b = src[ib];
+    dst[ia] = from_f32<act_t>(a * cs - b * sn);
+    dst[ib] = from_f32<act_t>(a * sn + b * cs);
+  }
+  for (int i = rot + threadIdx.x; i < hd; i += blockDim.x) dst[i] = from_f32<act_t>(src[i]);
+}
+
+TQ_API int tq_rope_kv_write(const float* qkv, const int* positions, const int* seq_of_token,
+                            const int* block_table, int bt_stride, const float* inv_freq, int pairing, int rot,
+                            void* q_out, void* k_pool, void* v_pool, int page_size, int64_t page_stride, int T,
+                            int nh, int nkv, int hd, int write_kv, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (rot < 0 || rot > hd || (rot & 1) || (pairing != 0 && pairing != 1)) return TQ_ERR_BAD_ARG;
+  hipLaunchKernelGGL(rope_kv_write_kernel, dim3(T, nh + 2 * nkv), dim3(64), 0, st, qkv, positions, seq_of_token,
+                     block_table, bt_stride, inv_freq, pairing, rot, (act_t*)q_out, (act_t*)k_pool, (act_t*)v_pool,
+                     page_size, page_stride, nh, nkv, hd, write_kv);
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------- sum of expert outputs
+// out[t] = sum_j weights[t][j] * y[slot[t][j]]   (j ascending: the order in which experts were selected,
+//          /root/reference/src/engine/tq_moe.c:720,864-999)
+//        + gate[t] * sum_s shared[s][t]           (shared expert last, tq_moe.c:1005-1058)
+__global__ void moe_combine_kernel(const float* __restrict__ y, const int* __restrict__ pair_slot,
+                                   const float* __restrict__ weights, int topk, const float* __restrict__ shared,
+                                   int S, size_t shared_stride, const float* __restrict__ gate,
+                                   float* __restrict__ out, int H) {
+  const int t = blockIdx.x;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float acc = 0.f;
+    for (int j = 0; j < topk; ++j) {
+      const int p = pair_slot[t * topk + j];
+      acc += weights[t * topk + j] * y[(size_t)p * H + i];
+    }
+    if (shared) {
+      float sh = 0.f;
+      for (int s = 0; s < S; ++s) sh += shared[s * shared_stride + (size_t)t * H + i];
+      acc += (gate ? gate[t] : 1.0f) * sh;
+    }
+    out[(size_t)t * H + i] = acc;
+  }
+}
+
+TQ_API int tq_moe_combine(const float* y, const int* pair_slot, const float* weights, int topk,
+                          const float* shared, int S, int64_t shared_stride, const float* gate, float* out, int T,
+                          int H, hipStream_t st) {
+  if (T <= 0) return 0;
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(256), 0, st, y, pair_slot, weights, topk, shared, S,
+                     (size_t)shared_stride, gate, out, H);
+  TQ_LAUNCH_CHECK();
+  return 0;
+}

@@ -1,0 +1,385 @@
+"""Python face of the HIP kernels: one function per kernel, on torch tensors that live on the GPU.
+
+Every function checks on the host that shapes, types and strides are what its kernel and launch
+grid assume before anything is launched, and raises :class:`KernelError` with the kernel's name
+otherwise.  There is no other implementation behind these functions: without a GPU, or without
+the compiled library, they raise.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+
+import torch
+
+from . import build as _build
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+ACT_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+_WTYPE = {torch.float32: 0, torch.bfloat16: 1}
+_LIBS: dict[str, ctypes.CDLL] = {}
+
+_c_int, _c_i64, _c_f32, _c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
+
+_SIGNATURES = {
+    "tq_embed": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr],
+    "tq_add_rmsnorm": [_c_ptr, _c_ptr, _c_int, _c_i64, _c_ptr, _c_int, _c_f32, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr],
+    "tq_rope_kv_write": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
+                         _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "tq_moe_combine": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
+    "tq_gemm_generic": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int,
+                        _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "tq_attention_generic": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_i64, _c_int, _c_int,
+                             _c_int, _c_int, _c_int, _c_f32, _c_ptr, _c_ptr],
+    "tq_router_topk": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
+    "tq_moe_align": [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+    "tq_argmax": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr],
+    "tq_rep_penalty": [_c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_ptr, _c_f32, _c_ptr],
+    "tq_sample_topp": [_c_ptr, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+}
+# entry points that only the bfloat16 library has
+_OPTIONAL = {
+    "tq_gemm_mfma": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int,
+                     _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+}
+
+
+def dtype_name(dtype) -> str:
+    if isinstance(dtype, str):
+        if dtype in ("float32", "f32", "fp32"):
+            return "float32"
+        if dtype in ("bfloat16", "bf16"):
+            return "bfloat16"
+    elif dtype == torch.float32:
+        return "float32"
+    elif dtype == torch.bfloat16:
+        return "bfloat16"
+    raise KernelError(f"no kernels for activation type {dtype!r}: float32 and bfloat16 are built")
+
+
+def library(dtype) -> ctypes.CDLL:
+    """The compiled kernels for one activation type; builds them at the first call if they are not there."""
+    name = dtype_name(dtype)
+    lib = _LIBS.get(name)
+    if lib is not None:
+        return lib
+    if not torch.cuda.is_available():
+        raise KernelError("no GPU is visible: the kernels of this library run on gfx950 only and have no CPU form")
+    path = _build.find_library(name) or _build.build(name)
+    try:
+        lib = ctypes.CDLL(path)
+    except OSError as e:
+        raise KernelError(f"cannot load the kernel library {path}: {e}") from e
+    for fn, sig in _SIGNATURES.items():
+        f = getattr(lib, fn)
+        f.argtypes, f.restype = sig, _c_int
+    for fn, sig in _OPTIONAL.items():
+        if hasattr(lib, fn):
+            f = getattr(lib, fn)
+            f.argtypes, f.restype = sig, _c_int
+    _LIBS[name] = lib
+    return lib
+
+
+def has_kernel(dtype, name: str) -> bool:
+    return hasattr(library(dtype), name)
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def _need(cond: bool, kernel: str, what: str) -> None:
+    if not cond:
+        raise KernelError(f"{kernel}: {what}")
+
+
+def _check(t: torch.Tensor, kernel: str, name: str, dtype=None, shape=None) -> None:
+    _need(isinstance(t, torch.Tensor) and t.is_cuda, kernel, f"{name} must be a GPU tensor")
+    _need(t.is_contiguous(), kernel, f"{name} must be contiguous, has strides {t.stride()}")
+    if dtype is not None:
+        ok = t.dtype in dtype if isinstance(dtype, (tuple, list)) else t.dtype == dtype
+        _need(ok, kernel, f"{name} must be {dtype}, is {t.dtype}")
+    if shape is not None:
+        _need(tuple(t.shape) == tuple(shape), kernel, f"{name} must have shape {tuple(shape)}, has {tuple(t.shape)}")
+
+
+def _run(kernel: str, code: int) -> None:
+    if code == 0:
+        return
+    if code == -1:
+        raise KernelError(f"{kernel}: arguments rejected by the launcher")
+    if code == -2:
+        raise KernelError(f"{kernel}: size not supported by this kernel")
+    raise KernelError(f"{kernel}: HIP error {code} at launch")
+
+
+# ------------------------------------------------------------------ row-wise kernels
+def embed(tokens: torch.Tensor, table: torch.Tensor, act) -> torch.Tensor:
+    """x[t] = table[tokens[t]] as float32 [T, H]."""
+    k = "embed"
+    _check(tokens, k, "tokens", torch.int32)
+    _need(tokens.dim() == 1 and table.dim() == 2, k, "tokens [T], table [V, H]")
+    _check(table, k, "table", tuple(_WTYPE))
+    T, (V, H) = tokens.numel(), table.shape
+    x = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    _run(k, library(act).tq_embed(_ptr(tokens), _ptr(table), _WTYPE[table.dtype], _ptr(x), T, H, _stream()))
+    return x
+
+
+def add_rmsnorm(x: torch.Tensor, delta: torch.Tensor | None, weight: torch.Tensor, eps: float, act,
+                rows: torch.Tensor | None = None, want_act: bool = True, want_f32: bool = False):
+    """x += sum_s delta[s] (in place, unless ``rows`` picks rows); returns rmsnorm(x) * weight as
+    (activation-typed or None, float32 or None), one row per entry of ``rows`` (all rows if None)."""
+    k = "add_rmsnorm"
+    _check(x, k, "x", torch.float32)
+    _need(x.dim() == 2, k, "x must be [T, H]")
+    T, H = x.shape
+    _check(weight, k, "weight", tuple(_WTYPE), (H,))
+    S, stride = 0, 0
+    if delta is not None:
+        _check(delta, k, "delta", torch.float32)
+        _need(delta.dim() == 3 and tuple(delta.shape[1:]) == (T, H), k, f"delta must be [S, {T}, {H}], is {tuple(delta.shape)}")
+        S, stride = delta.shape[0], T * H
+    R = T
+    if rows is not None:
+        _check(rows, k, "rows", torch.int32)
+        _need(rows.dim() == 1, k, "rows must be [R]")
+        R = rows.numel()
+    adt = ACT_DTYPES[dtype_name(act)]
+    out = torch.empty((R, H), dtype=adt, device=x.device) if want_act else None
+    out32 = torch.empty((R, H), dtype=torch.float32, device=x.device) if want_f32 else None
+    _run(k, library(act).tq_add_rmsnorm(_ptr(x), _ptr(delta), S, stride, _ptr(weight), _WTYPE[weight.dtype],
+                                        float(eps), _ptr(rows), R, _ptr(out), _ptr(out32), H, _stream()))
+    return out, out32
+
+
+def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor,
+                  inv_freq: torch.Tensor, pairing: int, rotary_dim: int, k_pages: torch.Tensor | None,
+                  v_pages: torch.Tensor | None, layer_offset: int, page_size: int, page_stride: int,
+                  num_heads: int, num_kv_heads: int, head_dim: int, act) -> torch.Tensor:
+    """Rotates queries and keys, returns the queries [T, nh*hd] and writes keys and values into the pages.
+    ``k_pages``/``v_pages`` are the flat page pools of the cache group (None: nothing is written, for a
+    layer that reads another layer's cache); ``layer_offset`` is the layer's offset inside a page."""
+    k = "rope_kv_write"
+    T = positions.numel()
+    width = (num_heads + 2 * num_kv_heads) * head_dim
+    _check(qkv, k, "qkv", torch.float32, (T, width))
+    _check(positions, k, "positions", torch.int32, (T,))
+    _check(seq_of_token, k, "seq_of_token", torch.int32, (T,))
+    _check(block_table, k, "block_table", torch.int32)
+    _need(block_table.dim() == 2, k, "block_table must be [B, pages]")
+    _check(inv_freq, k, "inv_freq", torch.float32)
+    _need(inv_freq.numel() * 2 == rotary_dim or rotary_dim == 0, k, f"inv_freq must hold rotary_dim/2 = {rotary_dim // 2} entries")
+    adt = ACT_DTYPES[dtype_name(act)]
+    q = torch.empty((T, num_heads * head_dim), dtype=adt, device=qkv.device)
+    write = k_pages is not None
+    kp = vp = None
+    if write:
+        _check(k_pages, k, "k_pages", adt)
+        _check(v_pages, k, "v_pages", adt)
+        _need(layer_offset + num_kv_heads * page_size * head_dim <= page_stride, k, "layer does not fit in a page")
+        esz = k_pages.element_size()
+        kp, vp = k_pages.data_ptr() + layer_offset * esz, v_pages.data_ptr() + layer_offset * esz
+    _run(k, library(act).tq_rope_kv_write(_ptr(qkv), _ptr(positions), _ptr(seq_of_token), _ptr(block_table),
+                                          block_table.shape[1], _ptr(inv_freq), pairing, rotary_dim, _ptr(q), kp, vp,
+                                          page_size, page_stride, T, num_heads, num_kv_heads, head_dim, int(write),
+                                          _stream()))
+    return q
+
+
+def moe_combine(y: torch.Tensor, pair_slot: torch.Tensor, weights: torch.Tensor, shared: torch.Tensor | None,
+                shared_gate: torch.Tensor | None, act) -> torch.Tensor:
+    """out[t] = sum_j weights[t, j] * y[pair_slot[t, j]] + shared_gate[t] * sum_s shared[s, t]; float32 [1, T, H]."""
+    k = "moe_combine"
+    _check(y, k, "y", torch.float32)
+    T, topk = pair_slot.shape
+    H = y.shape[1]
+    _check(pair_slot, k, "pair_slot", torch.int32)
+    _check(weights, k, "weights", torch.float32, (T, topk))
+    S, stride = 0, 0
+    if shared is not None:
+        _check(shared, k, "shared", torch.float32)
+        _need(shared.dim() == 3 and tuple(shared.shape[1:]) == (T, H), k, f"shared must be [S, {T}, {H}]")
+        S, stride = shared.shape[0], T * H
+    if shared_gate is not None:
+        _check(shared_gate, k, "shared_gate", torch.float32, (T,))
+    out = torch.empty((1, T, H), dtype=torch.float32, device=y.device)
+    _run(k, library(act).tq_moe_combine(_ptr(y), _ptr(pair_slot), _ptr(weights), topk, _ptr(shared), S, stride,
+                                        _ptr(shared_gate), _ptr(out), T, H, _stream()))
+    return out
+
+
+# ------------------------------------------------------------------ matrix products
+def _use_mfma(act, a: torch.Tensor, w: torch.Tensor, K: int) -> bool:
+    return (dtype_name(act) == "bfloat16" and w.dtype == torch.bfloat16 and K % 8 == 0
+            and has_kernel(act, "tq_gemm_mfma"))
+
+
+def gemm(a: torch.Tensor, w: torch.Tensor, act, bias: torch.Tensor | None = None, w2: torch.Tensor | None = None,
+         out_act: bool = False, a_rows: torch.Tensor | None = None, tile_group: torch.Tensor | None = None,
+         n_tiles: torch.Tensor | None = None, tile_rows: int | None = None, gather: bool = True) -> torch.Tensor:
+    """out[m, n] = sum_k a[row(m), k] * w[g, n, k]  (+ bias[n]);  with ``w2``: silu(a w^T) * (a w2^T).
+
+    ``a`` [M, K] activations.  ``w`` [N, K], or [G, N, K] with ``tile_group`` naming the matrix of each tile of
+    ``tile_rows`` output rows and ``a_rows`` [P] the row of ``a`` behind each output row (-1: none; with
+    ``gather`` false a live output row m reads row m of ``a``).
+    Output is float32 unless ``out_act``.  Sums run over k in ascending order whatever M is.
+    """
+    k = "gemm"
+    adt = ACT_DTYPES[dtype_name(act)]
+    _check(a, k, "a", adt)
+    _need(a.dim() == 2, k, "a must be [M, K]")
+    K = a.shape[1]
+    _check(w, k, "w", tuple(_WTYPE))
+    grouped = tile_group is not None
+    if grouped:
+        _need(w.dim() == 3 and w.shape[2] == K, k, f"grouped w must be [G, N, {K}], is {tuple(w.shape)}")
+        _need(a_rows is not None and n_tiles is not None and tile_rows in (16, 64), k,
+              "grouped product needs a_rows, n_tiles and tile_rows of 16 or 64")
+        _check(a_rows, k, "a_rows", torch.int32)
+        _check(tile_group, k, "tile_group", torch.int32)
+        _check(n_tiles, k, "n_tiles", torch.int32)
+        M = a_rows.numel()
+        _need(M % tile_rows == 0 and tile_group.numel() >= M // tile_rows, k, "a_rows must hold whole tiles, each with a group")
+        N = w.shape[1]
+        gstride = N * K
+    else:
+        _need(w.dim() == 2 and w.shape[1] == K, k, f"w must be [N, {K}], is {tuple(w.shape)}")
+        N = w.shape[0]
+        M = a.shape[0] if a_rows is None else a_rows.numel()
+        if a_rows is not None:
+            _check(a_rows, k, "a_rows", torch.int32)
+        gstride = 0
+        if tile_rows is None:
+            tile_rows = 16 if M <= 32 else 64
+    if w2 is not None:
+        _check(w2, k, "w2", w.dtype, tuple(w.shape))
+    if bias is not None:
+        _check(bias, k, "bias", tuple(_WTYPE), (N,))
+    out = torch.empty((M, N), dtype=adt if out_act else torch.float32, device=a.device)
+    lib = library(act)
+    if _use_mfma(act, a, w, K) and (bias is None or bias.dtype in _WTYPE):
+        _run("gemm_mfma", lib.tq_gemm_mfma(_ptr(a), a.stride(0), _ptr(a_rows), int(gather), _ptr(w), _ptr(w2), gstride,
+                                           _ptr(tile_group), _ptr(n_tiles), _ptr(bias),
+                                           _WTYPE[bias.dtype] if bias is not None else 0, _ptr(out), N, int(out_act),
+                                           M, N, K, tile_rows, _stream()))
+        return out
+    _run(k, lib.tq_gemm_generic(_ptr(a), a.stride(0), _ptr(a_rows), int(gather), _ptr(w), _ptr(w2), _WTYPE[w.dtype], gstride,
+                                _ptr(tile_group), _ptr(n_tiles), _ptr(bias),
+                                _WTYPE[bias.dtype] if bias is not None else 0, _ptr(out), N, int(out_act), M, N, K,
+                                tile_rows, _stream()))
+    return out
+
+
+# ------------------------------------------------------------------ attention
+def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, layer_offset: int,
+              positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor, page_size: int,
+              page_stride: int, num_heads: int, num_kv_heads: int, head_dim: int, window: int | None,
+              scale: float, act) -> torch.Tensor:
+    """Each token attends to its sequence's cached positions up to its own; returns [T, nh*hd]."""
+    k = "attention"
+    adt = ACT_DTYPES[dtype_name(act)]
+    T = positions.numel()
+    _check(q, k, "q", adt, (T, num_heads * head_dim))
+    _check(k_pages, k, "k_pages", adt)
+    _check(v_pages, k, "v_pages", adt)
+    _check(positions, k, "positions", torch.int32, (T,))
+    _check(seq_of_token, k, "seq_of_token", torch.int32, (T,))
+    _check(block_table, k, "block_table", torch.int32)
+    _need(block_table.dim() == 2, k, "block_table must be [B, pages]")
+    _need(num_heads % num_kv_heads == 0, k, "heads must be a multiple of kv heads")
+    _need(head_dim <= 512, k, f"head size {head_dim} is beyond the 512 this kernel takes")
+    _need(layer_offset + num_kv_heads * page_size * head_dim <= page_stride, k, "layer does not fit in a page")
+    out = torch.empty_like(q)
+    esz = k_pages.element_size()
+    _run(k, library(act).tq_attention_generic(_ptr(q), k_pages.data_ptr() + layer_offset * esz,
+                                              v_pages.data_ptr() + layer_offset * esz, _ptr(positions),
+                                              _ptr(seq_of_token), _ptr(block_table), block_table.shape[1], page_size,
+                                              page_stride, T, num_heads, num_kv_heads, head_dim, int(window or 0),
+                                              float(scale), _ptr(out), _stream()))
+    return out
+
+
+# ------------------------------------------------------------------ routing
+def router_topk(x32: torch.Tensor, router: torch.Tensor, shared_scale: torch.Tensor | None, top_k: int,
+                renormalize: bool, act):
+    """ids int32 [T, k], weights float32 [T, k], and sigmoid(x . shared_scale) float32 [T] (or None)."""
+    k = "router_topk"
+    _check(x32, k, "x", torch.float32)
+    T, H = x32.shape
+    _check(router, k, "router", tuple(_WTYPE))
+    _need(router.dim() == 2 and router.shape[1] == H, k, f"router must be [E, {H}]")
+    E = router.shape[0]
+    _need(1 <= top_k <= min(E, 64), k, f"top_k {top_k} must be within 1..min(E, 64)")
+    if shared_scale is not None:
+        _check(shared_scale, k, "shared_scale", router.dtype)
+        _need(shared_scale.numel() == H, k, f"shared_scale must hold {H} values")
+    ids = torch.empty((T, top_k), dtype=torch.int32, device=x32.device)
+    weights = torch.empty((T, top_k), dtype=torch.float32, device=x32.device)
+    gate = torch.empty((T,), dtype=torch.float32, device=x32.device) if shared_scale is not None else None
+    _run(k, library(act).tq_router_topk(_ptr(x32), _ptr(router), _ptr(shared_scale), _WTYPE[router.dtype], E, top_k,
+                                        int(bool(renormalize)), _ptr(ids), _ptr(weights), _ptr(gate), T, H, _stream()))
+    return ids, weights, gate
+
+
+def moe_align(ids: torch.Tensor, num_experts: int, unit: int, act):
+    """Orders the (token, expert) pairs by expert.  Returns sorted_token [cap], pair_slot [T, k],
+    tile_expert [cap/unit], n_tiles [1]; each expert's rows start at a multiple of ``unit``."""
+    k = "moe_align"
+    _check(ids, k, "ids", torch.int32)
+    T, topk = ids.shape
+    n_pairs = T * topk
+    # every expert with at least one pair wastes at most unit-1 rows
+    cap = n_pairs + min(num_experts, n_pairs) * (unit - 1)
+    cap = (cap + unit - 1) // unit * unit
+    dev = ids.device
+    sorted_token = torch.empty((cap,), dtype=torch.int32, device=dev)
+    pair_slot = torch.empty((T, topk), dtype=torch.int32, device=dev)
+    tile_expert = torch.empty((cap // unit,), dtype=torch.int32, device=dev)
+    n_tiles = torch.empty((1,), dtype=torch.int32, device=dev)
+    _run(k, library(act).tq_moe_align(_ptr(ids), n_pairs, num_experts, topk, unit, cap, _ptr(sorted_token),
+                                      _ptr(pair_slot), _ptr(tile_expert), _ptr(n_tiles), _stream()))
+    return sorted_token, pair_slot, tile_expert, n_tiles
+
+
+# ------------------------------------------------------------------ sampling
+def argmax(logits: torch.Tensor, act) -> torch.Tensor:
+    k = "argmax"
+    _check(logits, k, "logits", torch.float32)
+    R, V = logits.shape
+    out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    _run(k, library(act).tq_argmax(_ptr(logits), R, V, _ptr(out), _stream()))
+    return out
+
+
+def rep_penalty(logits: torch.Tensor, recent: torch.Tensor, counts: torch.Tensor, penalty: float, act) -> None:
+    k = "rep_penalty"
+    _check(logits, k, "logits", torch.float32)
+    R, V = logits.shape
+    _check(recent, k, "recent", torch.int32)
+    _need(recent.dim() == 2 and recent.shape[0] == R, k, f"recent must be [{R}, window]")
+    _check(counts, k, "counts", torch.int32, (R,))
+    _run(k, library(act).tq_rep_penalty(_ptr(logits), R, V, _ptr(recent), recent.shape[1], _ptr(counts),
+                                        float(penalty), _stream()))
+
+
+def sample_topp(logits: torch.Tensor, temperature: float, top_p: float, uniforms: torch.Tensor, act) -> torch.Tensor:
+    k = "sample_topp"
+    _check(logits, k, "logits", torch.float32)
+    R, V = logits.shape
+    _check(uniforms, k, "uniforms", torch.float32, (R,))
+    _need(temperature > 0 and top_p > 0, k, "temperature and top_p must be positive (else use argmax)")
+    probs = torch.empty((R, V), dtype=torch.float32, device=logits.device)
+    out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    _run(k, library(act).tq_sample_topp(_ptr(logits), R, V, float(temperature), float(top_p), _ptr(uniforms),
+                                        _ptr(probs), _ptr(out), _stream()))
+    return out

@@ -1,0 +1,150 @@
+"""The generation loop: batches of prompts of unequal length, stop tokens, sequences that end early.
+
+The reference's loop serves one prompt (/root/reference/src/engine/tq_generate.c:167-643): prefill, sample;
+then, while fewer than ``max_tokens`` tokens are out: stop on an end token (:426-446) without emitting it,
+emit, run the token, apply the repetition penalty, sample, and stop when the same 4-gram has come three
+times (:611-629).  Here the same decisions are taken per sequence of a batch: all prompts of a batch run
+in one step, then every live sequence decodes one token per step; a sequence that ends gives its slot
+and pages back at once and the others go on; when more requests wait than a batch holds, batch follows
+batch.  The decisions are kept apart from the device work (``Decision`` and ``SequenceTrack``) so that
+they are tested without one.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Callable, Sequence
+
+from ..sampling.sampler import Sampler, SamplingOptions
+
+
+@dataclass
+class GenerationOptions:
+    max_tokens: int = 256                     # reference default (tq_ops.c:1883-1897)
+    temperature: float = 0.7
+    top_p: float = 0.9
+    seed: int = 42
+    rep_penalty: float = 1.1
+    rep_window: int = 32
+    stop_tokens: tuple[int, ...] = ()
+    loop_detection: bool = True               # stop when a 4-gram has repeated three times
+    max_batch: int = 8
+    on_token: Callable[[int, int], None] | None = None   # (request index, token)
+
+    def sampling(self) -> SamplingOptions:
+        return SamplingOptions(self.temperature, self.top_p, self.seed, self.rep_penalty, self.rep_window)
+
+
+@dataclass
+class GenerationResult:
+    tokens: list[int]
+    finish_reason: str            # "stop" (end token), "length" (max_tokens), "context" (cache or model limit), "loop"
+
+
+class LoopDetector:
+    """Hash of the last four tokens kept in a ring of 64; three earlier occurrences end the sequence
+    (/root/reference/src/engine/tq_generate.c:611-629)."""
+
+    def __init__(self):
+        self.hashes: list[int] = []
+        self.count = 0
+
+    def push(self, recent: Sequence[int]) -> bool:
+        if len(recent) < 4:
+            return False
+        h = 0
+        for t in recent[-4:]:
+            h = (h * 31 + t) & 0xFFFFFFFF
+        ring = self.hashes[:64]
+        matches = sum(1 for x in ring if x == h)
+        if len(self.hashes) < 64:
+            self.hashes.append(h)
+        else:
+            self.hashes[self.count % 64] = h
+        self.count += 1
+        return matches >= 3
+
+
+@dataclass
+class SequenceTrack:
+    """The decisions for one sequence: what to do with each sampled token."""
+    request: int
+    prompt_len: int
+    options: GenerationOptions
+    max_positions: int
+    out: list[int] = field(default_factory=list)
+    history: list[int] = field(default_factory=list)    # prompt tail and sampled tokens, for the loop detector
+    detector: LoopDetector = field(default_factory=LoopDetector)
+    finish_reason: str | None = None
+
+    def accept(self, token: int) -> bool:
+        """Takes the sampled token.  Returns True if the token is to be run through the model next,
+        False if the sequence has ended (``finish_reason`` says why)."""
+        o = self.options
+        self.history.append(token)
+        looped = o.loop_detection and self.detector.push(self.history)
+        if token in o.stop_tokens:
+            self.finish_reason = "stop"          # the end token is not emitted
+            return False
+        self.out.append(token)
+        if o.on_token is not None:
+            o.on_token(self.request, token)
+        if len(self.out) >= o.max_tokens:
+            self.finish_reason = "length"
+            return False
+        if looped:
+            self.finish_reason = "loop"
+            return False
+        if self.prompt_len + len(self.out) >= self.max_positions:
+            self.finish_reason = "context"       # no room for another position; the reference would shift (:456-514)
+            return False
+        return True
+
+
+def plan_batches(n_requests: int, max_batch: int) -> list[list[int]]:
+    """Requests in order, ``max_batch`` at a time."""
+    if max_batch < 1:
+        raise ValueError("max_batch must be at least 1")
+    return [list(range(i, min(i + max_batch, n_requests))) for i in range(0, n_requests, max_batch)]
+
+
+def generate(engine, prompts: Sequence[Sequence[int]], options: GenerationOptions | None = None) -> list[GenerationResult]:
+    """Generates a continuation for every prompt (lists of token ids)."""
+    o = options or GenerationOptions()
+    if any(len(p) == 0 for p in prompts):
+        raise ValueError("every prompt needs at least one token")
+    if o.max_tokens < 1:
+        return [GenerationResult([], "length") for _ in prompts]
+    stop = tuple(o.stop_tokens)
+    sampler = Sampler(o.sampling(), engine.model.act, engine.device)
+    results: list[GenerationResult | None] = [None] * len(prompts)
+    max_pos = engine.cache.max_positions
+    for batch in plan_batches(len(prompts), o.max_batch):
+        too_long = [r for r in batch if len(prompts[r]) > max_pos]
+        for r in too_long:
+            results[r] = GenerationResult([], "context")
+        batch = [r for r in batch if r not in too_long]
+        if not batch:
+            continue
+        slots = engine.open(len(batch))
+        tracks = {r: SequenceTrack(r, len(prompts[r]), o, max_pos) for r in batch}
+        samp = {r: sampler.new_sequence(r, list(prompts[r])) for r in batch}
+        slot_of = dict(zip(batch, slots))
+        live = list(batch)
+        try:
+            logits = engine.step([slot_of[r] for r in live], [list(prompts[r]) for r in live])
+            while True:
+                tokens = sampler.sample(logits, [samp[r] for r in live])
+                going = []
+                for r, t in zip(live, tokens):
+                    if tracks[r].accept(t):
+                        going.append((r, t))
+                    else:
+                        engine.close([slot_of.pop(r)])
+                        results[r] = GenerationResult(tracks[r].out, tracks[r].finish_reason)
+                if not going:
+                    break
+                live = [r for r, _ in going]
+                logits = engine.step([slot_of[r] for r in live], [[t] for _, t in going])
+        finally:
+            engine.close(list(slot_of.values()))
+    return results

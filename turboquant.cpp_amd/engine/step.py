@@ -1,0 +1,90 @@
+"""The step function: runs the next tokens of a batch of sequences, from the cache, and returns the logits
+at the wanted places.
+
+The reference steps one token of one sequence (``tq_forward``, /root/reference/src/engine/tq_transformer.c:2281)
+and its multi-token path serves one sequence and no experts (``tq_forward_batch``, :3049-3083).  Here a
+step takes any set of live sequences, each with its own next tokens (a whole prompt, or one decoded
+token) and its own length; the tokens run as one packed batch without padding, every token at position
+``length of its sequence + its place``, and afterwards the lengths have grown by what was run.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..cache.paged import CacheError
+from .batch import pack_step
+from .context import StepContext
+from .model import CausalLM
+
+
+class StepError(ValueError):
+    pass
+
+
+class Engine:
+    """A model with its cache.  ``max_tokens`` is the most positions that live sequences hold at once,
+    each sequence rounded up to whole pages of ``page_size``."""
+
+    def __init__(self, model: CausalLM, max_tokens: int, page_size: int = 64, max_slots: int | None = None):
+        self.model = model
+        self.cache = model.new_cache(max_tokens, page_size=page_size, max_slots=max_slots)
+        self.device = model.device
+        self.vocab_size = model.plan.vocab_size
+
+    # ------------------------------------------------------------ sequences
+    def open(self, n: int = 1) -> list[int]:
+        """Slots for ``n`` new sequences."""
+        slots = []
+        try:
+            for _ in range(n):
+                slots.append(self.cache.open())
+        except CacheError:
+            for s in slots:
+                self.cache.close(s)
+            raise
+        return slots
+
+    def close(self, slots) -> None:
+        for s in slots:
+            self.cache.close(s)
+
+    def length(self, slot: int) -> int:
+        return self.cache.length(slot)
+
+    # ------------------------------------------------------------ the step
+    def step(self, slots: list[int], token_lists: list[list[int]], wants: list[list[int]] | None = None) -> torch.Tensor:
+        """Runs ``token_lists[i]`` as the next tokens of the sequence in ``slots[i]``.
+
+        ``wants[i]`` lists the places among those tokens whose logits are returned (default: the last).
+        Returns float32 logits [number of wanted places, vocab] in the order of the sequences and of
+        their wanted places."""
+        if len(slots) != len(token_lists) or not slots:
+            raise StepError("a step needs as many token lists as slots, and at least one")
+        if len(set(slots)) != len(slots):
+            raise StepError("a slot appears twice in one step")
+        if wants is None:
+            wants = [[len(t) - 1] for t in token_lists]
+        V = self.vocab_size
+        for i, toks in enumerate(token_lists):
+            if len(toks) == 0:
+                raise StepError(f"sequence {i} of the step brings no token")
+            bad = [t for t in toks if not 0 <= t < V]
+            if bad:
+                raise StepError(f"sequence {i} brings token {bad[0]}, outside the vocabulary of {V}")
+        starts, reserved = [], []
+        try:
+            for slot, toks in zip(slots, token_lists):
+                starts.append(self.cache.reserve(slot, len(toks)))
+                reserved.append(slot)
+        except CacheError:
+            for slot in reserved:
+                s = self.cache.slots[slot]
+                s.reserved = 0
+            raise
+        self.cache.sync()
+        batch = pack_step(slots, starts, token_lists, wants, self.device)
+        ctx = StepContext(batch=batch, cache=self.cache, act=self.model.act, device=self.device)
+        logits = self.model.forward(ctx)
+        for slot in slots:
+            self.cache.commit(slot)
+        return logits

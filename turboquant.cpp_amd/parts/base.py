@@ -1,0 +1,108 @@
+"""What every part of a layer has in common, and the registries parts are chosen from.
+
+A part is built from a :class:`~..config.plan.PartSpec`: a kind (the registry key), arguments (its sizes
+and constants) and the checkpoint tensors behind its parameters.  It declares its parameters with
+:class:`ParamSpec`, receives them as device tensors, and does its work through the kernels in
+``csrc.ops``.  A part never looks at the model or the architecture it is used in.
+
+Interfaces (``ctx`` is the :class:`~..engine.context.StepContext` of the running step):
+
+* norm      ``forward(x, delta, ctx, rows=None, want_f32=False) -> (normed, normed32)``: adds the pending
+            ``delta`` [S, T, H] float32 into the residual stream ``x`` [T, H] float32 and returns the normalised
+            rows in the activation type (and in float32 if asked).
+* mixer     ``forward(normed, ctx, entry) -> delta``: mixes tokens of each sequence; ``entry`` is the index of
+            the schedule entry that runs, by which it finds its cache (``ctx.kv(entry)``) or its fixed-size
+            state (``ctx.state(entry)``).  ``cache_need()`` / ``state_need()`` say what storage each run wants.
+* ffn       ``forward(normed, normed32, ctx) -> delta``; ``wants_f32`` says whether it reads the float32 copy.
+* position  ``table(device)``, ``pairing``, ``rotary_dim``: the rotation a mixer applies to queries and keys.
+* block     ``forward(x, pending, ctx, entry) -> pending``: the arrangement of norms, mixer and ffn around
+            the residual stream.
+
+``delta`` is always float32 [S, T, H]: S partial results that the next norm adds to the stream in order.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any, Callable
+
+import torch
+
+from ..config.plan import PartSpec
+
+
+@dataclass(frozen=True)
+class ParamSpec:
+    """One parameter: its shape, its role (``matrix``, ``bias``, ``scale`` for norm weights, ``table`` for
+    embeddings) and, if it is several checkpoint tensors joined along dimension 0, their sizes there."""
+    shape: tuple[int, ...]
+    role: str = "matrix"
+    splits: tuple[int, ...] | None = None
+
+
+@dataclass(frozen=True)
+class CacheNeed:
+    """Keys and values per position: ``window`` None keeps all positions, else the last ``window``."""
+    num_kv_heads: int
+    head_dim: int
+    window: int | None = None
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """State of fixed size per sequence, zero when a sequence starts."""
+    shape: tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+class Part:
+    category: str = ""
+    kind: str = ""
+
+    def param_specs(self) -> dict[str, ParamSpec]:
+        return {}
+
+    def children(self) -> dict[str, "Part"]:
+        return {}
+
+    def set_params(self, tensors: dict[str, torch.Tensor]) -> None:
+        for name, t in tensors.items():
+            setattr(self, name, t)
+
+    def prepare(self, device, act: str) -> None:
+        """Called once after the parameters are on the device."""
+
+
+_REGISTRIES: dict[str, dict[str, Callable[..., Part]]] = {
+    "norm": {}, "mixer": {}, "ffn": {}, "position": {}, "block": {},
+}
+
+
+def register_part(category: str, kind: str):
+    """Class decorator: makes a part available to model plans under ``kind``."""
+    if category not in _REGISTRIES:
+        raise ValueError(f"unknown part category {category!r}; known: {sorted(_REGISTRIES)}")
+
+    def deco(cls):
+        if kind in _REGISTRIES[category]:
+            raise ValueError(f"{category} {kind!r} is already registered")
+        cls.category, cls.kind = category, kind
+        _REGISTRIES[category][kind] = cls
+        return cls
+    return deco
+
+
+def unregister_part(category: str, kind: str) -> None:
+    _REGISTRIES[category].pop(kind, None)
+
+
+def known_parts(category: str) -> list[str]:
+    return sorted(_REGISTRIES[category])
+
+
+def build_part(category: str, spec: PartSpec) -> Part:
+    try:
+        cls = _REGISTRIES[category][spec.kind]
+    except KeyError:
+        raise ValueError(f"unknown {category} {spec.kind!r}; known: {', '.join(known_parts(category))}") from None
+    args: dict[str, Any] = dict(spec.args)
+    return cls(**args)

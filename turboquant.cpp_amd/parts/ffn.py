@@ -1,0 +1,74 @@
+"""Feed-forward parts: a dense gated one and a sparse one with routed experts and a shared expert.
+
+Dense (/root/reference/src/engine/tq_transformer.c:2707-2824): ``down(silu(gate x) * (up x))``, no biases.
+Sparse (/root/reference/src/engine/tq_moe.c:600-1059): router logits in float32, top-k with the highest index
+winning ties, weights from a softmax; every chosen expert is the dense formula with its own matrices, summed
+with its weight in the order chosen; the shared expert, scaled by ``sigmoid(x . shared_scale)``, is added
+last.  ``renormalize`` false keeps the softmax over all experts un-normalised for the chosen ones; true is
+the reference's softmax over the chosen logits.
+"""
+from __future__ import annotations
+
+from ..csrc import ops
+from .base import ParamSpec, Part, register_part
+
+
+@register_part("ffn", "dense_swiglu")
+class DenseSwiGLU(Part):
+    wants_f32 = False
+
+    def __init__(self, hidden_size: int, inner_size: int):
+        self.hidden_size, self.inner_size = hidden_size, inner_size
+        self.gate = self.up = self.down = None
+
+    def param_specs(self):
+        return {"gate": ParamSpec((self.inner_size, self.hidden_size)),
+                "up": ParamSpec((self.inner_size, self.hidden_size)),
+                "down": ParamSpec((self.hidden_size, self.inner_size))}
+
+    def forward(self, normed, normed32, ctx):
+        h = ops.gemm(normed, self.gate, ctx.act, w2=self.up, out_act=True)
+        return ops.gemm(h, self.down, ctx.act).unsqueeze(0)
+
+
+@register_part("ffn", "moe_swiglu")
+class SparseMoE(Part):
+    wants_f32 = True    # the router reads the normalised activations in float32
+
+    def __init__(self, hidden_size: int, num_experts: int, top_k: int, expert_size: int, shared_size: int = 0,
+                 shared_gated: bool = True, renormalize: bool = False):
+        if not 1 <= top_k <= num_experts:
+            raise ValueError(f"top_k {top_k} must be within 1..num_experts {num_experts}")
+        self.hidden_size, self.num_experts, self.top_k = hidden_size, num_experts, top_k
+        self.expert_size, self.shared_size = expert_size, shared_size
+        self.shared_gated, self.renormalize = shared_gated and shared_size > 0, renormalize
+        self.router = self.expert_gate = self.expert_up = self.expert_down = None
+        self.shared_gate = self.shared_up = self.shared_down = self.shared_scale = None
+
+    def param_specs(self):
+        E, H, I, S = self.num_experts, self.hidden_size, self.expert_size, self.shared_size
+        specs = {"router": ParamSpec((E, H)),
+                 "expert_gate": ParamSpec((E, I, H)), "expert_up": ParamSpec((E, I, H)),
+                 "expert_down": ParamSpec((E, H, I))}
+        if S > 0:
+            specs.update({"shared_gate": ParamSpec((S, H)), "shared_up": ParamSpec((S, H)),
+                          "shared_down": ParamSpec((H, S))})
+            if self.shared_gated:
+                specs["shared_scale"] = ParamSpec((1, H))
+        return specs
+
+    def forward(self, normed, normed32, ctx):
+        T = normed.shape[0]
+        ids, weights, gate = ops.router_topk(normed32, self.router, self.shared_scale if self.shared_gated else None,
+                                             self.top_k, self.renormalize, ctx.act)
+        unit = 16 if T * self.top_k <= 16 * self.num_experts else 64
+        sorted_token, pair_slot, tile_expert, n_tiles = ops.moe_align(ids, self.num_experts, unit, ctx.act)
+        h = ops.gemm(normed, self.expert_gate, ctx.act, w2=self.expert_up, out_act=True, a_rows=sorted_token,
+                     tile_group=tile_expert, n_tiles=n_tiles, tile_rows=unit)
+        y = ops.gemm(h, self.expert_down, ctx.act, a_rows=sorted_token, tile_group=tile_expert, n_tiles=n_tiles,
+                     tile_rows=unit, gather=False)
+        shared = None
+        if self.shared_size > 0:
+            hs = ops.gemm(normed, self.shared_gate, ctx.act, w2=self.shared_up, out_act=True)
+            shared = ops.gemm(hs, self.shared_down, ctx.act).unsqueeze(0)
+        return ops.moe_combine(y, pair_slot, weights, shared, gate, ctx.act)

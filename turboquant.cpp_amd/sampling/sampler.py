@@ -1,0 +1,74 @@
+"""Choice of the next token of every sequence of a step, on the GPU.
+
+The reference's order (/root/reference/src/engine/tq_generate.c:386-410, :587-603): repetition penalty over
+the last ``rep_window`` tokens (prompt tail included), then ``tq_sample_topp``: greedy when temperature
+or top_p is not positive (:84-86), else temperature and top-p with one uniform draw per token.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+
+from ..csrc import ops
+from .rng import XorShift64Star, stream_seed
+
+
+@dataclass
+class SamplingOptions:
+    temperature: float = 0.7
+    top_p: float = 0.9
+    seed: int = 42
+    rep_penalty: float = 1.1
+    rep_window: int = 32
+
+    @property
+    def greedy(self) -> bool:
+        return self.temperature <= 0.0 or self.top_p <= 0.0
+
+
+@dataclass
+class SequenceSampling:
+    """What sampling remembers of one sequence: its random stream and its recent tokens."""
+    rng: XorShift64Star
+    recent: list[int] = field(default_factory=list)
+
+    def push(self, token: int, keep: int) -> None:
+        self.recent.append(token)
+        if len(self.recent) > max(keep, 128):
+            del self.recent[:len(self.recent) - max(keep, 128)]
+
+
+class Sampler:
+    def __init__(self, options: SamplingOptions, act: str, device):
+        self.options, self.act, self.device = options, act, device
+        self.window = max(0, min(options.rep_window, 128))    # the reference caps the window at 128 (:367)
+
+    def new_sequence(self, index: int, prompt: list[int]) -> SequenceSampling:
+        st = SequenceSampling(XorShift64Star(stream_seed(self.options.seed, index)))
+        st.recent = list(prompt[-self.window:]) if self.window else []
+        return st
+
+    def sample(self, logits: torch.Tensor, states: list[SequenceSampling]) -> list[int]:
+        """One token per row of ``logits`` [R, V]; row i belongs to ``states[i]``.  Changes ``logits``
+        when a repetition penalty applies."""
+        o, R = self.options, logits.shape[0]
+        if o.rep_penalty > 1.0 and self.window > 0:
+            recent = np.full((R, self.window), -1, dtype=np.int32)
+            counts = np.zeros(R, dtype=np.int32)
+            for i, st in enumerate(states):
+                tail = st.recent[-self.window:][::-1]      # newest first, the reference's order
+                recent[i, :len(tail)] = tail
+                counts[i] = len(tail)
+            ops.rep_penalty(logits, torch.from_numpy(recent).to(self.device), torch.from_numpy(counts).to(self.device),
+                            o.rep_penalty, self.act)
+        if o.greedy:
+            ids = ops.argmax(logits, self.act)
+        else:
+            u = np.array([st.rng.next_float() for st in states], dtype=np.float32)
+            ids = ops.sample_topp(logits, o.temperature, o.top_p, torch.from_numpy(u).to(self.device), self.act)
+        out = ids.tolist()
+        for st, t in zip(states, out):
+            st.push(t, self.window)
+        return out
