@@ -1,0 +1,189 @@
+"""Decode and prefill throughput of the engine on one MI355X, at Qwen1.5-MoE-A2.7B layer sizes with random weights.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C]
+
+A step is one decode step of the whole batch: the step function, greedy sampling on the GPU and the copy of the
+chosen tokens to the host, exactly what the generation loop runs.  Prints one JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# Qwen1.5-MoE-A2.7B layer sizes
+A27B = {
+    "architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe",
+    "vocab_size": 151936, "hidden_size": 2048, "num_hidden_layers": 24, "num_attention_heads": 16,
+    "num_key_value_heads": 16, "intermediate_size": 5632, "moe_intermediate_size": 1408,
+    "shared_expert_intermediate_size": 5632, "num_experts": 60, "num_experts_per_tok": 4, "norm_topk_prob": False,
+    "decoder_sparse_step": 1, "mlp_only_layers": [], "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
+    "use_sliding_window": False, "sliding_window": 32768, "max_window_layers": 24, "max_position_embeddings": 8192,
+    "tie_word_embeddings": False, "torch_dtype": "bfloat16",
+}
+FULL_LAYERS = 24
+PEAK_HBM_GBS = 8000.0
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+PREFILL_TOKENS = 2048
+
+
+def layer_weight_elems(c, experts_used: float) -> float:
+    H, Q = c["hidden_size"], c["num_attention_heads"] * (c["hidden_size"] // c["num_attention_heads"])
+    KV = c["num_key_value_heads"] * (c["hidden_size"] // c["num_attention_heads"])
+    attn = H * (Q + 2 * KV) + (Q + 2 * KV) + Q * H
+    moe = c["num_experts"] * H + H + 3 * H * c["shared_expert_intermediate_size"] + experts_used * 3 * H * c["moe_intermediate_size"]
+    return attn + moe + 2 * H
+
+
+def decode_bytes(c, layers: int, batch: int, context: float, wbytes: int = 2) -> float:
+    """Bytes a decode step has to read: every weight it uses once (the experts that a batch of random tokens
+    reaches, in expectation) and the keys and values of the live requests."""
+    E, k = c["num_experts"], c["num_experts_per_tok"]
+    used = E * (1.0 - (1.0 - k / E) ** batch)
+    hd = c["hidden_size"] // c["num_attention_heads"]
+    w = layers * layer_weight_elems(c, used) + c["vocab_size"] * c["hidden_size"] + c["hidden_size"]
+    kv = batch * context * layers * 2 * c["num_key_value_heads"] * hd
+    return wbytes * (w + kv)
+
+
+def prefill_flops(c, layers: int, T: int, rows_out: int = 1) -> float:
+    H, nh = c["hidden_size"], c["num_attention_heads"]
+    hd = H // nh
+    Q, KV = nh * hd, c["num_key_value_heads"] * hd
+    per_layer = (2 * T * H * (Q + 2 * KV) + 2 * T * Q * H + 4 * nh * hd * T * (T + 1) / 2
+                 + 2 * T * H * (c["num_experts"] + 1)
+                 + 2 * T * c["num_experts_per_tok"] * 3 * H * c["moe_intermediate_size"]
+                 + 2 * T * 3 * H * c["shared_expert_intermediate_size"])
+    return layers * per_layer + 2 * rows_out * H * c["vocab_size"]
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=FULL_LAYERS)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=8192)
+    ap.add_argument("--points-context", type=int, default=2048)
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--no-points", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single device)")
+        return 2
+
+    import torch
+    from turboquant_cpp_amd.csrc import ops
+    from turboquant_cpp_amd.engine.model import random_model
+    from turboquant_cpp_amd.engine.step import Engine
+
+    cfg = dict(A27B)
+    cfg["num_hidden_layers"] = args.layers
+    cfg["max_window_layers"] = args.layers
+    cfg["max_position_embeddings"] = max(args.context, args.points_context, PREFILL_TOKENS)
+    act = args.dtype
+    short = "bf16" if act == "bfloat16" else "fp32"
+    dev = "cuda:0"
+    ops.library(act)
+    t0 = time.time()
+    model = random_model(cfg, seed=2, act=act, device=dev)
+    torch.cuda.synchronize()
+    print(f"[bench] {args.layers}-layer model with random weights on the device in {time.time() - t0:.1f}s "
+          f"({model.weight_bytes / 1e9:.1f} GB)", file=sys.stderr, flush=True)
+    V = cfg["vocab_size"]
+    gen = torch.Generator().manual_seed(2)
+
+    def run_decode(batch: int, context: int, steps: int, warmup: int):
+        """Prefills `batch` prompts so that the timed steps end at `context`, then times `steps` decode steps."""
+        prompt_len = context - steps - warmup - 1
+        page = 64
+        per_seq = -(-context // page) * page
+        engine = Engine(model, max_tokens=per_seq * batch, page_size=page, max_slots=batch)
+        slots = engine.open(batch)
+        prompts = [torch.randint(0, V, (prompt_len,), generator=gen).tolist() for _ in range(batch)]
+        tp = time.time()
+        logits = None
+        # prompts go in one sequence at a time to bound the size of the activations
+        for s, p in zip(slots, prompts):
+            lg = engine.step([s], [p])
+            logits = lg if logits is None else torch.cat([logits, lg])
+        torch.cuda.synchronize()
+        print(f"[bench] prefilled {batch} x {prompt_len} tokens in {time.time() - tp:.1f}s", file=sys.stderr, flush=True)
+        tokens = ops.argmax(logits, act).tolist()
+
+        def one_step(tokens):
+            lg = engine.step(slots, [[t] for t in tokens])
+            return ops.argmax(lg, act).tolist()
+
+        for _ in range(warmup):
+            tokens = one_step(tokens)
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(steps):
+            tokens = one_step(tokens)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t
+        mean_ctx = prompt_len + warmup + steps / 2.0
+        engine.close(slots)
+        del engine
+        torch.cuda.empty_cache()
+        return dt / steps, mean_ctx
+
+    def run_prefill(T: int):
+        engine = Engine(model, max_tokens=T + 64, page_size=64, max_slots=1)
+        prompt = torch.randint(0, V, (T,), generator=gen).tolist()
+        times = []
+        for i in range(3):
+            slot = engine.open(1)
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            engine.step(slot, [prompt])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t)
+            engine.close(slot)
+        del engine
+        torch.cuda.empty_cache()
+        return min(times[1:])
+
+    pf = run_prefill(PREFILL_TOKENS)
+    sec, mean_ctx = run_decode(args.batch, args.context, args.steps, args.warmup)
+    value = args.batch / sec
+    read = decode_bytes(cfg, args.layers, args.batch, mean_ctx, 2 if act == "bfloat16" else 4)
+    achieved = read / sec / 1e9
+    points = {}
+    if not args.no_points:
+        for b in (1, 64):
+            s, _ = run_decode(b, args.points_context, 32, 4)
+            points[f"decode_b{b}"] = round(b / s, 1)
+    out = {
+        "metric": "decode tok/s at batch 8, context 8192 (Qwen1.5-MoE-A2.7B layer sizes, random weights)",
+        "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": short, "data": "synthetic",
+        "config": {
+            "model": "Qwen1.5-MoE-A2.7B sizes", "layers": args.layers, "layers_of_full_model": FULL_LAYERS,
+            "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
+            "head_dim": cfg["hidden_size"] // cfg["num_attention_heads"], "vocab": V, "experts": cfg["num_experts"],
+            "top_k": cfg["num_experts_per_tok"], "expert_inner": cfg["moe_intermediate_size"],
+            "shared_inner": cfg["shared_expert_intermediate_size"], "global_batch": args.batch,
+            "seq_len": args.context, "parallelism": "single GPU", "points_context": args.points_context,
+            "prefill_tokens": PREFILL_TOKENS, "weights": "random N(0,0.02) seed 2", "kv_cache": short,
+        },
+        "prefill": {"value": round(PREFILL_TOKENS / pf, 1), "tokens": PREFILL_TOKENS, "ms": round(pf * 1e3, 3),
+                    "frac": round(prefill_flops(cfg, args.layers, PREFILL_TOKENS) / pf / PEAK_FLOPS[short], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
+        "points": points,
+    }
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

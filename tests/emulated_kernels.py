@@ -60,12 +60,13 @@ def rope_kv_write(qkv, positions, slot_of_token, block_table, inv_freq, pairing,
             for h in range(num_kv_heads):
                 o = page * page_stride + layer_offset + (h * page_size + p % page_size) * head_dim
                 k_pages[o:o + head_dim] = k[t, h]
-                v_pages[o:o + head_dim] = v[t, h]
+                ov = page * page_stride + layer_offset + h * page_size * head_dim + p % page_size
+                v_pages[ov:ov + head_dim * page_size:page_size] = v[t, h]      # values lie [hd][row]
     return q
 
 
 def attention(q, k_pages, v_pages, layer_offset, positions, slot_of_token, block_table, page_size, page_stride,
-              num_heads, num_kv_heads, head_dim, window, scale, act):
+              num_heads, num_kv_heads, head_dim, window, scale, act, runs=None):
     T = positions.numel()
     out = torch.empty_like(q)
     qf = q.float().view(T, num_heads, head_dim)
@@ -78,8 +79,9 @@ def attention(q, k_pages, v_pages, layer_offset, positions, slot_of_token, block
         for h in range(num_heads):
             kvh = h // (num_heads // num_kv_heads)
             base = pages * page_stride + layer_offset + (kvh * page_size + js % page_size) * head_dim
-            idx = base[:, None] + torch.arange(head_dim)[None, :]
-            K, V = k_pages[idx].float(), v_pages[idx].float()
+            K = k_pages[base[:, None] + torch.arange(head_dim)[None, :]].float()
+            vbase = pages * page_stride + layer_offset + kvh * page_size * head_dim + js % page_size
+            V = v_pages[vbase[:, None] + page_size * torch.arange(head_dim)[None, :]].float()
             s = (K @ qf[t, h]) * scale
             pr = torch.softmax(s, dim=0)
             out[t, h * head_dim:(h + 1) * head_dim] = (pr @ V).to(out.dtype)

@@ -1,0 +1,469 @@
+"""Each HIP kernel alone against a plain torch float32 (or float64) computation of the same operation,
+at sizes other than the engine's: widths and vocabularies that are no power of two, head sizes in steps
+of 16, odd numbers of heads and groups, rows that do not fill a tile."""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+ACTS = ["float32", "bfloat16"]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from turboquant_cpp_amd.csrc import ops as _ops
+    for a in ACTS:
+        _ops.library(a)
+    return _ops
+
+
+def adt(act):
+    return torch.float32 if act == "float32" else torch.bfloat16
+
+
+def rnd(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (scale * torch.randn(shape, generator=g)).to(dtype)
+
+
+def tol(act, scale=1.0):
+    return (2e-5 if act == "float32" else 2e-2) * scale
+
+
+# ------------------------------------------------------------------------------------------------ embed / norm
+@pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16])
+def test_embed(ops, act, wdtype):
+    if act == "float32" and wdtype != torch.float32:
+        pytest.skip("the 32-bit path keeps its weights in 32 bits")
+    table = rnd((37, 50), wdtype, 1)
+    tokens = torch.tensor([0, 36, 5, 5, 17], dtype=torch.int32)
+    x = ops.embed(tokens.to(DEV), table.to(DEV), act).cpu()
+    assert torch.equal(x, table[tokens.long()].float())
+
+
+@pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("H", [48, 200, 1000])
+def test_add_rmsnorm(ops, act, H):
+    T, S, eps = 7, 3, 1e-5
+    x = rnd((T, H), torch.float32, 2)
+    delta = rnd((S, T, H), torch.float32, 3)
+    w = rnd((H,), adt(act), 4) + 1
+    xd = x.clone().to(DEV)
+    out, out32 = ops.add_rmsnorm(xd, delta.to(DEV), w.to(DEV), eps, act, want_f32=True)
+    v = x.double() + delta.double().sum(0)
+    ref = v * (1.0 / torch.sqrt((v * v).mean(-1, keepdim=True) + eps)) * w.double()
+    assert (xd.cpu().double() - v).abs().max() < 1e-5          # the residual stream holds the sum
+    assert (out32.cpu().double() - ref).abs().max() < 1e-4
+    assert (out.cpu().double() - ref).abs().max() < tol(act, 4)
+    # picked rows: x stays as it is, rows may repeat
+    rows = torch.tensor([5, 0, 5], dtype=torch.int32)
+    xd2 = x.clone().to(DEV)
+    out_r, _ = ops.add_rmsnorm(xd2, delta.to(DEV), w.to(DEV), eps, act, rows=rows.to(DEV))
+    assert torch.equal(xd2.cpu(), x)
+    assert torch.equal(out_r.cpu(), out.cpu()[rows.long()])
+    # no pending sum: x is only normalised
+    xd3 = x.clone().to(DEV)
+    out_n, _ = ops.add_rmsnorm(xd3, None, w.to(DEV), eps, act)
+    ref_n = x.double() * (1.0 / torch.sqrt((x.double() ** 2).mean(-1, keepdim=True) + eps)) * w.double()
+    assert (out_n.cpu().double() - ref_n).abs().max() < tol(act, 4)
+
+
+# ------------------------------------------------------------------------------------------------ products
+def ref_gemm(a, w, bias=None, w2=None):
+    y = a.double() @ w.double().T
+    if bias is not None:
+        y = y + bias.double()
+    if w2 is not None:
+        y = torch.nn.functional.silu(y) * (a.double() @ w2.double().T)
+    return y
+
+
+@pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("M,N,K", [(5, 33, 50), (1, 50, 72), (5, 130, 200), (16, 64, 64), (17, 33, 136), (40, 257, 264),
+                                   (64, 96, 1000), (65, 130, 72), (200, 300, 520), (300, 129, 64)])
+@pytest.mark.parametrize("mode", ["plain", "bias", "gated"])
+def test_gemm_dense(ops, act, M, N, K, mode):
+    a = rnd((M, K), adt(act), 10)
+    w = rnd((N, K), adt(act), 11, 0.2)
+    bias = rnd((N,), adt(act), 12) if mode == "bias" else None
+    w2 = rnd((N, K), adt(act), 13, 0.2) if mode == "gated" else None
+    for out_act in (False, True):
+        y = ops.gemm(a.to(DEV), w.to(DEV), act, bias=None if bias is None else bias.to(DEV),
+                     w2=None if w2 is None else w2.to(DEV), out_act=out_act).cpu()
+        ref = ref_gemm(a, w, bias, w2)
+        scale = ref.abs().max().item()
+        err = (y.double() - ref).abs().max().item()
+        limit = 1e-5 * scale * math.sqrt(K) if act == "float32" else (2e-2 if out_act else 4e-3) * scale
+        assert err < limit, (err, scale)
+
+
+@pytest.mark.parametrize("act", ACTS)
+def test_gemm_float32_weights_on_the_bfloat16_path(ops, act):
+    """A matrix the checkpoint stores in 32 bits stays so and still multiplies."""
+    a = rnd((9, 72), adt(act), 20)
+    w = rnd((50, 72), torch.float32, 21, 0.2)
+    y = ops.gemm(a.to(DEV), w.to(DEV), act).cpu()
+    ref = ref_gemm(a, w)
+    assert (y.double() - ref).abs().max() < 1e-4 * ref.abs().max() * 10
+
+
+@pytest.mark.parametrize("act", ACTS)
+def test_gemm_rows_do_not_depend_on_the_batch(ops, act):
+    """A row's result is the same bits whether it is multiplied alone or among others (same kernel family)."""
+    K, N = 264, 130
+    a = rnd((16, K), adt(act), 30)
+    w = rnd((N, K), adt(act), 31, 0.2)
+    full = ops.gemm(a.to(DEV), w.to(DEV), act).cpu()
+    for m in (1, 3, 9):
+        part = ops.gemm(a[:m].contiguous().to(DEV), w.to(DEV), act).cpu()
+        assert torch.equal(part, full[:m])
+
+
+@pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("unit", [16, 64])
+@pytest.mark.parametrize("T,E,k,H,I", [(1, 5, 2, 72, 40), (9, 7, 3, 136, 88), (150, 6, 2, 64, 200)])
+def test_expert_products(ops, act, unit, T, E, k, H, I):
+    """Pairs ordered by expert, the gated product over gathered rows, the second product over rows in place."""
+    g = torch.Generator().manual_seed(40)
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32)
+    x = rnd((T, H), adt(act), 41)
+    wg, wu = rnd((E, I, H), adt(act), 42, 0.2), rnd((E, I, H), adt(act), 43, 0.2)
+    wd = rnd((E, H, I), adt(act), 44, 0.2)
+    st, slot, tile_e, n_tiles = ops.moe_align(ids.to(DEV), E, unit, act)
+    st_c, slot_c, tile_c, nt = st.cpu(), slot.cpu(), tile_e.cpu(), int(n_tiles.cpu())
+    # the order: every pair has its row, rows of one expert are together and in order of token, tiles are whole
+    assert sorted(slot_c.view(-1).tolist()) == [r for r in range(st_c.numel()) if st_c[r] >= 0]
+    for t in range(T):
+        for j in range(k):
+            r = int(slot_c[t, j])
+            assert int(st_c[r]) == t and int(tile_c[r // unit]) == int(ids[t, j])
+    assert nt == sum(-(-int((ids == e).sum()) // unit) for e in range(E))
+    rows_by_expert = [[r for r in range(nt * unit) if st_c[r] >= 0 and tile_c[r // unit] == e] for e in range(E)]
+    for rows in rows_by_expert:
+        assert [int(st_c[r]) for r in rows] == sorted(int(st_c[r]) for r in rows)
+    h = ops.gemm(x.to(DEV), wg.to(DEV), act, w2=wu.to(DEV), out_act=True, a_rows=st, tile_group=tile_e,
+                 n_tiles=n_tiles, tile_rows=unit)
+    y = ops.gemm(h, wd.to(DEV), act, a_rows=st, tile_group=tile_e, n_tiles=n_tiles, tile_rows=unit, gather=False).cpu()
+    hc = h.cpu()
+    for t in range(T):
+        for j in range(k):
+            e, r = int(ids[t, j]), int(slot_c[t, j])
+            href = ref_gemm(x[t:t + 1], wg[e], w2=wu[e])[0]
+            assert (hc[r].double() - href).abs().max() < tol(act, 2) * max(1.0, href.abs().max().item())
+            yref = hc[r:r + 1].double() @ wd[e].double().T
+            assert (y[r].double() - yref[0]).abs().max() < tol(act, 2) * max(1.0, yref.abs().max().item())
+
+
+@pytest.mark.parametrize("act", ACTS)
+def test_moe_combine(ops, act):
+    T, k, H, P, S = 6, 3, 100, 40, 2
+    g = torch.Generator().manual_seed(50)
+    y = rnd((P, H), torch.float32, 51)
+    slot = torch.stack([torch.randperm(P, generator=g)[:k] for _ in range(T)]).to(torch.int32)
+    wts = torch.rand((T, k), generator=g)
+    shared = rnd((S, T, H), torch.float32, 52)
+    gate = torch.rand((T,), generator=g)
+    out = ops.moe_combine(y.to(DEV), slot.to(DEV), wts.to(DEV), shared.to(DEV), gate.to(DEV), act).cpu()[0]
+    ref = (wts[:, :, None].double() * y[slot.long()].double()).sum(1) + gate[:, None].double() * shared.double().sum(0)
+    assert (out.double() - ref).abs().max() < 1e-5
+    out2 = ops.moe_combine(y.to(DEV), slot.to(DEV), wts.to(DEV), None, None, act).cpu()[0]
+    assert (out2.double() - (wts[:, :, None].double() * y[slot.long()].double()).sum(1)).abs().max() < 1e-5
+
+
+# ------------------------------------------------------------------------------------------------ router
+@pytest.mark.parametrize("act", ACTS)
+def test_router_reference_vector(ops, act):
+    """The vector of /root/reference/tests/test_gguf_moe.cpp:273-304: 8 experts, top 2, x = e0; expert 3 has
+    logit 10, expert 5 has 8, expert 0 has 1 -> ids [3, 5], weights softmax([10, 8])."""
+    E, H = 8, 4
+    wr = torch.zeros((E, H))
+    wr[3, 0], wr[5, 0], wr[0, 0] = 10.0, 8.0, 1.0
+    x = torch.tensor([[1.0, 0, 0, 0]])
+    ids, w, gate = ops.router_topk(x.to(DEV), wr.to(adt(act)).to(DEV), None, 2, True, act)
+    assert ids.cpu().tolist() == [[3, 5]] and gate is None
+    assert torch.allclose(w.cpu(), torch.tensor([[0.880797, 0.119203]]), atol=1e-5)
+    ids, w, _ = ops.router_topk(x.to(DEV), wr.to(adt(act)).to(DEV), None, 2, False, act)
+    full = torch.softmax(wr[:, 0], 0)
+    assert ids.cpu().tolist() == [[3, 5]]
+    assert torch.allclose(w.cpu()[0], full[[3, 5]], atol=1e-6) and w.sum() < 1
+
+
+@pytest.mark.parametrize("act", ACTS)
+def test_router_ties_and_shared_gate(ops, act):
+    """Equal logits: the highest index wins (>= in /root/reference/src/engine/tq_moe.c:630-638); a zero shared
+    gate vector gives exactly one half."""
+    E, H, T = 6, 40, 3
+    x = rnd((T, H), torch.float32, 60)
+    ids, w, gate = ops.router_topk(x.to(DEV), torch.zeros((E, H), dtype=adt(act)).to(DEV),
+                                   torch.zeros((1, H), dtype=adt(act)).to(DEV), 3, True, act)
+    assert ids.cpu().tolist() == [[5, 4, 3]] * T
+    assert torch.allclose(w.cpu(), torch.full((T, 3), 1 / 3))
+    assert torch.equal(gate.cpu(), torch.full((T,), 0.5))
+
+
+@pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("E,k,H,renorm", [(5, 5, 72, True), (60, 4, 200, False), (130, 8, 64, True)])
+def test_router_random(ops, act, E, k, H, renorm):
+    T = 11
+    x = rnd((T, H), torch.float32, 61)
+    wr = rnd((E, H), adt(act), 62)
+    sg = rnd((1, H), adt(act), 63, 0.1)
+    ids, w, gate = ops.router_topk(x.to(DEV), wr.to(DEV), sg.to(DEV), k, renorm, act)
+    logits = x.double() @ wr.double().T
+    top = torch.topk(logits, k, dim=-1)
+    assert torch.equal(ids.cpu().long(), top.indices)
+    ref = torch.softmax(top.values, -1) if renorm else torch.softmax(logits, -1).gather(1, top.indices)
+    assert (w.cpu().double() - ref).abs().max() < 1e-5
+    assert (gate.cpu().double() - torch.sigmoid(x.double() @ sg.double()[0])).abs().max() < 1e-5
+
+
+# ------------------------------------------------------------------------------------------------ rope + cache + attention
+def paged_setup(lens, page_size, nkv, hd, n_layers, act, seed):
+    """Pages handed out in a scrambled order, so that a kernel that ignores the table fails."""
+    n_pages_seq = [-(-n // page_size) for n in lens]
+    total = sum(n_pages_seq) + 3
+    perm = torch.randperm(total, generator=torch.Generator().manual_seed(seed)).tolist()
+    table = torch.full((len(lens) + 2, max(n_pages_seq) + 1), -1, dtype=torch.int32)
+    slots = [len(lens) + 1 - i for i in range(len(lens))]       # slots in reverse order, slot 0 unused
+    it = iter(perm)
+    for s, n in zip(slots, n_pages_seq):
+        for p in range(n):
+            table[s, p] = next(it)
+    page_stride = n_layers * nkv * page_size * hd
+    kp = torch.zeros(total * page_stride, dtype=adt(act))
+    vp = torch.zeros(total * page_stride, dtype=adt(act))
+    return table, slots, page_stride, kp, vp
+
+
+@pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("pairing,rot", [("half", None), ("interleaved", None), ("half", 16)])
+def test_rope_kv_write(ops, act, pairing, rot):
+    from plain_qwen2moe import rope as plain_rope, rope_frequencies
+    nh, nkv, hd, page, layers, layer = 3, 1, 48, 16, 2, 1
+    rot = hd if rot is None else rot
+    lens = [5, 37]
+    table, slots, page_stride, kp, vp = paged_setup(lens, page, nkv, hd, layers, act, 70)
+    T = sum(lens)
+    qkv = rnd((T, (nh + 2 * nkv) * hd), torch.float32, 71)
+    positions = torch.cat([torch.arange(n) for n in lens]).to(torch.int32)
+    slot_of = torch.cat([torch.full((n,), s) for n, s in zip(lens, slots)]).to(torch.int32)
+    inv_freq = torch.from_numpy(rope_frequencies(rot, 10000.0))
+    kd, vd = kp.to(DEV), vp.to(DEV)
+    off = layer * nkv * page * hd
+    q = ops.rope_kv_write(qkv.to(DEV), positions.to(DEV), slot_of.to(DEV), table.to(DEV), inv_freq.to(DEV),
+                          0 if pairing == "half" else 1, rot, kd, vd, off, page, page_stride, nh, nkv, hd, act).cpu()
+    x = qkv.view(T, nh + 2 * nkv, hd).double()
+    qref = plain_rope(x[:, :nh], positions.tolist(), 10000.0, pairing, rot)
+    kref = plain_rope(x[:, nh:nh + nkv], positions.tolist(), 10000.0, pairing, rot)
+    assert (q.double().view(T, nh, hd) - qref).abs().max() < tol(act, 4)
+    kc, vc = kd.cpu(), vd.cpu()
+    for t in range(T):
+        p, s = int(positions[t]), int(slot_of[t])
+        base = int(table[s, p // page]) * page_stride + off + (p % page) * hd     # kv head 0
+        assert (kc[base:base + hd].double() - kref[t, 0]).abs().max() < tol(act, 4)
+        vbase = int(table[s, p // page]) * page_stride + off + p % page                # values lie [hd][row]
+        assert (vc[vbase:vbase + hd * page:page].double() - x[t, nh + nkv]).abs().max() < tol(act, 4)
+    # nothing outside the written rows was touched
+    assert int((kc != 0).sum()) <= T * nkv * hd and int((vc != 0).sum()) <= T * nkv * hd
+
+
+def test_rope_pairings_are_one_rotation(ops):
+    """interleaved(P x) = P half(x) for the permutation P that interleaves the two halves."""
+    from plain_qwen2moe import rope as plain_rope
+    hd = 16
+    x = rnd((4, 2, hd), torch.float64, 72)
+    perm = torch.tensor([i // 2 + (hd // 2) * (i % 2) for i in range(hd)])    # P x: (x0, x8, x1, x9, ...)
+    pos = [0, 3, 17, 100]
+    a = plain_rope(x[..., perm], pos, 10000.0, "interleaved")
+    b = plain_rope(x, pos, 10000.0, "half")[..., perm]
+    assert (a - b).abs().max() < 1e-12
+
+
+def ref_attention(q, k, v, window, scale):
+    from plain_qwen2moe import attention
+    return attention(q.double(), k.double(), v.double(), window=window, scale=scale)
+
+
+@pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("nh,nkv,hd,window,page", [(4, 4, 16, None, 16), (6, 2, 48, 24, 64), (3, 1, 80, 5, 16),
+                                                     (8, 4, 128, None, 64), (5, 5, 32, 1, 16)])
+def test_attention_over_pages(ops, act, nh, nkv, hd, window, page):
+    """Whole sequences of unequal length in one call, and the last token of each alone (as in decoding),
+    against the plain attention."""
+    lens = [1, 19, 150]
+    layers, layer = 2, 1
+    table, slots, page_stride, kp, vp = paged_setup(lens, page, nkv, hd, layers, act, 80)
+    off = layer * nkv * page * hd
+    scale = 1.0 / math.sqrt(hd)
+    qs, ks, vs = [], [], []
+    for i, n in enumerate(lens):
+        qs.append(rnd((n, nh, hd), adt(act), 81 + i))
+        ks.append(rnd((n, nkv, hd), adt(act), 84 + i))
+        vs.append(rnd((n, nkv, hd), adt(act), 87 + i))
+        for p in range(n):
+            for h in range(nkv):
+                base = int(table[slots[i], p // page]) * page_stride + off + (h * page + p % page) * hd
+                kp[base:base + hd] = ks[i][p, h]
+                vbase = int(table[slots[i], p // page]) * page_stride + off + h * page * hd + p % page
+                vp[vbase:vbase + hd * page:page] = vs[i][p, h]
+    positions = torch.cat([torch.arange(n) for n in lens]).to(torch.int32)
+    slot_of = torch.cat([torch.full((n,), s) for n, s in zip(lens, slots)]).to(torch.int32)
+    q = torch.cat(qs).reshape(-1, nh * hd)
+    kd, vd, td = kp.to(DEV), vp.to(DEV), table.to(DEV)
+    out = ops.attention(q.to(DEV), kd, vd, off, positions.to(DEV), slot_of.to(DEV), td, page, page_stride, nh, nkv,
+                        hd, window, scale, act).cpu()
+    ref = torch.cat([ref_attention(a, b, c, window, scale) for a, b, c in zip(qs, ks, vs)]).reshape(-1, nh * hd)
+    assert (out.double() - ref).abs().max() < tol(act, 2)
+    last = torch.tensor([sum(lens[:i + 1]) - 1 for i in range(len(lens))])
+    out1 = ops.attention(q[last].contiguous().to(DEV), kd, vd, off, positions[last].to(DEV), slot_of[last].to(DEV),
+                         td, page, page_stride, nh, nkv, hd, window, scale, act).cpu()
+    assert (out1.double() - ref[last]).abs().max() < tol(act, 2)
+
+
+@pytest.mark.parametrize("act", ACTS)
+def test_attention_finds_a_far_key(ops, act):
+    """One key among hundreds is made to stand out; its value must come through, whichever page it lies in."""
+    nh = nkv = 2
+    hd, page, n = 32, 16, 300
+    table, slots, page_stride, kp, vp = paged_setup([n], page, nkv, hd, 1, act, 90)
+    q = torch.zeros((1, nh, hd))
+    q[0, :, 0] = 8.0
+    k = rnd((n, nkv, hd), torch.float32, 91, 0.1)
+    v = rnd((n, nkv, hd), torch.float32, 92)
+    far = 37
+    k[far, :, 0] = 40.0
+    for p in range(n):
+        for h in range(nkv):
+            base = int(table[slots[0], p // page]) * page_stride + (h * page + p % page) * hd
+            kp[base:base + hd] = k[p, h].to(adt(act))
+            vbase = int(table[slots[0], p // page]) * page_stride + h * page * hd + p % page
+            vp[vbase:vbase + hd * page:page] = v[p, h].to(adt(act))
+    out = ops.attention(q.reshape(1, -1).to(adt(act)).to(DEV), kp.to(DEV), vp.to(DEV), 0,
+                        torch.tensor([n - 1], dtype=torch.int32).to(DEV),
+                        torch.tensor([slots[0]], dtype=torch.int32).to(DEV), table.to(DEV), page, page_stride, nh,
+                        nkv, hd, None, 1.0 / math.sqrt(hd), act).cpu()
+    assert (out.float().view(nh, hd) - v[far].to(adt(act)).float()).abs().max() < 1e-2
+    # with a window that ends before the far key, it is not seen
+    out_w = ops.attention(q.reshape(1, -1).to(adt(act)).to(DEV), kp.to(DEV), vp.to(DEV), 0,
+                          torch.tensor([n - 1], dtype=torch.int32).to(DEV),
+                          torch.tensor([slots[0]], dtype=torch.int32).to(DEV), table.to(DEV), page, page_stride, nh,
+                          nkv, hd, n - 1 - far, 1.0 / math.sqrt(hd), act).cpu()
+    assert (out_w.float().view(nh, hd) - v[far].float()).abs().max() > 0.5
+    out_w2 = ops.attention(q.reshape(1, -1).to(adt(act)).to(DEV), kp.to(DEV), vp.to(DEV), 0,
+                           torch.tensor([n - 1], dtype=torch.int32).to(DEV),
+                           torch.tensor([slots[0]], dtype=torch.int32).to(DEV), table.to(DEV), page, page_stride, nh,
+                           nkv, hd, n - far, 1.0 / math.sqrt(hd), act).cpu()
+    assert (out_w2.float().view(nh, hd) - v[far].to(adt(act)).float()).abs().max() < 1e-2
+
+
+# ------------------------------------------------------------------------------------------------ sampling
+@pytest.mark.parametrize("V", [10, 1000, 151937])
+def test_argmax_first_maximum(ops, V):
+    logits = rnd((3, V), torch.float32, 100)
+    logits[1, V // 3] = logits[1, V - 1] = 50.0          # equal maxima: the first wins
+    logits[2, :] = 0.0
+    out = ops.argmax(logits.to(DEV), "float32").cpu().tolist()
+    assert out == [int(torch.argmax(logits[0])), V // 3, 0]
+    # the vectors of /root/reference/tests/test_ops.cpp:528-542
+    v = torch.tensor([[1.0, 5.0, 3.0, 2.0], [-3.0, -1.0, -2.0, -5.0]])
+    assert ops.argmax(v.to(DEV), "float32").cpu().tolist() == [1, 1]
+
+
+def test_rep_penalty(ops):
+    from plain_qwen2moe import apply_rep_penalty
+    V = 50
+    logits = rnd((2, V), torch.float32, 110)
+    recent = torch.tensor([[3, 7, 3, -1], [49, 0, 1, 2]], dtype=torch.int32)
+    counts = torch.tensor([3, 4], dtype=torch.int32)
+    d = logits.clone().to(DEV)
+    ops.rep_penalty(d, recent.to(DEV), counts.to(DEV), 1.1, "float32")
+    ref = logits.numpy().copy()
+    apply_rep_penalty(ref[0], [3, 7, 3], 4, 1.1)       # token 3 twice: penalised twice
+    apply_rep_penalty(ref[1], [2, 1, 0, 49], 4, 1.1)
+    assert (d.cpu() - torch.from_numpy(ref)).abs().max() < 1e-6
+
+
+def test_sample_topp_against_plain(ops):
+    """Same logits, same uniform draws: the kernel's choice is the plain sorted walk's choice."""
+    from plain_qwen2moe import sample_topp
+
+    class Fixed:
+        def __init__(self, u):
+            self.u = u
+
+        def next(self):
+            return self.u
+
+    g = torch.Generator().manual_seed(120)
+    for V, T, P in [(4, 0.7, 0.9), (97, 0.7, 0.9), (1000, 1.3, 0.5), (5000, 0.3, 0.95), (300, 0.7, 1.0)]:
+        logits = 3 * torch.randn((16, V), generator=g)
+        u = torch.rand((16,), generator=g)
+        got = ops.sample_topp(logits.to(DEV), T, P, u.to(DEV), "float32").cpu().tolist()
+        want = [sample_topp(logits[r].numpy(), T, P, Fixed(float(u[r]))) for r in range(16)]
+        assert got == want, (V, T, P)
+
+
+def test_sample_topp_distribution(ops):
+    """/root/reference/tests/test_ops.cpp:544-571: T = 0.001 is greedy; uniform logits give each of 4 tokens
+    between 10 % and 50 % of 1000 draws."""
+    from turboquant_cpp_amd.sampling.rng import XorShift64Star
+    logits = torch.tensor([[1.0, 5.0, 3.0, 2.0]])
+    u = torch.tensor([0.73])
+    assert ops.sample_topp(logits.to(DEV), 0.001, 0.9, u.to(DEV), "float32").cpu().tolist() == [1]
+    rng = XorShift64Star(42)
+    draws = torch.tensor([rng.next_float() for _ in range(1000)])
+    out = ops.sample_topp(torch.zeros((1000, 4)).to(DEV), 1.0, 1.0, draws.to(DEV), "float32").cpu()
+    counts = torch.bincount(out.long(), minlength=4)
+    assert all(100 < int(c) < 500 for c in counts), counts
+
+
+# ------------------------------------------------------------------------------------------------ tiled attention
+@pytest.mark.parametrize("nh,nkv,hd,window,page", [(4, 4, 16, None, 64), (6, 2, 48, 24, 64), (3, 1, 80, 70, 128),
+                                                     (16, 16, 128, None, 64), (40, 2, 32, 200, 64), (2, 1, 256, None, 64),
+                                                     (5, 5, 96, 1, 64)])
+def test_attention_tiled(ops, nh, nkv, hd, window, page):
+    """The matrix-core kernels (whole runs of tokens, and one token per sequence split over the cache) against the
+    plain attention: unequal lengths, a sequence that goes on from a cached prefix, groups of more than 16 heads."""
+    act = "bfloat16"
+    lens = [1, 19, 150, 333]
+    layers, layer = 3, 1
+    table, slots, page_stride, kp, vp = paged_setup(lens, page, nkv, hd, layers, act, 130)
+    off = layer * nkv * page * hd
+    scale = 1.0 / math.sqrt(hd)
+    qs, ks, vs = [], [], []
+    for i, n in enumerate(lens):
+        qs.append(rnd((n, nh, hd), adt(act), 131 + i))
+        ks.append(rnd((n, nkv, hd), adt(act), 135 + i))
+        vs.append(rnd((n, nkv, hd), adt(act), 139 + i))
+        for p in range(n):
+            for h in range(nkv):
+                base = int(table[slots[i], p // page]) * page_stride + off + (h * page + p % page) * hd
+                kp[base:base + hd] = ks[i][p, h]
+                vbase = int(table[slots[i], p // page]) * page_stride + off + h * page * hd + p % page
+                vp[vbase:vbase + hd * page:page] = vs[i][p, h]
+    kd, vd, td = kp.to(DEV), vp.to(DEV), table.to(DEV)
+    ref = [ref_attention(a, b, c, window, scale).reshape(-1, nh * hd) for a, b, c in zip(qs, ks, vs)]
+
+    def run(first):          # tokens first[i] .. lens[i]-1 of every sequence in one call
+        new = [n - f for n, f in zip(lens, first)]
+        keep = [i for i, n in enumerate(new) if n > 0]
+        positions = torch.cat([torch.arange(first[i], lens[i]) for i in keep]).to(torch.int32)
+        slot_of = torch.cat([torch.full((new[i],), slots[i]) for i in keep]).to(torch.int32)
+        q = torch.cat([qs[i][first[i]:] for i in keep]).reshape(-1, nh * hd)
+        cu = torch.tensor([0] + list(torch.tensor([new[i] for i in keep]).cumsum(0)), dtype=torch.int32)
+        runs = {"cu_seqlens": cu.to(DEV), "slots": torch.tensor([slots[i] for i in keep], dtype=torch.int32).to(DEV),
+                "start": torch.tensor([first[i] for i in keep], dtype=torch.int32).to(DEV),
+                "max_new": max(new), "max_end": max(lens[i] for i in keep), "decode": all(new[i] == 1 for i in keep)}
+        out = ops.attention(q.to(DEV), kd, vd, off, positions.to(DEV), slot_of.to(DEV), td, page, page_stride, nh, nkv,
+                            hd, window, scale, act, runs=runs).cpu()
+        want = torch.cat([ref[i][first[i]:] for i in keep])
+        return (out.double() - want).abs().max().item()
+
+    assert run([0, 0, 0, 0]) < tol(act, 2)                       # whole prompts
+    assert run([0, 7, 100, 300]) < tol(act, 2)                   # runs that go on from a cached prefix
+    assert run([n - 1 for n in lens]) < tol(act, 2)              # one token each: the split kernel
+    assert run([1, 18, 149, 200]) < tol(act, 2)                  # mixed: not all single tokens

@@ -99,8 +99,10 @@ class CacheGroup:
         self.dirty: set[int] = set()
         self.device = device
         if device is not None:
-            self.k_pages = torch.empty(n_pages * self.page_stride, dtype=dtype, device=device)
-            self.v_pages = torch.empty(n_pages * self.page_stride, dtype=dtype, device=device)
+            # zeroed once: rows beyond a sequence's length are read by tiled kernels (and masked), so they
+            # must always hold finite numbers; pages that come back from a sequence do
+            self.k_pages = torch.zeros(n_pages * self.page_stride, dtype=dtype, device=device)
+            self.v_pages = torch.zeros(n_pages * self.page_stride, dtype=dtype, device=device)
             self.table = torch.full((max_slots, max_pages_per_seq), -1, dtype=torch.int32, device=device)
         else:   # bookkeeping only
             self.k_pages = self.v_pages = self.table = None

@@ -8,7 +8,8 @@
 // (tq_transformer.c:1975-1976).  The softmax is computed chunk by chunk with a running maximum;
 // chunks start at multiples of CHUNK positions, so the order of every sum depends only on the
 // token's own position.  The same kernel serves whole prompts and single decoded tokens: the cache
-// has been written for all tokens of the step before it runs.
+// has been written for all tokens of the step before it runs.  In a page, keys lie [kv head][row][hd]
+// and values transposed, [kv head][hd][row].
 #include "common.h"
 
 #define CHUNK 128
@@ -22,7 +23,8 @@ __global__ __launch_bounds__(CHUNK) void attention_generic_kernel(
   float* qs = sm;                       // hd
   float* ps = qs + hd;                  // CHUNK probabilities
   float* red = ps + CHUNK;              // one per wave
-  int64_t* row_off = (int64_t*)(red + 4);  // CHUNK offsets of the chunk's rows in the pools
+  int64_t* head_off = (int64_t*)(red + 4);  // per row of the chunk: offset of its page's block for this kv head
+  int* row_in_page = (int*)(head_off + CHUNK);
   const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int kvh = h / (nh / nkv);
   const int pos = positions[t];
@@ -43,18 +45,19 @@ __global__ __launch_bounds__(CHUNK) void attention_generic_kernel(
     int64_t off = 0;
     if (valid) {
       const int page = table[j / page_size];
-      off = (int64_t)page * page_stride + ((int64_t)kvh * page_size + j % page_size) * hd;
-      const act_t* kr = k_pool + off;
+      off = (int64_t)page * page_stride + (int64_t)kvh * page_size * hd;
+      const act_t* kr = k_pool + off + (int64_t)(j % page_size) * hd;   // keys: [row][hd]
       float d = 0.f;
       for (int i = 0; i < hd; ++i) d = fmaf(qs[i], to_f32(kr[i]), d);
       sc = d * scale;
     }
-    row_off[tid] = off;
+    head_off[tid] = off;
+    row_in_page[tid] = j % page_size;
     const float m_chunk = block_max(sc, red);
     const float m_new = fmaxf(m_run, m_chunk);
     const float p = valid ? expf(sc - m_new) : 0.f;
     ps[tid] = p;
-    const float l_chunk = block_sum(p, red);   // has the barriers that publish ps and row_off
+    const float l_chunk = block_sum(p, red);   // has the barriers that publish ps and the offsets
     const float alpha = m_run == -INFINITY ? 0.f : expf(m_run - m_new);
     l_run = l_run * alpha + l_chunk;
     m_run = m_new;
@@ -66,7 +69,8 @@ __global__ __launch_bounds__(CHUNK) void attention_generic_kernel(
         float a = acc[c] * alpha;
         for (int jj = 0; jj < n_in_chunk; ++jj) {
           const float pj = ps[jj];
-          if (pj != 0.f) a = fmaf(pj, to_f32(v_pool[row_off[jj] + d]), a);
+          // values: [hd][row]
+          if (pj != 0.f) a = fmaf(pj, to_f32(v_pool[head_off[jj] + (int64_t)d * page_size + row_in_page[jj]]), a);
         }
         acc[c] = a;
       }
@@ -88,7 +92,7 @@ TQ_API int tq_attention_generic(const void* q, const void* k_pool, const void* v
   if (T <= 0) return 0;
   if (hd > 4 * CHUNK || nkv <= 0 || nh % nkv != 0) return TQ_ERR_UNSUPPORTED;
   if (nh > 65535) return TQ_ERR_UNSUPPORTED;
-  const size_t shmem = (size_t)(hd + CHUNK + 4) * sizeof(float) + CHUNK * sizeof(int64_t);
+  const size_t shmem = (size_t)(hd + CHUNK + 4) * sizeof(float) + CHUNK * (sizeof(int64_t) + sizeof(int));
   hipLaunchKernelGGL(attention_generic_kernel, dim3(T, nh), dim3(CHUNK), shmem, st, (const act_t*)q,
                      (const act_t*)k_pool, (const act_t*)v_pool, positions, seq_of_token, block_table, bt_stride,
                      page_size, page_stride, nh, nkv, hd, window, scale, (act_t*)out);

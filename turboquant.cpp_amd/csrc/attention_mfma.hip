@@ -1,0 +1,313 @@
+// Attention over the paged cache on the matrix cores (bfloat16 in, float softmax and sums).
+//
+// Formulas as in attention_generic.hip (/root/reference/src/engine/tq_transformer.c:1646-1654 window,
+// :1675-1679 head mapping, :1908-1976 scores, softmax, value sum).  A wave works on 16 "columns" that
+// share keys and values and runs over tiles of 64 cache positions (a page, or a quarter of one):
+//
+//   S^T = K Q^T     v_mfma_f32_16x16x32_bf16 with A = 16 keys x 32 of hd (16 bytes per lane straight from the
+//                   page, keys lie [row][hd]) and B = the columns' queries, kept in registers.  Lane l then
+//                   holds, for column l % 16, the scores of keys 4 * (l / 16) + v of each 16-key block.
+//   softmax         per column, that is per lane: maxima and sums over a lane's registers and over the four
+//                   lanes l % 16 + 16 c; all in float, running maximum across tiles.
+//   O^T += V^T P^T  A = 16 of hd x 32 keys (values lie transposed in the page, [hd][row], so a lane reads 4
+//                   consecutive keys of one dimension with 8 bytes) and B = the probabilities exactly as the
+//                   lane already holds them: the 32 keys of one product are the lane group's 4 keys of two
+//                   16-key blocks.  No transpose through LDS anywhere.
+//
+// Two entry points share this: whole prompts (columns = 16 consecutive tokens of a sequence, one head; four
+// waves per workgroup) and decoding (columns = the query heads that share one kv head, one token; the cache is
+// split into runs of SPLIT tiles, one wave each, and a second kernel joins the runs in order).  Tiles start at
+// multiples of 64 positions and runs at multiples of SPLIT tiles, so the order of every sum depends only on
+// the token's own position.
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+#define TILE 64
+#define SPLIT 4          // tiles per run when decoding: 256 positions
+
+struct AttnArgs {
+  const bf16_t* q;              // [T][nh][hd]
+  const bf16_t* k_pool;         // layer's offset already added
+  const bf16_t* v_pool;
+  const int* block_table;
+  int bt_stride;
+  const int* cu_seqlens;        // [B + 1]
+  const int* slots;             // [B]
+  const int* start;             // [B] position of each sequence's first new token
+  int page_size;
+  int64_t page_stride;
+  int nh, nkv, hd, window;
+  float scale;
+  bf16_t* out;                  // [T][nh][hd]
+  float* partial;               // decoding: [B][nh][max_runs][hd + 2]
+  int max_runs;
+};
+
+__device__ __forceinline__ bf16x8 ld16(const bf16_t* p) {
+  const uint4 v = *reinterpret_cast<const uint4*>(p);
+  return __builtin_bit_cast(bf16x8, v);
+}
+__device__ __forceinline__ bf16x8 zero16() {
+  const uint4 v = make_uint4(0, 0, 0, 0);
+  return __builtin_bit_cast(bf16x8, v);
+}
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+  return (uint32_t)f32_to_bf16(a).bits | ((uint32_t)f32_to_bf16(b).bits << 16);
+}
+__device__ __forceinline__ float group_max(float v) {     // over the four lanes that share l % 16
+  v = fmaxf(v, __shfl_xor(v, 16, 64));
+  return fmaxf(v, __shfl_xor(v, 32, 64));
+}
+__device__ __forceinline__ float group_sum(float v) {
+  v += __shfl_xor(v, 16, 64);
+  return v + __shfl_xor(v, 32, 64);
+}
+
+// Runs the wave's 16 columns over tiles [tile_beg, tile_end).  DT: number of 16-wide blocks of hd held in
+// registers (hd <= 16 * DT).  p_q: position of this lane's column (-1: no such column), lo_q: first position
+// it may see.  qf: the column's query, 8 values of hd per 32-wide step at 8 * (l / 16).
+template <int DT>
+__device__ __forceinline__ void attend(f32x4 (&o)[DT], float& m_run, float& l_run, const bf16x8 (&qf)[(DT + 1) / 2],
+                                       const bf16_t* kh, const bf16_t* vh, const int* table, int page_size,
+                                       int64_t page_stride, int hd, int tile_beg, int tile_end, int p_q, int lo_q,
+                                       float scale) {
+  constexpr int KS = (DT + 1) / 2;
+  const int lane = threadIdx.x % 64, r = lane % 16, c = lane / 16;
+  const int n_dt = hd / 16, n_ks = (hd + 31) / 32;
+  for (int tile = tile_beg; tile < tile_end; ++tile) {
+    const int pos0 = tile * TILE;
+    const int page = table[pos0 / page_size];
+    const int in_page = pos0 % page_size;
+    const bf16_t* kt = kh + (int64_t)page * page_stride + (int64_t)in_page * hd;      // [row][hd]
+    const bf16_t* vt = vh + (int64_t)page * page_stride + in_page;                     // [hd][row]
+    f32x4 s[4];
+#pragma unroll
+    for (int jt = 0; jt < 4; ++jt) {
+      s[jt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        if (ks < n_ks) {
+          const int d0 = 32 * ks + 8 * c;
+          const bf16x8 kf = d0 < hd ? ld16(kt + (16 * jt + r) * hd + d0) : zero16();
+          s[jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], s[jt], 0, 0, 0);
+        }
+      }
+    }
+    // mask, running maximum, probabilities
+    float m_tile = -INFINITY;
+#pragma unroll
+    for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int key = pos0 + 16 * jt + 4 * c + v;
+        const bool ok = key <= p_q && key >= lo_q;
+        s[jt][v] = ok ? s[jt][v] * scale : -INFINITY;
+        m_tile = fmaxf(m_tile, s[jt][v]);
+      }
+    m_tile = group_max(m_tile);
+    const float m_new = fmaxf(m_run, m_tile);
+    const bool any = m_new != -INFINITY;
+    const float alpha = any && m_run != -INFINITY ? expf(m_run - m_new) : (any ? 0.f : 1.f);
+    float l_tile = 0.f;
+#pragma unroll
+    for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const float p = any ? expf(s[jt][v] - m_new) : 0.f;      // exp(-inf) = 0 for masked keys
+        s[jt][v] = p;
+        l_tile += p;
+      }
+    l_run = l_run * alpha + group_sum(l_tile);
+    m_run = m_new;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) o[dt][v] *= alpha;
+    // values
+#pragma unroll
+    for (int pr = 0; pr < 2; ++pr) {
+      const uint4 pw = make_uint4(pack2(s[2 * pr][0], s[2 * pr][1]), pack2(s[2 * pr][2], s[2 * pr][3]),
+                                  pack2(s[2 * pr + 1][0], s[2 * pr + 1][1]), pack2(s[2 * pr + 1][2], s[2 * pr + 1][3]));
+      const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        if (dt < n_dt) {
+          const bf16_t* vr = vt + (int64_t)(16 * dt + r) * page_size + 32 * pr + 4 * c;
+          const uint2 a = *reinterpret_cast<const uint2*>(vr);
+          const uint2 b = *reinterpret_cast<const uint2*>(vr + 16);
+          const bf16x8 vf = __builtin_bit_cast(bf16x8, make_uint4(a.x, a.y, b.x, b.y));
+          o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[dt], 0, 0, 0);
+        }
+      }
+    }
+  }
+}
+
+template <int DT>
+__device__ __forceinline__ void load_query(bf16x8 (&qf)[(DT + 1) / 2], const bf16_t* qrow, int hd, bool valid) {
+  const int c = (threadIdx.x % 64) / 16;
+#pragma unroll
+  for (int ks = 0; ks < (DT + 1) / 2; ++ks) {
+    const int d0 = 32 * ks + 8 * c;
+    qf[ks] = valid && d0 < hd ? ld16(qrow + d0) : zero16();
+  }
+}
+
+// ------------------------------------------------------------------------------------------ whole prompts
+// grid (ceil(longest run of new tokens / 64), nh, B), block 256: wave w takes tokens 64 x + 16 w .. + 15 of
+// sequence z.  The cache already holds the step's keys and values.
+template <int DT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_kernel(AttnArgs a) {
+  const int seq = blockIdx.z, h = blockIdx.y;
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, r = lane % 16, c = lane / 16;
+  const int t0 = a.cu_seqlens[seq], n = a.cu_seqlens[seq + 1] - t0;
+  const int q0 = blockIdx.x * 64 + wave * 16;
+  if (q0 >= n) return;
+  const int start = a.start[seq];
+  const int qi = q0 + r;
+  const bool valid = qi < n;
+  const int p_q = valid ? start + qi : -1;
+  const int lo_q = a.window > 0 ? max(0, p_q - a.window + 1) : 0;
+  const int kvh = h / (a.nh / a.nkv);
+  const int64_t head_off = (int64_t)kvh * a.page_size * a.hd;
+  const int* table = a.block_table + (size_t)a.slots[seq] * a.bt_stride;
+
+  bf16x8 qf[(DT + 1) / 2];
+  load_query<DT>(qf, a.q + ((size_t)(t0 + (valid ? qi : 0)) * a.nh + h) * a.hd, a.hd, valid);
+  f32x4 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;
+  const int p_first = start + q0, p_last = start + min(q0 + 15, n - 1);
+  const int lo_first = a.window > 0 ? max(0, p_first - a.window + 1) : 0;
+  attend<DT>(o, m_run, l_run, qf, a.k_pool + head_off, a.v_pool + head_off, table, a.page_size, a.page_stride, a.hd,
+             lo_first / TILE, p_last / TILE + 1, p_q, lo_q, a.scale);
+  if (!valid) return;
+  const float inv = 1.0f / l_run;
+  bf16_t* orow = a.out + ((size_t)(t0 + qi) * a.nh + h) * a.hd;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    if (16 * dt < a.hd) {
+      const uint2 w = make_uint2(pack2(o[dt][0] * inv, o[dt][1] * inv), pack2(o[dt][2] * inv, o[dt][3] * inv));
+      *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * c) = w;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------ decoding
+// One new token per sequence at position start[b].  grid (max_runs, nkv * ceil(g / 16), B), block 64: the wave
+// takes run x (tiles SPLIT x .. SPLIT x + SPLIT - 1) for up to 16 of the g = nh / nkv heads of one kv head and
+// writes their unnormalised sums with maximum and denominator.
+template <int DT>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DT > 8 ? 2 : 3))) void attn_decode_kernel(AttnArgs a) {
+  const int b = blockIdx.z, run = blockIdx.x;
+  const int g = a.nh / a.nkv, ngc = (g + 15) / 16;
+  const int kvh = blockIdx.y / ngc, cg = blockIdx.y % ngc;
+  const int lane = threadIdx.x, r = lane % 16, c = lane / 16;
+  const int p = a.start[b];
+  const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
+  const int tile_beg = max(run * SPLIT, lo / TILE), tile_end = min((run + 1) * SPLIT, p / TILE + 1);
+  if (tile_beg >= tile_end) return;
+  const int hg = cg * 16 + r;                 // head within the group
+  const bool valid = hg < g;
+  const int h = kvh * g + (valid ? hg : 0);
+  const int64_t head_off = (int64_t)kvh * a.page_size * a.hd;
+  const int* table = a.block_table + (size_t)a.slots[b] * a.bt_stride;
+  const int t = a.cu_seqlens[b];
+
+  bf16x8 qf[(DT + 1) / 2];
+  load_query<DT>(qf, a.q + ((size_t)t * a.nh + h) * a.hd, a.hd, valid);
+  f32x4 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;
+  attend<DT>(o, m_run, l_run, qf, a.k_pool + head_off, a.v_pool + head_off, table, a.page_size, a.page_stride, a.hd,
+             tile_beg, tile_end, valid ? p : -1, lo, a.scale);
+  if (!valid) return;
+  float* out = a.partial + (((size_t)b * a.nh + h) * a.max_runs + run) * (a.hd + 2);
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    if (16 * dt < a.hd) {
+#pragma unroll
+      for (int v = 0; v < 4; ++v) out[16 * dt + 4 * c + v] = o[dt][v];
+    }
+  }
+  if (c == 0) {
+    out[a.hd] = m_run;
+    out[a.hd + 1] = l_run;
+  }
+}
+
+// Joins the runs of one (sequence, head) in order of position: grid (nh, B), block 64.
+__global__ __launch_bounds__(64) void attn_join_kernel(AttnArgs a) {
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int p = a.start[b];
+  const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
+  const int run_beg = lo / TILE / SPLIT, run_end = p / TILE / SPLIT + 1;
+  const float* part = a.partial + ((size_t)b * a.nh + h) * a.max_runs * (a.hd + 2);
+  float m = -INFINITY;
+  for (int s = run_beg; s < run_end; ++s) m = fmaxf(m, part[(size_t)s * (a.hd + 2) + a.hd]);
+  float l = 0.f;
+  for (int s = run_beg; s < run_end; ++s) {
+    const float* ps = part + (size_t)s * (a.hd + 2);
+    l += expf(ps[a.hd] - m) * ps[a.hd + 1];
+  }
+  const float inv = 1.0f / l;
+  bf16_t* orow = a.out + ((size_t)a.cu_seqlens[b] * a.nh + h) * a.hd;
+  for (int d = threadIdx.x; d < a.hd; d += 64) {
+    float acc = 0.f;
+    for (int s = run_beg; s < run_end; ++s) {
+      const float* ps = part + (size_t)s * (a.hd + 2);
+      acc += expf(ps[a.hd] - m) * ps[d];
+    }
+    orow[d] = f32_to_bf16(acc * inv);
+  }
+}
+
+// ------------------------------------------------------------------------------------------ launch
+template <int DT>
+static void launch_prefill(const AttnArgs& a, int B, int max_new, hipStream_t st) {
+  hipLaunchKernelGGL(attn_prefill_kernel<DT>, dim3((max_new + 63) / 64, a.nh, B), dim3(256), 0, st, a);
+}
+template <int DT>
+static void launch_decode(const AttnArgs& a, int B, hipStream_t st) {
+  const int g = a.nh / a.nkv;
+  hipLaunchKernelGGL(attn_decode_kernel<DT>, dim3(a.max_runs, a.nkv * ((g + 15) / 16), B), dim3(64), 0, st, a);
+  hipLaunchKernelGGL(attn_join_kernel, dim3(a.nh, B), dim3(64), 0, st, a);
+}
+
+// Number of floats of `partial` that decoding B sequences up to position max_end needs.
+TQ_API int64_t tq_attention_decode_scratch(int B, int nh, int hd, int max_end) {
+  const int max_runs = (max_end + TILE * SPLIT - 1) / (TILE * SPLIT);
+  return (int64_t)B * nh * max_runs * (hd + 2);
+}
+
+// decode != 0: every sequence brings exactly one token.  max_new: longest run of new tokens of a sequence;
+// max_end: largest position + 1 that any token of the step has.
+TQ_API int tq_attention_mfma(const void* q, const void* k_pool, const void* v_pool, const int* block_table,
+                             int bt_stride, const int* cu_seqlens, const int* slots, const int* start, int page_size,
+                             int64_t page_stride, int B, int nh, int nkv, int hd, int window, float scale, void* out,
+                             float* partial, int decode, int max_new, int max_end, hipStream_t st) {
+  if (B <= 0) return 0;
+  if (hd % 16 != 0 || hd < 16 || hd > 256 || page_size % TILE != 0 || nkv <= 0 || nh % nkv != 0)
+    return TQ_ERR_UNSUPPORTED;
+  if (nh > 65535 || B > 65535 || page_stride % 8 != 0) return TQ_ERR_UNSUPPORTED;
+  AttnArgs a{(const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, bt_stride, cu_seqlens, slots,
+             start, page_size, page_stride, nh, nkv, hd, window, scale, (bf16_t*)out, partial,
+             (max_end + TILE * SPLIT - 1) / (TILE * SPLIT)};
+  const int dt = hd / 16;
+  if (decode) {
+    if (!partial) return TQ_ERR_BAD_ARG;
+    if (dt <= 4) launch_decode<4>(a, B, st);
+    else if (dt <= 8) launch_decode<8>(a, B, st);
+    else launch_decode<16>(a, B, st);
+  } else {
+    if (dt <= 4) launch_prefill<4>(a, B, max_new, st);
+    else if (dt <= 8) launch_prefill<8>(a, B, max_new, st);
+    else launch_prefill<16>(a, B, max_new, st);
+  }
+  TQ_LAUNCH_CHECK();
+  return 0;
+}

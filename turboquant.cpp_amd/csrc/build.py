@@ -137,6 +137,12 @@ def build(dtype: str, force: bool = False, verbose: bool = True) -> str:
         raise BuildError(f"hipcc failed to link {target}:\n{link.stdout}")
     os.replace(tmp, target)
     shutil.rmtree(obj_dir, ignore_errors=True)
+    for old in os.listdir(out_dir):     # libraries of earlier sources
+        if old.startswith(f"libtq_{dtype}-") and old.endswith(".so") and old != os.path.basename(target):
+            try:
+                os.remove(os.path.join(out_dir, old))
+            except OSError:
+                pass
     say(f"built {os.path.basename(target)} in {time.time() - t0:.0f}s")
     return target
 

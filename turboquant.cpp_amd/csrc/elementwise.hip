@@ -80,8 +80,9 @@ TQ_API int tq_add_rmsnorm(float* x, const float* delta, int S, int64_t delta_str
 //   pairing 1 ("interleaved"): (x[2i], x[2i+1])        (/root/reference/src/engine/tq_ops.c:1418-1448)
 // as (a, b) <- (a cos - b sin, a sin + b cos); dimensions from rot on pass through.  Rotated queries
 // go to q_out; rotated keys and the values go into the page that holds position pos of the token's
-// sequence: page = block_table[seq][pos / page_size], row pos % page_size of kv head h, laid out
-// [page][kv head][row][hd] after the layer's own offset (already added to k_pool / v_pool).
+// sequence: page = block_table[seq][pos / page_size], row pos % page_size of kv head h.  After the
+// layer's own offset (already added to k_pool / v_pool) keys lie [page][kv head][row][hd] and values
+// transposed, [page][kv head][hd][row].
 __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, const int* __restrict__ positions,
                                      const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
                                      int bt_stride, const float* __restrict__ inv_freq, int pairing, int rot,
@@ -93,7 +94,6 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, const int* _
   const int pos = positions[t];
   const float* src = qkv + ((size_t)t * (nh + 2 * nkv) + slot) * hd;
   act_t* dst;
-  bool rotate = true;
   if (slot < nh) {
     dst = q_out + ((size_t)t * nh + slot) * hd;
   } else {
@@ -101,13 +101,12 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, const int* _
     const int kvh = (slot - nh) % nkv;
     const bool is_v = slot >= nh + nkv;
     const int page = block_table[(size_t)seq_of_token[t] * bt_stride + pos / page_size];
-    act_t* pool = is_v ? v_pool : k_pool;
-    dst = pool + (size_t)page * page_stride + ((size_t)kvh * page_size + pos % page_size) * hd;
-    rotate = !is_v;
-  }
-  if (!rotate) {
-    for (int i = threadIdx.x; i < hd; i += blockDim.x) dst[i] = from_f32<act_t>(src[i]);
-    return;
+    if (is_v) {   // values lie transposed, [hd][row], so that a dimension's values over positions are contiguous
+      act_t* col = v_pool + (size_t)page * page_stride + (size_t)kvh * page_size * hd + pos % page_size;
+      for (int i = threadIdx.x; i < hd; i += blockDim.x) col[(size_t)i * page_size] = from_f32<act_t>(src[i]);
+      return;
+    }
+    dst = k_pool + (size_t)page * page_stride + ((size_t)kvh * page_size + pos % page_size) * hd;
   }
   const int half = rot / 2;
   for (int i = threadIdx.x; i < half; i += blockDim.x) {

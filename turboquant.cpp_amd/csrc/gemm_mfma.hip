@@ -1,0 +1,415 @@
+// Matrix products out[m, n] = sum_k a[m, k] * w[n, k] on the matrix cores, bfloat16 in, float sums.
+//
+// Same contract as the plain product (gemm_generic.hip): optional bias, optional gated pair
+// silu(a w^T) * (a w2^T), optional row gather and per-row-tile matrices for experts.  Two kernels:
+//
+//  * gemm_stream_kernel, for few rows (decoding): the work is reading w once.  A wave owns 16 rows of w
+//    and streams them straight from memory into the operand registers of v_mfma_f32_16x16x32_bf16 (lane
+//    l holds 8 consecutive k of row l % 16: four lanes read 64 contiguous bytes of a row); the few rows of
+//    `a` are read the same way and stay in cache.  The waves of a workgroup split k among them and
+//    add their partial sums in wave order through LDS, so that even a narrow matrix gives the chip enough
+//    waves and bytes in flight.  How k is split depends on N and K only, never on the number of rows.
+//  * gemm_tile_kernel, for many rows (prompts): tiles of BM x 128 outputs with 64 of k at a time staged
+//    through LDS (16-byte chunks, XOR-swizzled by row so that the operand reads of
+//    v_mfma_f32_32x32x16_bf16 do not collide), the next tile prefetched into registers meanwhile.
+//
+// Operand layouts (wave of 64 lanes): 16x16x32: A lane l = row l%16, k 8*(l/16)..+7; B lane l = column l%16,
+// same k; D lane l = column l%16, rows 4*(l/16)+v, v<4.  32x32x16: A lane l = row l%32, k 8*(l/32)..+7;
+// B alike; D lane l = column l%32, rows 8*(v/4) + 4*(l/32) + v%4, v<16.
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+struct MfmaGemmArgs {
+  const bf16_t* a;
+  int64_t lda;
+  const int* a_rows;
+  int a_gather;
+  const bf16_t* w;
+  const bf16_t* w2;
+  int64_t group_stride;
+  const int* tile_group;
+  const int* n_tiles;
+  const void* bias;
+  int bias_type;
+  void* out;
+  int64_t ldc;
+  int M, N, K;
+};
+
+__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
+
+__device__ __forceinline__ bf16x8 load8(const bf16_t* p) {
+  const uint4 v = *reinterpret_cast<const uint4*>(p);
+  return __builtin_bit_cast(bf16x8, v);
+}
+__device__ __forceinline__ bf16x8 zero8() {
+  const uint4 v = make_uint4(0, 0, 0, 0);
+  return __builtin_bit_cast(bf16x8, v);
+}
+
+__device__ __forceinline__ float bias_at(const MfmaGemmArgs& g, int n) {
+  if (!g.bias) return 0.f;
+  return g.bias_type == TQ_F32 ? ((const float*)g.bias)[n] : to_f32(((const bf16_t*)g.bias)[n]);
+}
+
+template <bool OUT_ACT>
+__device__ __forceinline__ void store_out(const MfmaGemmArgs& g, int m, int n, float v) {
+  if (OUT_ACT)
+    ((bf16_t*)g.out)[(size_t)m * g.ldc + n] = f32_to_bf16(v);
+  else
+    ((float*)g.out)[(size_t)m * g.ldc + n] = v;
+}
+
+// ------------------------------------------------------------------------------------------ few rows
+// grid (ceil(N / 16), row tiles of 16 * MT rows); block 64 * (waves that split k).
+template <int MT, bool DUAL, bool OUT_ACT>
+__global__ __launch_bounds__(1024) void gemm_stream_kernel(MfmaGemmArgs g) {
+  extern __shared__ float red[];   // [waves][MT * (DUAL ? 2 : 1)][4][64]
+  const int tile_m = blockIdx.y;
+  if (g.n_tiles && tile_m >= g.n_tiles[0]) return;
+  const int group = g.tile_group ? g.tile_group[tile_m] : 0;
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, nw = blockDim.x / 64;
+  const int r = lane % 16, c = lane / 16;
+  const int n0 = blockIdx.x * 16, m0 = tile_m * 16 * MT;
+  const int n = n0 + r;
+  const bool n_ok = n < g.N;
+  const bf16_t* wp = g.w + (size_t)group * g.group_stride + (size_t)(n_ok ? n : 0) * g.K + c * 8;
+  const bf16_t* vp = DUAL ? g.w2 + (size_t)group * g.group_stride + (size_t)(n_ok ? n : 0) * g.K + c * 8 : nullptr;
+  const bf16_t* ap[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = m0 + mt * 16 + r;
+    int src = -1;
+    if (m < g.M) {
+      src = g.a_rows ? g.a_rows[m] : m;
+      if (src >= 0 && !g.a_gather) src = m;
+    }
+    ap[mt] = src >= 0 ? g.a + (size_t)src * g.lda + c * 8 : nullptr;
+  }
+  // this wave's share of k, in steps of 32
+  const int steps = (g.K + 31) / 32;
+  const int per = (steps + nw - 1) / nw;
+  const int k_beg = wave * per * 32, k_end = min(g.K, (wave + 1) * per * 32);
+
+  f32x4 acc[MT], acc2[DUAL ? MT : 1];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (DUAL) acc2[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  // Main part: U steps of 32 at a time with every load issued before the first product, so that a wave
+  // keeps U (2U with the gated pair) kilobytes of w in flight.  Rows that do not exist read row 0 instead;
+  // what they produce is never stored.
+  constexpr int U = (DUAL ? 4 : 8) / (MT == 4 ? 2 : 1);
+  int k = k_beg;
+  {
+    const bf16_t* wq = n_ok ? wp : g.w + (size_t)group * g.group_stride + c * 8;
+    const bf16_t* vq = DUAL ? (n_ok ? vp : g.w2 + (size_t)group * g.group_stride + c * 8) : nullptr;
+    const bf16_t* aq[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) aq[mt] = ap[mt] ? ap[mt] : g.a + c * 8;
+    const int k_main = k_beg + (min(k_end, g.K / 32 * 32) - k_beg) / (32 * U) * (32 * U);
+    for (; k < k_main; k += 32 * U) {
+      bf16x8 wf[U], vf[DUAL ? U : 1], af[MT][U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        wf[u] = load8(wq + k + 32 * u);
+        if (DUAL) vf[u] = load8(vq + k + 32 * u);
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int u = 0; u < U; ++u) af[mt][u] = load8(aq[mt] + k + 32 * u);
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mt][u], wf[u], acc[mt], 0, 0, 0);
+          if (DUAL) acc2[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mt][u], vf[u], acc2[mt], 0, 0, 0);
+        }
+    }
+  }
+  // the rest, one step at a time with bounds checked
+  for (; k < k_end; k += 32) {
+    const bool k_ok = k + c * 8 < g.K;     // K is a multiple of 8: a chunk of 8 is inside or outside as a whole
+    const bf16x8 wf = n_ok && k_ok ? load8(wp + k) : zero8();
+    bf16x8 vf;
+    if (DUAL) vf = n_ok && k_ok ? load8(vp + k) : zero8();
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const bf16x8 af = ap[mt] && k_ok ? load8(ap[mt] + k) : zero8();
+      acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, wf, acc[mt], 0, 0, 0);
+      if (DUAL) acc2[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, vf, acc2[mt], 0, 0, 0);
+    }
+  }
+  constexpr int SETS = MT * (DUAL ? 2 : 1);
+  if (nw > 1) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        red[((wave * SETS + mt) * 4 + v) * 64 + lane] = acc[mt][v];
+        if (DUAL) red[((wave * SETS + MT + mt) * 4 + v) * 64 + lane] = acc2[mt][v];
+      }
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        float s = 0.f, s2 = 0.f;
+        for (int w = 0; w < nw; ++w) {     // partial sums in wave order
+          s += red[((w * SETS + mt) * 4 + v) * 64 + lane];
+          if (DUAL) s2 += red[((w * SETS + MT + mt) * 4 + v) * 64 + lane];
+        }
+        acc[mt][v] = s;
+        if (DUAL) acc2[mt][v] = s2;
+      }
+  }
+  if (!n_ok) return;
+  const float b = bias_at(g, n);
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int m = m0 + mt * 16 + 4 * c + v;
+      if (m >= g.M) continue;
+      if (g.a_rows && g.a_rows[m] < 0) continue;
+      float o = acc[mt][v] + b;
+      if (DUAL) o = silu_f(o) * acc2[mt][v];
+      store_out<OUT_ACT>(g, m, n, o);
+    }
+}
+
+// ------------------------------------------------------------------------------------------ many rows
+// grid (row tiles of BM, ceil(N / 128)); block 256.  BM = 64: waves side by side along n, each 64 x 32;
+// BM = 128: waves 2 x 2, each 64 x 64.
+#define TBN 128
+#define TBK 64
+
+template <int BM>
+__device__ __forceinline__ int swz(int row, int chunk) { return row * TBK + ((chunk ^ (row & 7)) << 3); }
+
+template <int BM, bool DUAL, bool OUT_ACT>
+__global__ __launch_bounds__(256) void gemm_tile_kernel(MfmaGemmArgs g) {
+  constexpr int NI = BM == 128 ? 2 : 1;          // 32-wide column tiles per wave
+  constexpr int MI = 2;                          // 32-high row tiles per wave
+  constexpr int A_CH = BM * 8 / 256;             // 16-byte chunks of the a tile per thread
+  constexpr int W_CH = TBN * 8 / 256;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  bf16_t* As = (bf16_t*)smem;
+  bf16_t* Ws = As + BM * TBK;
+  bf16_t* Vs = Ws + TBN * TBK;
+  const int tile_m = blockIdx.x, tile_n = blockIdx.y;
+  if (g.n_tiles && tile_m >= g.n_tiles[0]) return;
+  const int group = g.tile_group ? g.tile_group[tile_m] : 0;
+  const bf16_t* w = g.w + (size_t)group * g.group_stride;
+  const bf16_t* w2 = DUAL ? g.w2 + (size_t)group * g.group_stride : nullptr;
+  const int m0 = tile_m * BM, n0 = tile_n * TBN;
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const int wm = BM == 128 ? wave / 2 : 0, wn = BM == 128 ? wave % 2 : wave;
+
+  // what this thread fetches of each tile: chunk `ch` of row `row`
+  const bf16_t* a_src[A_CH];
+  int a_dst[A_CH], w_dst[W_CH];
+  const bf16_t *w_src[W_CH], *v_src[W_CH];
+#pragma unroll
+  for (int i = 0; i < A_CH; ++i) {
+    const int idx = tid + i * 256, row = idx / 8, ch = idx % 8;
+    const int m = m0 + row;
+    int src = -1;
+    if (m < g.M) {
+      src = g.a_rows ? g.a_rows[m] : m;
+      if (src >= 0 && !g.a_gather) src = m;
+    }
+    a_src[i] = src >= 0 ? g.a + (size_t)src * g.lda + ch * 8 : nullptr;
+    a_dst[i] = swz<BM>(row, ch);
+  }
+#pragma unroll
+  for (int i = 0; i < W_CH; ++i) {
+    const int idx = tid + i * 256, row = idx / 8, ch = idx % 8;
+    const int n = n0 + row;
+    w_src[i] = n < g.N ? w + (size_t)n * g.K + ch * 8 : nullptr;
+    v_src[i] = DUAL && n < g.N ? w2 + (size_t)n * g.K + ch * 8 : nullptr;
+    w_dst[i] = swz<BM>(row, ch);
+  }
+  const int ch_of_thread = tid % 8;     // (tid + i * 256) % 8
+
+  f32x16 acc[MI][NI], acc2[DUAL ? MI : 1][DUAL ? NI : 1];
+#pragma unroll
+  for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        acc[mi][ni][v] = 0.f;
+        if (DUAL) acc2[mi][ni][v] = 0.f;
+      }
+
+  uint4 pa[A_CH], pw[W_CH], pv[DUAL ? W_CH : 1];
+  const uint4 z = make_uint4(0, 0, 0, 0);
+  auto fetch = [&](int k0) {
+    const bool k_ok = k0 + ch_of_thread * 8 < g.K;
+#pragma unroll
+    for (int i = 0; i < A_CH; ++i) pa[i] = a_src[i] && k_ok ? *reinterpret_cast<const uint4*>(a_src[i] + k0) : z;
+#pragma unroll
+    for (int i = 0; i < W_CH; ++i) {
+      pw[i] = w_src[i] && k_ok ? *reinterpret_cast<const uint4*>(w_src[i] + k0) : z;
+      if (DUAL) pv[i] = v_src[i] && k_ok ? *reinterpret_cast<const uint4*>(v_src[i] + k0) : z;
+    }
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int i = 0; i < A_CH; ++i) *reinterpret_cast<uint4*>(As + a_dst[i]) = pa[i];
+#pragma unroll
+    for (int i = 0; i < W_CH; ++i) {
+      *reinterpret_cast<uint4*>(Ws + w_dst[i]) = pw[i];
+      if (DUAL) *reinterpret_cast<uint4*>(Vs + w_dst[i]) = pv[i];
+    }
+  };
+
+  fetch(0);
+  stage();
+  __syncthreads();
+  const int lr = lane % 32, lc = lane / 32;
+  for (int k0 = 0; k0 < g.K; k0 += TBK) {
+    const bool more = k0 + TBK < g.K;
+    if (more) fetch(k0 + TBK);
+#pragma unroll
+    for (int j = 0; j < TBK / 16; ++j) {
+      bf16x8 af[MI], wf[NI], vf[DUAL ? NI : 1];
+#pragma unroll
+      for (int mi = 0; mi < MI; ++mi) {
+        const int row = wm * 64 + mi * 32 + lr;
+        af[mi] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(As + swz<BM>(row, 2 * j + lc)));
+      }
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni) {
+        const int row = wn * (NI * 32) + ni * 32 + lr;
+        wf[ni] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(Ws + swz<BM>(row, 2 * j + lc)));
+        if (DUAL) vf[ni] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(Vs + swz<BM>(row, 2 * j + lc)));
+      }
+#pragma unroll
+      for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni) {
+          acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[mi], wf[ni], acc[mi][ni], 0, 0, 0);
+          if (DUAL) acc2[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[mi], vf[ni], acc2[mi][ni], 0, 0, 0);
+        }
+    }
+    __syncthreads();
+    if (more) {
+      stage();
+      __syncthreads();
+    }
+  }
+
+#pragma unroll
+  for (int ni = 0; ni < NI; ++ni) {
+    const int n = n0 + wn * (NI * 32) + ni * 32 + lr;
+    if (n >= g.N) continue;
+    const float b = bias_at(g, n);
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + wm * 64 + mi * 32 + 8 * (v / 4) + 4 * lc + (v % 4);
+        if (m >= g.M) continue;
+        if (g.a_rows && g.a_rows[m] < 0) continue;
+        float o = acc[mi][ni][v] + b;
+        if (DUAL) o = silu_f(o) * acc2[mi][ni][v];
+        store_out<OUT_ACT>(g, m, n, o);
+      }
+  }
+}
+
+// ------------------------------------------------------------------------------------------ launch
+// Waves that split k in the streaming kernel: enough for about 2048 waves on the chip, a power of two,
+// each wave keeping at least 128 of k.  A function of N and K only.
+static int split_k_waves(int N, int K) {
+  const int n_tiles = (N + 15) / 16;
+  int s = 1;
+  while (s < 16 && n_tiles * s < 2048 && K / (s * 2) >= 128) s *= 2;
+  return s;
+}
+
+template <int MT>
+static int launch_stream(const MfmaGemmArgs& g, bool dual, bool out_act, int row_tiles, hipStream_t st) {
+  const int nw = split_k_waves(g.N, g.K);
+  const dim3 grid((g.N + 15) / 16, row_tiles);
+  const size_t shmem = nw > 1 ? (size_t)nw * MT * (dual ? 2 : 1) * 4 * 64 * sizeof(float) : 0;
+  if (shmem > 64 * 1024) return TQ_ERR_UNSUPPORTED;
+  if (dual && out_act)
+    hipLaunchKernelGGL((gemm_stream_kernel<MT, true, true>), grid, dim3(64 * nw), shmem, st, g);
+  else if (dual)
+    hipLaunchKernelGGL((gemm_stream_kernel<MT, true, false>), grid, dim3(64 * nw), shmem, st, g);
+  else if (out_act)
+    hipLaunchKernelGGL((gemm_stream_kernel<MT, false, true>), grid, dim3(64 * nw), shmem, st, g);
+  else
+    hipLaunchKernelGGL((gemm_stream_kernel<MT, false, false>), grid, dim3(64 * nw), shmem, st, g);
+  return 0;
+}
+
+template <int BM>
+static int launch_tile(const MfmaGemmArgs& g, bool dual, bool out_act, hipStream_t st) {
+  const dim3 grid((g.M + BM - 1) / BM, (g.N + TBN - 1) / TBN);
+  const size_t shmem = (size_t)(BM + TBN * (dual ? 2 : 1)) * TBK * sizeof(bf16_t);
+#define TQ_TILE(D, O)                                                                                          \
+  do {                                                                                                         \
+    if (shmem > 48 * 1024)                                                                                     \
+      hipFuncSetAttribute((const void*)gemm_tile_kernel<BM, D, O>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                          (int)shmem);                                                                         \
+    hipLaunchKernelGGL((gemm_tile_kernel<BM, D, O>), grid, dim3(256), shmem, st, g);                           \
+  } while (0)
+  if (dual && out_act)
+    TQ_TILE(true, true);
+  else if (dual)
+    TQ_TILE(true, false);
+  else if (out_act)
+    TQ_TILE(false, true);
+  else
+    TQ_TILE(false, false);
+#undef TQ_TILE
+  return 0;
+}
+
+// a: bfloat16 [.., K] with row stride lda (a multiple of 8, as K must be); w, w2: bfloat16.
+// tile_rows: with tile_group set, the padding unit of the row order (16 or 64); else a hint that is ignored.
+TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gather, const void* w, const void* w2,
+                        int64_t group_stride, const int* tile_group, const int* n_tiles, const void* bias,
+                        int bias_type, void* out, int64_t ldc, int out_is_act, int M, int N, int K, int tile_rows,
+                        hipStream_t st) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || K % 8 != 0 || lda % 8 != 0) return TQ_ERR_BAD_ARG;
+  if (((uintptr_t)a | (uintptr_t)w | (uintptr_t)w2) % 16 != 0 || (group_stride % 8) != 0) return TQ_ERR_BAD_ARG;
+  MfmaGemmArgs g{(const bf16_t*)a, lda, a_rows, a_gather, (const bf16_t*)w, (const bf16_t*)w2, group_stride,
+                 tile_group, n_tiles, bias, bias_type, out, ldc, M, N, K};
+  const bool dual = w2 != nullptr, out_act = out_is_act != 0;
+  int rc = 0;
+  if (tile_group) {
+    if (tile_rows == 16) {
+      if (M % 16) return TQ_ERR_BAD_ARG;
+      rc = launch_stream<1>(g, dual, out_act, M / 16, st);
+    } else if (tile_rows == 64) {
+      if ((N + TBN - 1) / TBN > 65535) return TQ_ERR_UNSUPPORTED;
+      rc = launch_tile<64>(g, dual, out_act, st);
+    } else {
+      return TQ_ERR_BAD_ARG;
+    }
+  } else if (M <= 16) {
+    rc = launch_stream<1>(g, dual, out_act, 1, st);
+  } else if (M <= 32) {
+    rc = launch_stream<2>(g, dual, out_act, 1, st);
+  } else if (M <= 64) {
+    rc = launch_stream<4>(g, dual, out_act, 1, st);
+  } else {
+    if ((N + TBN - 1) / TBN > 65535) return TQ_ERR_UNSUPPORTED;
+    rc = M <= 64 * 16 && !dual ? launch_tile<64>(g, dual, out_act, st) : launch_tile<128>(g, dual, out_act, st);
+  }
+  if (rc) return rc;
+  TQ_LAUNCH_CHECK();
+  return 0;
+}

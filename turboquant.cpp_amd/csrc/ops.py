@@ -45,6 +45,8 @@ _SIGNATURES = {
 _OPTIONAL = {
     "tq_gemm_mfma": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int,
                      _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "tq_attention_mfma": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int,
+                          _c_int, _c_int, _c_int, _c_f32, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
 }
 
 
@@ -284,8 +286,13 @@ def gemm(a: torch.Tensor, w: torch.Tensor, act, bias: torch.Tensor | None = None
 def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, layer_offset: int,
               positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor, page_size: int,
               page_stride: int, num_heads: int, num_kv_heads: int, head_dim: int, window: int | None,
-              scale: float, act) -> torch.Tensor:
-    """Each token attends to its sequence's cached positions up to its own; returns [T, nh*hd]."""
+              scale: float, act, runs: dict | None = None) -> torch.Tensor:
+    """Each token attends to its sequence's cached positions up to its own; returns [T, nh*hd].
+
+    ``seq_of_token`` gives each token's row of ``block_table`` (its slot).  ``runs`` describes the same tokens
+    as runs of consecutive positions, one per sequence, for the kernels that work on tiles of tokens:
+    ``cu_seqlens`` [B+1], ``slots`` [B], ``start`` [B] (device, int32) and the host numbers ``max_new``,
+    ``max_end`` and ``decode`` (every sequence brings one token).  Without it the token-by-token kernel runs."""
     k = "attention"
     adt = ACT_DTYPES[dtype_name(act)]
     T = positions.numel()
@@ -301,7 +308,26 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, lay
     _need(layer_offset + num_kv_heads * page_size * head_dim <= page_stride, k, "layer does not fit in a page")
     out = torch.empty_like(q)
     esz = k_pages.element_size()
-    _run(k, library(act).tq_attention_generic(_ptr(q), k_pages.data_ptr() + layer_offset * esz,
+    lib = library(act)
+    if (runs is not None and dtype_name(act) == "bfloat16" and hasattr(lib, "tq_attention_mfma")
+            and head_dim % 16 == 0 and head_dim <= 256 and page_size % 64 == 0 and page_stride % 8 == 0):
+        B = runs["slots"].numel()
+        _check(runs["cu_seqlens"], k, "cu_seqlens", torch.int32, (B + 1,))
+        _check(runs["slots"], k, "slots", torch.int32, (B,))
+        _check(runs["start"], k, "start", torch.int32, (B,))
+        _need(runs["max_end"] <= block_table.shape[1] * page_size, k, "positions reach beyond the page table")
+        partial = None
+        if runs["decode"]:
+            _need(T == B, k, "decoding brings one token per sequence")
+            n_runs = -(-runs["max_end"] // 256)
+            partial = torch.empty((B * num_heads * n_runs * (head_dim + 2),), dtype=torch.float32, device=q.device)
+        _run("attention_mfma", lib.tq_attention_mfma(
+            _ptr(q), k_pages.data_ptr() + layer_offset * esz, v_pages.data_ptr() + layer_offset * esz,
+            _ptr(block_table), block_table.shape[1], _ptr(runs["cu_seqlens"]), _ptr(runs["slots"]), _ptr(runs["start"]),
+            page_size, page_stride, B, num_heads, num_kv_heads, head_dim, int(window or 0), float(scale), _ptr(out),
+            _ptr(partial), int(bool(runs["decode"])), int(runs["max_new"]), int(runs["max_end"]), _stream()))
+        return out
+    _run(k, lib.tq_attention_generic(_ptr(q), k_pages.data_ptr() + layer_offset * esz,
                                               v_pages.data_ptr() + layer_offset * esz, _ptr(positions),
                                               _ptr(seq_of_token), _ptr(block_table), block_table.shape[1], page_size,
                                               page_stride, T, num_heads, num_kv_heads, head_dim, int(window or 0),

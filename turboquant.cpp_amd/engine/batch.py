@@ -44,6 +44,11 @@ class StepBatch:
     def max_end(self) -> int:
         return max(s + n for s, n in zip(self.start, self.n_new))
 
+    def runs(self) -> dict:
+        """The step as runs of consecutive positions, one per sequence, for kernels that tile over tokens."""
+        return {"cu_seqlens": self.cu_seqlens, "slots": self.slots_dev, "start": self.start_dev,
+                "max_new": self.max_new, "max_end": self.max_end, "decode": self.is_decode}
+
 
 def pack_step(slots, starts, token_lists, wants, device) -> StepBatch:
     """Packs per-sequence token lists into the arrays of a step and sends them to the device in one copy.

@@ -71,5 +71,5 @@ class GroupedQueryAttention(Part):
                               self.num_heads, self.num_kv_heads, self.head_dim, ctx.act)
         o = ops.attention(q, kv.k_pages, kv.v_pages, kv.layer_offset, b.positions, b.slot_of_token, kv.table,
                           kv.page_size, kv.page_stride, self.num_heads, self.num_kv_heads, self.head_dim,
-                          self.window, self.scale, ctx.act)
+                          self.window, self.scale, ctx.act, runs=b.runs())
         return ops.gemm(o, self.out_weight, ctx.act).unsqueeze(0)
