@@ -126,19 +126,31 @@ def route(x: torch.Tensor, router: torch.Tensor, top_k: int, renormalize: bool):
     return ids, w
 
 
+def route_margin(x: torch.Tensor, router: torch.Tensor, top_k: int) -> float:
+    """How far the last selected logit lies above the best one left out, in units of the logits' spread:
+    a small margin means that a rounding error upstream can change which experts run."""
+    logits = matvec_rows(router, x)
+    if top_k >= logits.shape[0]:
+        return math.inf
+    top = torch.sort(logits, descending=True).values
+    return float((top[top_k - 1] - top[top_k]) / (logits.std() + 1e-30))
+
+
 def swiglu_mlp(x: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torch.Tensor) -> torch.Tensor:
     """down (silu(gate x) * (up x)) (/root/reference/src/engine/tq_transformer.c:2770-2806; experts:
     /root/reference/src/engine/tq_moe.c:864-999 with an exact exponential)."""
     return matvec_rows(down, silu(matvec_rows(gate, x)) * matvec_rows(up, x))
 
 
-def moe(x: torch.Tensor, w: dict, top_k: int, renormalize: bool) -> torch.Tensor:
+def moe(x: torch.Tensor, w: dict, top_k: int, renormalize: bool, margins: list | None = None) -> torch.Tensor:
     """x [T, H].  out = sum over the selected experts, in the order selected, of weight * expert(x)
     (/root/reference/src/engine/tq_moe.c:720,864-999); then + sigmoid(x . shared_scale) * shared(x)
     (tq_moe.c:1005-1058)."""
     out = torch.zeros_like(x)
     for t in range(x.shape[0]):
         ids, wts = route(x[t], w["router"], top_k, renormalize)
+        if margins is not None:
+            margins.append(route_margin(x[t], w["router"], top_k))
         acc = torch.zeros_like(x[t])
         for e, wt in zip(ids, wts):
             acc = acc + wt * swiglu_mlp(x[t], w["experts"][e]["gate"], w["experts"][e]["up"], w["experts"][e]["down"])
@@ -171,6 +183,7 @@ class PlainQwen2Moe:
         self.nkv = c.get("num_key_value_heads", self.nh)
         self.hd = c.get("head_dim") or self.H // self.nh
         self.eps, self.theta = c["rms_norm_eps"], c["rope_theta"]
+        self.margins: dict[int, list] = {}      # per sparse layer, the routing margin of every token of the last call
 
     def layer_is_sparse(self, l: int) -> bool:
         """No rule in the reference (it looks for a router tensor, /root/reference/src/engine/tq_model.c:3440-3444);
@@ -212,7 +225,8 @@ class PlainQwen2Moe:
         if c["shared_expert_intermediate_size"] > 0:
             w["shared"] = {n: t[f"{p}shared_expert.{n}_proj.weight"] for n in ("gate", "up", "down")}
             w["shared_scale"] = t[p + "shared_expert_gate.weight"]
-        return moe(xb, w, c["num_experts_per_tok"], c.get("norm_topk_prob", False))
+        self.margins[l] = []
+        return moe(xb, w, c["num_experts_per_tok"], c.get("norm_topk_prob", False), self.margins[l])
 
     def logits(self, tokens) -> torch.Tensor:
         """Logits [T, vocab] at every position of one sequence (step order of
@@ -227,6 +241,12 @@ class PlainQwen2Moe:
         x = rmsnorm(x, t["model.norm.weight"], self.eps)                                      # :2922
         head = t["lm_head.weight"] if "lm_head.weight" in t else t["model.embed_tokens.weight"]   # tq_model.c:1499-1516
         return matvec_rows(head, x)                                                           # :2931-2942
+
+    def min_margins(self) -> torch.Tensor:
+        """For every token of the last ``logits`` call, its smallest routing margin over the sparse layers."""
+        if not self.margins:
+            return torch.empty(0)
+        return torch.tensor([self.margins[l] for l in sorted(self.margins)]).min(dim=0).values
 
 
 # ----------------------------------------------------------------------------- sampling and generation

@@ -1,0 +1,243 @@
+"""Configuration from config.json, the architecture registry, weights by tensor name and their errors.  No GPU."""
+import copy
+import json
+import os
+
+import pytest
+import torch
+
+from tiny_configs import TINY, TINY_A, TINY_B
+from turboquant_cpp_amd.config import ConfigError, config_from_dict, config_from_dir, known_architectures
+from turboquant_cpp_amd.engine.model import model_from_config, write_random_model_dir
+from turboquant_cpp_amd.weights import (SafetensorsError, SafetensorsFolder, TensorDict, WeightError, check,
+                                        load_bindings, stored_dtype, write_safetensors)
+
+
+# ------------------------------------------------------------------------------------------------ configuration
+def test_config_reads_every_key_of_both_tiny_models():
+    _, a = config_from_dict(TINY_A)
+    _, b = config_from_dict(TINY_B)
+    assert (a.hidden_size, a.num_attention_heads, a.num_key_value_heads, a.head_dim) == (64, 4, 4, 16)
+    assert (b.hidden_size, b.num_attention_heads, b.num_key_value_heads, b.head_dim) == (144, 6, 2, 24)
+    assert a.norm_topk_prob is False and b.norm_topk_prob is True
+    assert [a.layer_is_sparse(l) for l in range(2)] == [True, True]
+    assert [b.layer_is_sparse(l) for l in range(3)] == [False, True, False]      # mlp_only [0], sparse step 2
+    assert [a.layer_window(l) for l in range(2)] == [None, None]
+    assert [b.layer_window(l) for l in range(3)] == [None, 24, 24]
+    assert b.stop_token_ids == [7, 11] and a.stop_token_ids == []
+    assert (a.rms_norm_eps, b.rms_norm_eps, a.rope_theta, b.rope_theta) == (1e-6, 1e-5, 1e4, 1e6)
+
+
+def test_head_dim_defaults_to_hidden_over_heads_and_kv_heads_to_heads():
+    d = copy.deepcopy(TINY_A)
+    del d["num_key_value_heads"]
+    _, c = config_from_dict(d)
+    assert c.head_dim == 16 and c.num_key_value_heads == 4
+
+
+def test_changing_mlp_only_layers_changes_which_layers_are_sparse():
+    d = copy.deepcopy(TINY_B)
+    d["mlp_only_layers"] = []
+    _, c = config_from_dict(d)
+    assert [c.layer_is_sparse(l) for l in range(3)] == [False, True, False]       # the step rule alone
+    d["decoder_sparse_step"] = 1
+    _, c = config_from_dict(d)
+    assert [c.layer_is_sparse(l) for l in range(3)] == [True, True, True]
+
+
+@pytest.mark.parametrize("key", ["vocab_size", "hidden_size", "num_hidden_layers", "num_attention_heads",
+                                 "intermediate_size", "moe_intermediate_size", "num_experts", "num_experts_per_tok",
+                                 "rope_theta", "rms_norm_eps", "max_position_embeddings",
+                                 "shared_expert_intermediate_size"])
+def test_a_size_or_constant_that_is_missing_is_an_error_not_a_default(key):
+    d = copy.deepcopy(TINY_A)
+    del d[key]
+    with pytest.raises(ConfigError, match=key):
+        config_from_dict(d)
+
+
+@pytest.mark.parametrize("change,word", [
+    ({"num_key_value_heads": 3}, "multiple"),
+    ({"num_experts_per_tok": 9}, "exceeds"),
+    ({"mlp_only_layers": [5]}, "mlp_only_layers"),
+    ({"use_sliding_window": True, "sliding_window": 0}, "sliding_window"),
+    ({"hidden_size": "64"}, "integer"),
+    ({"norm_topk_prob": 1}, "true or false"),
+    ({"head_dim": 15}, "even"),
+    ({"architectures": ["LlamaForCausalLM"]}, "unknown architecture"),
+    ({"architectures": []}, "architectures"),
+])
+def test_inconsistent_configurations_are_refused(change, word):
+    d = copy.deepcopy(TINY_A)
+    d.update(change)
+    with pytest.raises(ConfigError, match=word):
+        config_from_dict(d)
+
+
+def test_unknown_architecture_lists_the_known_ones():
+    d = copy.deepcopy(TINY_A)
+    d["architectures"] = ["Nope"]
+    with pytest.raises(ConfigError) as e:
+        config_from_dict(d)
+    assert "Qwen2MoeForCausalLM" in str(e.value) and known_architectures() == ["Qwen2MoeForCausalLM"]
+
+
+def test_config_from_dir_errors(tmp_path):
+    with pytest.raises(ConfigError, match="no config.json"):
+        config_from_dir(str(tmp_path))
+    (tmp_path / "config.json").write_text("{not json")
+    with pytest.raises(ConfigError, match="not valid JSON"):
+        config_from_dir(str(tmp_path))
+
+
+def test_plan_holds_the_layers_parts_by_kind():
+    arch, c = config_from_dict(TINY_B)
+    plan = arch.plan(c)
+    assert [l.parts["ffn"].kind for l in plan.layers] == ["dense_swiglu", "moe_swiglu", "dense_swiglu"]
+    assert [l.parts["mixer"].args["window"] for l in plan.layers] == [None, 24, 24]
+    assert [e.layer for e in plan.schedule] == [0, 1, 2] and plan.stop_tokens == (7, 11)
+    assert plan.layers[1].parts["ffn"].args["renormalize"] is True
+    assert plan.layers[0].parts["ffn"].args["inner_size"] == 160
+
+
+# ------------------------------------------------------------------------------------------------ safetensors
+def test_safetensors_round_trip_against_the_safetensors_library(tmp_path):
+    from safetensors import safe_open
+    tensors = {"a": torch.randn(3, 5), "b.c": torch.randn(7).to(torch.bfloat16), "i": torch.arange(6, dtype=torch.int32).view(2, 3),
+               "empty": torch.zeros(0, 4)}
+    path = str(tmp_path / "model.safetensors")
+    write_safetensors(path, tensors, metadata={"format": "pt"})
+    with safe_open(path, framework="pt") as f:                   # the library reads what the writer wrote
+        assert set(f.keys()) == set(tensors)
+        for n, t in tensors.items():
+            assert torch.equal(f.get_tensor(n), t)
+    with SafetensorsFolder(str(tmp_path)) as folder:             # and the reader reads it by name
+        for n, t in tensors.items():
+            got = folder.read(n)
+            assert got.dtype == t.dtype and torch.equal(got, t)
+
+
+def test_safetensors_reader_reads_shards_and_refuses_broken_files(tmp_path):
+    write_safetensors(str(tmp_path / "model-00001-of-00002.safetensors"), {"x": torch.ones(2)})
+    write_safetensors(str(tmp_path / "model-00002-of-00002.safetensors"), {"y": torch.zeros(3)})
+    with SafetensorsFolder(str(tmp_path)) as f:
+        assert sorted(f.names()) == ["x", "y"] and f.read("y").shape == (3,)
+    bad = tmp_path / "bad"
+    bad.mkdir()
+    with pytest.raises(SafetensorsError, match="no model.safetensors"):
+        SafetensorsFolder(str(bad))
+    (bad / "model.safetensors").write_bytes(b"\x00" * 4)
+    with pytest.raises(SafetensorsError, match="too small"):
+        SafetensorsFolder(str(bad))
+    (bad / "model.safetensors").write_bytes((10 ** 6).to_bytes(8, "little") + b"{}")
+    with pytest.raises(SafetensorsError, match="beyond the file"):
+        SafetensorsFolder(str(bad))
+    (bad / "model.safetensors").write_bytes((2).to_bytes(8, "little") + b"{x")
+    with pytest.raises(SafetensorsError, match="not valid JSON"):
+        SafetensorsFolder(str(bad))
+    hdr = json.dumps({"t": {"dtype": "F8_E4M3", "shape": [1], "data_offsets": [0, 1]}}).encode()
+    (bad / "model.safetensors").write_bytes(len(hdr).to_bytes(8, "little") + hdr + b"\x00")
+    with pytest.raises(SafetensorsError, match="unsupported dtype"):
+        SafetensorsFolder(str(bad))
+
+
+# ------------------------------------------------------------------------------------------------ weights by name
+def test_expected_tensor_names_and_shapes():
+    table = model_from_config(TINY_B, "float32").tensor_table()
+    assert table["model.embed_tokens.weight"] == ((384, 144), "table")
+    assert table["model.layers.1.self_attn.q_proj.bias"] == ((144,), "bias")
+    assert table["model.layers.1.self_attn.k_proj.weight"] == ((48, 144), "matrix")
+    assert table["model.layers.1.mlp.gate.weight"] == ((12, 144), "matrix")
+    assert table["model.layers.1.mlp.experts.11.down_proj.weight"] == ((144, 48), "matrix")
+    assert table["model.layers.1.mlp.shared_expert_gate.weight"] == ((1, 144), "matrix")
+    assert table["model.layers.0.mlp.up_proj.weight"] == ((160, 144), "matrix")
+    assert table["model.layers.2.post_attention_layernorm.weight"] == ((144,), "scale")
+    assert "model.layers.0.mlp.gate.weight" not in table and "lm_head.weight" in table
+
+
+def test_tied_embeddings_read_no_lm_head():
+    d = copy.deepcopy(TINY_A)
+    d["tie_word_embeddings"] = True
+    assert "lm_head.weight" not in model_from_config(d, "float32").tensor_table()
+
+
+def test_one_error_lists_missing_unexpected_and_wrong_shapes():
+    model = model_from_config(TINY_A, "float32")
+    table = model.tensor_table()
+    tensors = {n: torch.zeros(s) for n, (s, _r) in table.items()}
+    del tensors["model.layers.0.mlp.gate.weight"]
+    del tensors["model.norm.weight"]
+    tensors["model.layers.0.extra.weight"] = torch.zeros(1)
+    tensors["model.layers.1.self_attn.o_proj.weight"] = torch.zeros(64, 63)
+    with pytest.raises(WeightError) as e:
+        load_bindings(model.bindings, TensorDict(tensors), "float32", "cpu")
+    err = e.value
+    assert sorted(err.missing) == ["model.layers.0.mlp.gate.weight", "model.norm.weight"]
+    assert err.unexpected == ["model.layers.0.extra.weight"]
+    assert err.wrong_shape == [("model.layers.1.self_attn.o_proj.weight", (64, 63), (64, 64))]
+    msg = str(err)
+    for word in ("missing tensors (2)", "unexpected tensors (1)", "wrong shapes (1)", "is (64, 63), model wants (64, 64)"):
+        assert word in msg
+
+
+def test_stored_types():
+    bf, f32, f16 = torch.bfloat16, torch.float32, torch.float16
+    assert stored_dtype([bf], "bfloat16") == bf and stored_dtype([f16], "bfloat16") == bf
+    assert stored_dtype([f32], "bfloat16") == f32                 # stored in 32 bits: stays so
+    assert stored_dtype([bf, f32], "bfloat16") == f32
+    assert stored_dtype([bf], "float32") == f32 and stored_dtype([f32], "float32") == f32
+    assert stored_dtype([torch.int64], "bfloat16") == torch.int32
+
+
+def test_parameters_are_stacked_and_joined_from_their_tensors(model_dirs):
+    d = model_dirs("B")
+    model = model_from_config(TINY_B, "float32")
+    with SafetensorsFolder(d) as f:
+        model.load(f, "cpu")
+        attn = model.blocks[1].mixer
+        q, k, v = (f.read(f"model.layers.1.self_attn.{n}_proj.weight") for n in "qkv")
+        assert torch.equal(attn.qkv_weight, torch.cat([q, k, v]))
+        assert torch.equal(attn.qkv_bias, torch.cat([f.read(f"model.layers.1.self_attn.{n}_proj.bias") for n in "qkv"]))
+        moe = model.blocks[1].ffn
+        assert moe.expert_down.shape == (12, 144, 48)
+        assert torch.equal(moe.expert_up[7], f.read("model.layers.1.mlp.experts.7.up_proj.weight"))
+        assert torch.equal(model.lm_head, f.read("lm_head.weight"))
+
+
+def test_bfloat16_model_keeps_32_bit_tensors_in_32_bits(tmp_path):
+    d = write_random_model_dir(str(tmp_path / "m"), TINY_A, seed=3, dtype="bfloat16")
+    # rewrite one norm weight and the router of layer 0 in float32
+    with SafetensorsFolder(d) as f:
+        tensors = {n: f.read(n).clone() for n in f.names()}
+    tensors["model.norm.weight"] = tensors["model.norm.weight"].float()
+    tensors["model.layers.0.mlp.gate.weight"] = tensors["model.layers.0.mlp.gate.weight"].float()
+    write_safetensors(os.path.join(d, "model.safetensors"), tensors)
+    model = model_from_config(TINY_A, "bfloat16")
+    with SafetensorsFolder(d) as f:
+        model.load(f, "cpu")
+    assert model.final_norm.weight.dtype == torch.float32
+    assert model.blocks[0].ffn.router.dtype == torch.float32
+    assert model.blocks[1].ffn.router.dtype == torch.bfloat16 and model.embedding.dtype == torch.bfloat16
+    m32 = model_from_config(TINY_A, "float32")
+    with SafetensorsFolder(d) as f:
+        m32.load(f, "cpu")
+    assert all(getattr(b.owner, b.attr).dtype == torch.float32 for b in m32.bindings)
+
+
+def test_random_weights_mode_writes_a_folder_that_the_seed_fixes(tmp_path):
+    a = write_random_model_dir(str(tmp_path / "a"), TINY_B, seed=1, std=0.02, norm_std=0.02, dtype="float32")
+    b = write_random_model_dir(str(tmp_path / "b"), TINY_B, seed=1, std=0.02, norm_std=0.02, dtype="float32")
+    c = write_random_model_dir(str(tmp_path / "c"), TINY_B, seed=2, std=0.02, norm_std=0.02, dtype="float32")
+    assert sorted(os.listdir(a)) == ["config.json", "model.safetensors"]
+    assert json.load(open(os.path.join(a, "config.json")))["architectures"] == ["Qwen2MoeForCausalLM"]
+    _, cfg = config_from_dir(a)
+    assert cfg.sliding_window == 24 and cfg.stop_token_ids == [7, 11]
+    with SafetensorsFolder(a) as fa, SafetensorsFolder(b) as fb, SafetensorsFolder(c) as fc:
+        assert set(fa.names()) == set(model_from_config(TINY_B, "float32").tensor_table())
+        w = "model.layers.1.mlp.experts.3.gate_proj.weight"
+        assert torch.equal(fa.read(w), fb.read(w)) and not torch.equal(fa.read(w), fc.read(w))
+        assert abs(float(fa.read(w).std()) - 0.02) < 0.004
+        n = fa.read("model.layers.0.input_layernorm.weight")
+        assert abs(float(n.mean()) - 1.0) < 0.01 and 0.01 < float(n.std()) < 0.03
+    with SafetensorsFolder(write_random_model_dir(str(tmp_path / "d"), TINY_A, seed=0, dtype="bfloat16")) as fd:
+        assert fd.read("model.norm.weight").dtype == torch.bfloat16 and bool((fd.read("model.norm.weight") == 1).all())

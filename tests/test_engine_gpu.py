@@ -1,0 +1,497 @@
+"""The engine on the GPU against the plain implementation, in 32-bit and in bfloat16: each request alone and
+whole, with the last 32 tokens one by one, in batches of unequal lengths one after another (through
+``bin/trace_run``, as a user runs it); long decoding; the first tokens; generation through the entry point;
+each part alone; and a toy mixer with state of its own that is registered from here.
+
+How results are compared.  In 32-bit every logit must lie within 1e-4 of the plain implementation's.  In
+bfloat16 every rounding is about 2^-9 of a value, which through the layers comes to about a hundredth of the
+largest logit; but where two experts' router logits nearly tie, that rounding changes which expert runs and the
+logits of that position move by much more.  The plain model reports each position's routing margin; positions
+with a margin under 0.02 (in units of the router logits' spread) are left out, there may not be many of
+them, and the rest must be close: nine in ten within 2 %, all within 10 % of the largest logit.
+"""
+import json
+import math
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from plain_qwen2moe import PlainQwen2Moe, generate as plain_generate
+from tiny_configs import TINY
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DEV = "cuda:0"
+SHARP = 0.1        # weights this wide make attention and routing matter; 0.02 leaves softmaxes nearly flat
+ACTS = ["float32", "bfloat16"]
+MARGIN = 0.02
+
+
+@pytest.fixture(scope="module")
+def sharp_dirs(tmp_path_factory):
+    """Model folders with wide weights, stored in the activation type they are run in."""
+    from turboquant_cpp_amd.engine.model import write_random_model_dir
+    made = {}
+
+    def get(name, act):
+        if (name, act) not in made:
+            cfg, init = TINY[name]
+            d = str(tmp_path_factory.mktemp(f"sharp_{name}_{act}"))
+            write_random_model_dir(d, cfg, init["seed"], SHARP, init["norm_std"], act)
+            made[(name, act)] = (d, PlainQwen2Moe(d))
+        return made[(name, act)]
+    return get
+
+
+@pytest.fixture(scope="module")
+def engines(sharp_dirs):
+    from turboquant_cpp_amd.engine.model import load_model
+    from turboquant_cpp_amd.engine.step import Engine
+    made = {}
+
+    def get(name, act, max_tokens=4096):
+        key = (name, act, max_tokens)
+        if key not in made:
+            d, plain = sharp_dirs(name, act)
+            made[key] = (Engine(load_model(d, act=act, device=DEV), max_tokens=max_tokens), plain)
+        return made[key]
+    return get
+
+
+def prompts_for(name, lens, seed):
+    V = TINY[name][0]["vocab_size"]
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randint(0, V, (n,), generator=g).tolist() for n in lens]
+
+
+def check_logits(got, ref, margins, act, what):
+    """``got`` and ``ref``: [positions, vocab]; ``margins``: routing margin of each position."""
+    got, ref = got.double().cpu(), ref.double()
+    assert got.shape == ref.shape, what
+    err = (got - ref).abs().max(dim=-1).values
+    if act == "float32":
+        assert err.max() < 1e-4, f"{what}: float32 logits differ by {err.max():.2e} at position {int(err.argmax())}"
+        return
+    scale = ref.abs().max()
+    robust = margins >= MARGIN
+    assert robust.float().mean() > 0.6, f"{what}: only {robust.float().mean():.0%} of the positions have a clear routing margin"
+    rel = err[robust] / scale
+    assert rel.max() < 0.10, f"{what}: bfloat16 logits differ by {rel.max():.1%} of the largest logit at a position with a clear margin"
+    assert rel.quantile(0.9) < 0.02, f"{what}: a tenth of the bfloat16 logits differ by more than {rel.quantile(0.9):.1%}"
+
+
+def plain_rows(plain, prompt):
+    ref = plain.logits(prompt)
+    return ref, plain.min_margins() if plain.margins else torch.full((len(prompt),), math.inf)
+
+
+# ------------------------------------------------------------------------------------------------ replay through bin/trace_run
+def build_trace(prompts):
+    """One trace with three ways of cutting the same requests.  Returns (lines, expectations, max_tokens):
+    expectations map a step to [(request, position), ...] in the order of its output rows."""
+    lines, expect, step = [], {}, 0
+    live, peak = {}, 0
+
+    def emit(entries, end):
+        nonlocal step, peak
+        for rid, toks, want, first in entries:
+            live[rid] = live.get(rid, 0) + len(toks)
+        peak = max(peak, sum(-(-n // 64) * 64 for n in live.values()))
+        rows = [(rid.split(":")[1], first + w) for rid, toks, want, first in entries for w in want]
+        if rows:
+            expect[step] = rows
+        lines.append(json.dumps({"step": step, "entries": [{"id": rid, "tokens": toks, "want": want}
+                                                            for rid, toks, want, _ in entries], "end": end}))
+        for rid in end:
+            del live[rid]
+        step += 1
+
+    # 1. each request alone and whole
+    for i, p in enumerate(prompts):
+        emit([(f"w:{i}", p, list(range(len(p))), 0)], [f"w:{i}"])
+    # 2. each request with its last 32 tokens one by one
+    for i, p in enumerate(prompts):
+        cut = max(1, len(p) - 32)
+        emit([(f"d:{i}", p[:cut], list(range(cut)), 0)], [f"d:{i}"] if cut == len(p) else [])
+        for t in range(cut, len(p)):
+            emit([(f"d:{i}", [p[t]], [0], t)], [f"d:{i}"] if t == len(p) - 1 else [])
+    # 3. batches of unequal lengths that start together, go on token by token, and whose shorter members end
+    #    earlier; batch after batch, so that slots and pages are used again
+    order = sorted(range(len(prompts)), key=lambda i: -len(prompts[i]))
+    batches = [order[0::2], order[1::2], order[::-1][:3]]
+    for b, members in enumerate(batches):
+        ids = {i: f"b{b}:{i}" for i in members}
+        cut = {i: max(1, len(prompts[i]) - 5 - 3 * j) for j, i in enumerate(members)}
+        done = [i for i in members if cut[i] == len(prompts[i])]
+        emit([(ids[i], prompts[i][:cut[i]], [cut[i] - 1], 0) for i in members], [ids[i] for i in done])
+        pos = dict(cut)
+        going = [i for i in members if i not in done]
+        while going:
+            done = [i for i in going if pos[i] == len(prompts[i]) - 1]
+            emit([(ids[i], [prompts[i][pos[i]]], [0], pos[i]) for i in going], [ids[i] for i in done])
+            for i in going:
+                pos[i] += 1
+            going = [i for i in going if i not in done]
+    return lines, expect, peak
+
+
+@pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_replay(name, act, sharp_dirs, tmp_path):
+    d, plain = sharp_dirs(name, act)
+    prompts = prompts_for(name, [1, 7, 33, 70, 150], seed=11)
+    lines, expect, peak = build_trace(prompts)
+    out = tmp_path / "out"
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", d, "--dtype", act, "--out", str(out),
+           "--max-tokens", str(peak)]
+    run = subprocess.run(cmd, input="\n".join(lines) + "\n", capture_output=True, text=True, timeout=600)
+    assert run.returncode == 0, run.stderr[-2000:]
+    assert [l for l in run.stdout.splitlines() if l.startswith("done ")] == [f"done {s}" for s in range(len(lines))]
+    refs = [plain_rows(plain, p) for p in prompts]
+    V = TINY[name][0]["vocab_size"]
+    got, want, margins = {"w": [], "d": [], "b": []}, {"w": [], "d": [], "b": []}, {"w": [], "d": [], "b": []}
+    steps_with_output = sorted(int(f[:-4]) for f in os.listdir(out) if f.endswith(".f32"))
+    assert steps_with_output == sorted(expect)
+    for s, rows in expect.items():
+        data = torch.frombuffer(bytearray((out / f"{s}.f32").read_bytes()), dtype=torch.float32).view(-1, V)
+        assert data.shape[0] == len(rows)
+        kind = json.loads(lines[s])["entries"][0]["id"][0]
+        for r, (req, posn) in enumerate(rows):
+            got[kind].append(data[r])
+            want[kind].append(refs[int(req)][0][posn])
+            margins[kind].append(refs[int(req)][1][posn])
+    for kind, what in (("w", "whole"), ("d", "last 32 one by one"), ("b", "unequal batches")):
+        check_logits(torch.stack(got[kind]), torch.stack(want[kind]), torch.stack(margins[kind]).float(), act,
+                     f"{name} {act} {what}")
+
+
+# ------------------------------------------------------------------------------------------------ in process
+@pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_first_tokens_and_long_decoding(name, act, engines):
+    eng, plain = engines(name, act)
+    (seq,) = prompts_for(name, [330], seed=12)
+    ref, margins = plain_rows(plain, seq)
+    slot = eng.open(1)
+    rows = [eng.step(slot, [seq[:3]], [[0, 1, 2]])]                 # the first tokens of a sequence, in one step
+    for t in range(3, len(seq)):
+        rows.append(eng.step(slot, [[seq[t]]]))
+    eng.close(slot)
+    check_logits(torch.cat(rows), ref, margins, act, f"{name} {act} long decoding")
+    for n in (1, 2):                                                # and as the whole of a very short sequence
+        slot = eng.open(1)
+        lg = eng.step(slot, [seq[:n]], [list(range(n))])
+        eng.close(slot)
+        check_logits(lg, ref[:n], margins[:n], act, f"{name} {act} first {n} tokens")
+
+
+@pytest.mark.parametrize("act", ACTS)
+def test_a_request_does_not_feel_its_batch_or_its_place_in_the_cache(act, engines):
+    """Alone in a fresh cache, then among others after the cache has been used and its pages handed round:
+    the same logits, far inside what bfloat16 rounding allows."""
+    eng, plain = engines("B", act, max_tokens=64 * 14)
+    prompts = prompts_for("B", [90, 5, 150, 40], seed=13)
+    slot = eng.open(1)
+    alone = torch.cat([eng.step(slot, [prompts[0][:70]], [list(range(70))])] +
+                      [eng.step(slot, [[t]]) for t in prompts[0][70:]])
+    eng.close(slot)
+    for round_ in range(2):                                         # use the cache up and give it back
+        s = eng.open(3)
+        eng.step(s, [prompts[2], prompts[1], prompts[3]])
+        eng.close(s)
+    s = eng.open(4)
+    order = [1, 0, 2, 3]
+    lg = eng.step(s, [prompts[i][:70] if i == 0 else prompts[i] for i in order],
+                  [list(range(70)) if i == 0 else [] for i in order])
+    rows = [lg]
+    eng.close([s[0], s[3]])
+    for t in prompts[0][70:]:
+        rows.append(eng.step([s[1], s[2]], [[t], [5]], [[0], []]))
+    eng.close([s[1], s[2]])
+    diff = (torch.cat(rows) - alone).abs().max().item()
+    scale = alone.abs().max().item()
+    if act == "float32":
+        assert diff < 2e-5
+    else:
+        ref, margins = plain_rows(plain, prompts[0])
+        check_logits(torch.cat(rows), ref, margins, act, "in a batch")
+        check_logits(alone, ref, margins, act, "alone")
+    assert eng.cache.n_live == 0
+
+
+@pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_generation_through_the_entry_point(name, act, sharp_dirs):
+    from turboquant_cpp_amd import Model
+    d, plain = sharp_dirs(name, act)
+    prompts = prompts_for(name, [4, 1, 30, 9, 17], seed=14)
+    with Model(d, dtype=act, temperature=0.0, rep_penalty=1.0, max_tokens=12, max_batch=3, stop_tokens=()) as m:
+        got = m.generate(prompts, loop_detection=False)
+        single = m.generate(prompts[2], loop_detection=False)
+        assert single == got[2]
+        with_penalty = m.generate(prompts[:2], rep_penalty=1.5, loop_detection=False)
+    assert all(len(g) == 12 for g in got)
+    if act == "float32":
+        assert got == [plain_generate(plain, p, max_tokens=12) for p in prompts]
+        assert with_penalty == [plain_generate(plain, p, max_tokens=12, rep_penalty=1.5) for p in prompts[:2]]
+    else:
+        # every token the engine chose is, by the plain model's logits for the same history, the best or
+        # within rounding of the best
+        for p, g in zip(prompts, got):
+            ref = plain.logits(p + g)
+            for j, tok in enumerate(g):
+                row = ref[len(p) - 1 + j]
+                assert row[tok] >= row.max() - 0.05 * ref.abs().max(), (name, j)
+
+
+def test_sampling_through_the_entry_point_follows_the_plain_loop(sharp_dirs):
+    from turboquant_cpp_amd import Model
+    d, plain = sharp_dirs("A", "float32")
+    prompts = prompts_for("A", [6, 2], seed=15)
+    with Model(d, dtype="float32", temperature=0.8, top_p=0.9, max_tokens=10, seed=9, rep_penalty=1.1,
+               stop_tokens=(), max_batch=1) as m:
+        got = [m.generate(p, loop_detection=False) for p in prompts]
+        again = [m.generate(p, loop_detection=False) for p in prompts]
+        other = m.generate(prompts[0], seed=10, loop_detection=False)
+    want = [plain_generate(plain, p, max_tokens=10, temperature=0.8, top_p=0.9, seed=9, rep_penalty=1.1) for p in prompts]
+    assert got == want and again == got and other != got[0]
+
+
+def test_stop_tokens_of_the_configuration_end_generation(sharp_dirs):
+    from turboquant_cpp_amd import Model
+    d, plain = sharp_dirs("B", "float32")
+    (p,) = prompts_for("B", [8], seed=16)
+    free = plain_generate(plain, p, max_tokens=20)
+    with Model(d, dtype="float32", temperature=0.0, rep_penalty=1.0, max_tokens=20) as m:
+        assert m.options.stop_tokens == (7, 11)                     # eos_token_id of config.json
+        r = m.generate_detailed([p], stop_tokens=(free[6],), loop_detection=False)[0]
+    assert r.tokens == free[:free.index(free[6])] and r.finish_reason == "stop"
+
+
+# ------------------------------------------------------------------------------------------------ each part alone
+def part_context(part_needs, lens, act, starts=None):
+    """A cache and a packed step for one part: sequences of the given lengths, each in its own slot."""
+    from turboquant_cpp_amd.cache import PagedCache
+    from turboquant_cpp_amd.engine.batch import pack_step
+    from turboquant_cpp_amd.engine.context import StepContext
+    dtype = torch.float32 if act == "float32" else torch.bfloat16
+    cache = PagedCache(part_needs, 64 * 16, dtype, torch.device(DEV), page_size=64)
+    slots = [cache.open() for _ in lens]
+    slots = slots[::-1]
+    starts = [cache.reserve(s, n) for s, n in zip(slots, lens)]
+    cache.sync()
+    batch = pack_step(slots, starts, [[0] * n for n in lens], [[] for _ in lens], DEV)
+    return StepContext(batch=batch, cache=cache, act=act, device=torch.device(DEV)), cache, slots
+
+
+def wdt(act):
+    return torch.float32 if act == "float32" else torch.bfloat16
+
+
+def rnd(shape, act, seed, scale=1.0):
+    return (scale * torch.randn(shape, generator=torch.Generator().manual_seed(seed))).to(wdt(act))
+
+
+@pytest.mark.parametrize("act", ACTS)
+def test_attention_part_alone(act):
+    import plain_qwen2moe as P
+    from turboquant_cpp_amd.config import PartSpec
+    from turboquant_cpp_amd.parts import build_part
+    H, nh, nkv, hd, window = 80, 6, 3, 16, 20
+    spec = PartSpec("gqa_attention", dict(hidden_size=H, num_heads=nh, num_kv_heads=nkv, head_dim=hd, qkv_bias=True,
+                                          window=window, position=PartSpec("rope", dict(head_dim=hd, rotary_dim=hd,
+                                                                                        theta=5000.0, pairing="interleaved"))))
+    part = build_part("mixer", spec)
+    specs = part.param_specs()
+    assert specs["qkv_weight"].shape == ((nh + 2 * nkv) * hd, H) and specs["qkv_weight"].splits == (96, 48, 48)
+    w = {n: rnd(s.shape, act, 20 + i, 0.3) for i, (n, s) in enumerate(specs.items())}
+    part.set_params({n: t.to(DEV) for n, t in w.items()})
+    lens = [50, 1, 27]
+    ctx, cache, slots = part_context([(part.cache_need(), None, None)], lens, act)
+    x = rnd((sum(lens), H), act, 30)
+    y = part.forward(x.to(DEV), ctx, 0)
+    assert y.shape == (1, sum(lens), H) and y.dtype == torch.float32
+    o = 0
+    for n in lens:
+        xs = x[o:o + n].double()
+        qkv = xs @ w["qkv_weight"].double().T + w["qkv_bias"].double()
+        q, k, v = qkv[:, :96].view(n, nh, hd), qkv[:, 96:144].view(n, nkv, hd), qkv[:, 144:].view(n, nkv, hd)
+        pos = list(range(n))
+        att = P.attention(P.rope(q, pos, 5000.0, "interleaved"), P.rope(k, pos, 5000.0, "interleaved"), v, window=window)
+        ref = att.reshape(n, nh * hd) @ w["out_weight"].double().T
+        err = (y[0, o:o + n].cpu().double() - ref).abs().max() / ref.abs().max()
+        assert err < (1e-5 if act == "float32" else 3e-2)
+        o += n
+
+
+@pytest.mark.parametrize("act", ACTS)
+def test_feed_forward_parts_alone(act):
+    import plain_qwen2moe as P
+    from turboquant_cpp_amd.config import PartSpec
+    from turboquant_cpp_amd.parts import build_part
+    H, T = 72, 23
+    ctx, _, _ = part_context([(None, None, None)], [T], act)
+    x = rnd((T, H), act, 40)
+    dense = build_part("ffn", PartSpec("dense_swiglu", dict(hidden_size=H, inner_size=104)))
+    w = {n: rnd(s.shape, act, 41 + i, 0.2) for i, (n, s) in enumerate(dense.param_specs().items())}
+    dense.set_params({n: t.to(DEV) for n, t in w.items()})
+    y = dense.forward(x.to(DEV), None, ctx)[0].cpu().double()
+    ref = P.swiglu_mlp(x.double(), w["gate"].double(), w["up"].double(), w["down"].double())
+    assert (y - ref).abs().max() / ref.abs().max() < (1e-5 if act == "float32" else 2e-2)
+    for renorm, shared in ((False, 40), (True, 0)):
+        moe = build_part("ffn", PartSpec("moe_swiglu", dict(hidden_size=H, num_experts=7, top_k=3, expert_size=24,
+                                                            shared_size=shared, renormalize=renorm)))
+        assert moe.wants_f32 and ("shared_scale" in moe.param_specs()) == (shared > 0)
+        w = {n: rnd(s.shape, act, 50 + i, 0.3) for i, (n, s) in enumerate(moe.param_specs().items())}
+        moe.set_params({n: t.to(DEV) for n, t in w.items()})
+        y = moe.forward(x.to(DEV), x.float().to(DEV), ctx)[0].cpu().double()
+        pw = {"router": w["router"].double(),
+              "experts": [{"gate": w["expert_gate"][e].double(), "up": w["expert_up"][e].double(),
+                           "down": w["expert_down"][e].double()} for e in range(7)]}
+        if shared:
+            pw["shared"] = {"gate": w["shared_gate"].double(), "up": w["shared_up"].double(), "down": w["shared_down"].double()}
+            pw["shared_scale"] = w["shared_scale"].double()
+        ref = P.moe(x.double(), pw, 3, renorm)
+        assert (y - ref).abs().max() / ref.abs().max() < (1e-5 if act == "float32" else 2e-2)
+
+
+@pytest.mark.parametrize("act", ACTS)
+def test_norm_and_position_parts_alone(act):
+    import plain_qwen2moe as P
+    from turboquant_cpp_amd.config import PartSpec
+    from turboquant_cpp_amd.parts import build_part
+    norm = build_part("norm", PartSpec("rmsnorm", dict(size=100, eps=1e-3)))
+    w = rnd((100,), act, 60) + 1
+    norm.set_params({"weight": w.to(DEV)})
+    ctx, _, _ = part_context([(None, None, None)], [9], act)
+    x, delta = torch.randn(9, 100), torch.randn(2, 9, 100)
+    xd = x.clone().to(DEV)
+    out, out32 = norm.forward(xd, delta.to(DEV), ctx, want_f32=True)
+    ref = P.rmsnorm(x.double() + delta.double().sum(0), w.double(), 1e-3)
+    assert (out32.cpu().double() - ref).abs().max() < 1e-4 and out.dtype == wdt(act)
+    assert (xd.cpu().double() - (x.double() + delta.double().sum(0))).abs().max() < 1e-5
+    rope = build_part("position", PartSpec("rope", dict(head_dim=48, rotary_dim=32, theta=1e6, pairing="half")))
+    assert rope.pairing_code == 0 and rope.rotary_dim == 32
+    assert torch.equal(rope.table(DEV).cpu(), torch.from_numpy(P.rope_frequencies(32, 1e6)))
+    with pytest.raises(ValueError, match="pairing"):
+        build_part("position", PartSpec("rope", dict(head_dim=8, rotary_dim=8, theta=1.0, pairing="odd")))
+    with pytest.raises(ValueError, match="unknown norm"):
+        build_part("norm", PartSpec("layernorm", {}))
+
+
+# ------------------------------------------------------------------------------------------------ a toy mixer with state
+def test_a_mixer_with_state_of_its_own_is_registered_built_and_stepped():
+    """A recurrent mixer defined here: per sequence a state s of the model's width, s <- decay * s + x W_in for
+    every token in order, output s W_out.  It keeps no keys or values, only its state in the cache's fixed-size
+    area.  Registered, put into a model by a plan, loaded and stepped through the engine without touching the
+    library's files; whole prompts, token by token and unequal batches must agree with a plain loop."""
+    from turboquant_cpp_amd.config import LayerSpec, ModelPlan, PartSpec, ScheduleEntry, Source
+    from turboquant_cpp_amd.engine.model import CausalLM
+    from turboquant_cpp_amd.engine.step import Engine
+    from turboquant_cpp_amd.parts import ParamSpec, Part, StateNeed, register_part, unregister_part
+    from turboquant_cpp_amd.weights import TensorDict
+
+    H, V, INNER, L = 48, 90, 64, 2
+
+    class ToyDecayMixer(Part):
+        def __init__(self, hidden_size, decay):
+            self.hidden_size, self.decay = hidden_size, decay
+            self.w_in = self.w_out = None
+
+        def param_specs(self):
+            return {"w_in": ParamSpec((self.hidden_size, self.hidden_size)), "w_out": ParamSpec((self.hidden_size, self.hidden_size))}
+
+        def cache_need(self):
+            return None
+
+        def state_need(self):
+            return StateNeed((self.hidden_size,), torch.float32)
+
+        def forward(self, normed, ctx, entry):
+            state = ctx.state(entry)                               # [slots, H]; zero for a new sequence
+            u = normed.float() @ self.w_in.float().T
+            out = torch.empty_like(u)
+            b = ctx.batch
+            o = 0
+            for slot, n in zip(b.slots, b.n_new):                  # a scan over each sequence's new tokens
+                s = state[slot]
+                for t in range(o, o + n):
+                    s = self.decay * s + u[t]
+                    out[t] = s
+                state[slot] = s
+                o += n
+            return (out @ self.w_out.float().T).unsqueeze(0)
+
+    register_part("mixer", "toy_decay")(ToyDecayMixer)
+    try:
+        def norm(name):
+            return PartSpec("rmsnorm", dict(size=H, eps=1e-5), {"weight": Source.single(name)})
+        layers = [LayerSpec("prenorm", {
+            "mixer_norm": norm(f"l{l}.n1"), "ffn_norm": norm(f"l{l}.n2"),
+            "mixer": PartSpec("toy_decay", dict(hidden_size=H, decay=0.5 + 0.2 * l),
+                              {"w_in": Source.single(f"l{l}.in"), "w_out": Source.single(f"l{l}.out")}),
+            "ffn": PartSpec("dense_swiglu", dict(hidden_size=H, inner_size=INNER),
+                            {n: Source.single(f"l{l}.{n}") for n in ("gate", "up", "down")})}) for l in range(L)]
+        plan = ModelPlan("ToyRecurrentLM", V, H, layers, [ScheduleEntry(l) for l in range(L)], norm("final"),
+                         Source.single("embed"), None, max_positions=512)
+        model = CausalLM(plan, "float32")
+        g = torch.Generator().manual_seed(70)
+        tensors = {n: (torch.ones(s) if role == "scale" else 0.3 * torch.randn(s, generator=g))
+                   for n, (s, role) in model.tensor_table().items()}
+        model.load(TensorDict(tensors), DEV)
+        eng = Engine(model, max_tokens=64 * 4, max_slots=3)
+        assert eng.cache.groups == [] and sorted(eng.cache.states) == [0, 1]
+
+        def plain(tokens):
+            import plain_qwen2moe as P
+            t = {n: v.double() for n, v in tensors.items()}
+            x = t["embed"][tokens]
+            for l in range(L):
+                u = P.rmsnorm(x, t[f"l{l}.n1"], 1e-5) @ t[f"l{l}.in"].T
+                s, ys = torch.zeros(H, dtype=torch.float64), []
+                for i in range(len(tokens)):
+                    s = (0.5 + 0.2 * l) * s + u[i]
+                    ys.append(s)
+                x = x + torch.stack(ys) @ t[f"l{l}.out"].T
+                x = x + P.swiglu_mlp(P.rmsnorm(x, t[f"l{l}.n2"], 1e-5), t[f"l{l}.gate"], t[f"l{l}.up"], t[f"l{l}.down"])
+            return P.rmsnorm(x, t["final"], 1e-5) @ t["embed"].T
+
+        prompts = [torch.randint(0, V, (n,), generator=g).tolist() for n in (9, 1, 20)]
+        refs = [plain(p) for p in prompts]
+        slots = eng.open(3)
+        lg = eng.step(slots, prompts, [list(range(len(p))) for p in prompts]).cpu().double()
+        assert (lg - torch.cat(refs)).abs().max() < 1e-4
+        eng.close(slots)
+        # token by token in an unequal batch, in slots that have been used: state must start from zero again
+        slots = eng.open(3)
+        cut = [4, 1, 11]
+        eng.step(slots, [p[:c] for p, c in zip(prompts, cut)], [[] for _ in prompts])
+        pos, live = list(cut), [0, 2]
+        eng.close([slots[1]])
+        while live:
+            lg = eng.step([slots[i] for i in live], [[prompts[i][pos[i]]] for i in live]).cpu().double()
+            for j, i in enumerate(live):
+                assert (lg[j] - refs[i][pos[i]]).abs().max() < 1e-4
+                pos[i] += 1
+            for i in [i for i in live if pos[i] == len(prompts[i])]:
+                eng.close([slots[i]])
+                live.remove(i)
+        assert eng.cache.n_live == 0
+    finally:
+        unregister_part("mixer", "toy_decay")
+
+
+def test_the_kernels_refuse_to_run_without_their_library(monkeypatch):
+    """No silent fallback: if the compiled library cannot be found or built, the first kernel call raises."""
+    from turboquant_cpp_amd.csrc import build, ops
+    monkeypatch.setattr(ops, "_LIBS", {})
+    monkeypatch.setattr(build, "find_library", lambda dtype: None)
+
+    def no_build(dtype, **kw):
+        raise build.BuildError("hipcc not found")
+    monkeypatch.setattr(build, "build", no_build)
+    with pytest.raises(build.BuildError):
+        ops.embed(torch.zeros(1, dtype=torch.int32, device=DEV), torch.zeros((2, 4), device=DEV), "float32")
