@@ -495,3 +495,38 @@ def test_the_kernels_refuse_to_run_without_their_library(monkeypatch):
     monkeypatch.setattr(build, "build", no_build)
     with pytest.raises(build.BuildError):
         ops.embed(torch.zeros(1, dtype=torch.int32, device=DEV), torch.zeros((2, 4), device=DEV), "float32")
+
+
+# ------------------------------------------------------------------------------------------------ decode steps as graphs
+@pytest.mark.parametrize("act", ACTS)
+def test_replayed_decode_steps_give_the_bits_of_eager_steps(act, sharp_dirs):
+    """Many replays, with eager prompt steps, closed and reopened slots and synchronisations between them; every
+    replay is checked against the step run eagerly by a second engine on the same model."""
+    from turboquant_cpp_amd.engine.model import load_model
+    from turboquant_cpp_amd.engine.step import Engine
+    d, _ = sharp_dirs("B", act)
+    model = load_model(d, act=act, device=DEV)
+    fast, slow = Engine(model, max_tokens=64 * 12), Engine(model, max_tokens=64 * 12, use_graphs=False)
+    assert fast.graphs is not None and slow.graphs is None
+    prompts = prompts_for("B", [40, 3, 70], seed=17)
+    g = torch.Generator().manual_seed(18)
+    sf, ss = fast.open(3), slow.open(3)
+    assert torch.equal(fast.step(sf, prompts), slow.step(ss, prompts))
+    live = [0, 1, 2]
+    for step in range(40):
+        toks = [[int(torch.randint(0, 384, (1,), generator=g))] for _ in live]
+        a = fast.step([sf[i] for i in live], toks)
+        b = slow.step([ss[i] for i in live], toks)
+        torch.cuda.synchronize()
+        assert torch.equal(a, b), f"replay {step} differs from the eager step"
+        if step == 12:                       # a sequence ends; the others go on as a smaller batch
+            fast.close([sf[1]]), slow.close([ss[1]])
+            live = [0, 2]
+        if step == 20:                       # a new one starts in the freed slot: an eager prompt step in between
+            sf[1], ss[1] = fast.open(1)[0], slow.open(1)[0]
+            p = prompts_for("B", [25], seed=19)
+            assert torch.equal(fast.step([sf[1]], p), slow.step([ss[1]], p))
+            live = [1, 0, 2]
+    assert len(fast.graphs.graphs) >= 2
+    only_second = fast.step([sf[i] for i in live], [[1], [2], [3]], [[], [0], []])
+    assert torch.equal(only_second, slow.step([ss[i] for i in live], [[1], [2], [3]], [[], [0], []])) and only_second.shape[0] == 1

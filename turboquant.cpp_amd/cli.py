@@ -1,0 +1,125 @@
+"""Command line in the manner of the reference's ``quant <model> [options]`` (/root/reference/tools/quant.c:126-163,
+defaults :196-239): the model path first, then ``-p`` prompt, ``-n`` max tokens (256), ``-T`` temperature (0.7),
+``-P`` top-p (0.9), ``-s`` seed (42), ``--ctx`` context length, ``--info``, ``--profile``, ``--version``.  There is no
+tokenizer in this library, so a prompt is a list of token ids (``-p "5,17,3"``; several prompts are separated by
+``;`` and run as one batch), or ``--random-prompt LEN[,LEN...]`` draws them.  ``--random-weights CONFIG.json --save
+DIR`` is the random-weights mode: it writes a model folder for a configuration and a seed and exits.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+
+def parse_prompts(text: str) -> list[list[int]]:
+    prompts = []
+    for part in text.split(";"):
+        ids = [int(t) for t in part.replace(",", " ").split()]
+        if ids:
+            prompts.append(ids)
+    if not prompts:
+        raise ValueError("the prompt holds no token id")
+    return prompts
+
+
+def build_parser() -> argparse.ArgumentParser:
+    ap = argparse.ArgumentParser(prog="turboquant_cpp_amd", description="Qwen2-MoE generation on one MI355X.")
+    ap.add_argument("model", nargs="?", help="folder with config.json and model.safetensors")
+    ap.add_argument("-p", dest="prompt", default=None, help='token ids of the prompt, e.g. "5,17,3"; ";" separates prompts')
+    ap.add_argument("-n", dest="max_tokens", type=int, default=256, help="max tokens to generate (default: 256)")
+    ap.add_argument("-T", dest="temperature", type=float, default=0.7, help="sampling temperature (default: 0.7)")
+    ap.add_argument("-P", dest="top_p", type=float, default=0.9, help="top-p sampling (default: 0.9)")
+    ap.add_argument("-s", dest="seed", type=int, default=42, help="random seed (default: 42)")
+    ap.add_argument("-j", dest="threads", type=int, default=None, help="accepted for compatibility; the GPU does the work")
+    ap.add_argument("--ctx", type=int, default=0, help="override max context length (default: the model's, at most 4096)")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--rep-penalty", type=float, default=1.1, help="repetition penalty over the last 32 tokens (default: 1.1)")
+    ap.add_argument("--stop-id", type=int, action="append", default=None, help="stop token id (default: eos_token_id of config.json)")
+    ap.add_argument("--random-prompt", default=None, metavar="LEN[,LEN...]", help="prompts of random token ids of these lengths")
+    ap.add_argument("--max-batch", type=int, default=8, help="sequences that generate together")
+    ap.add_argument("--info", action="store_true", help="print model info and exit")
+    ap.add_argument("--profile", action="store_true", help="time the prompt step and the decode steps")
+    ap.add_argument("--json", action="store_true", help="print results as JSON")
+    ap.add_argument("--version", action="store_true")
+    ap.add_argument("--random-weights", metavar="CONFIG.json", default=None, help="write a model folder with random weights")
+    ap.add_argument("--save", metavar="DIR", default=None, help="where --random-weights writes")
+    ap.add_argument("--std", type=float, default=0.02)
+    ap.add_argument("--norm-std", type=float, default=0.0)
+    ap.add_argument("--file-dtype", default="bfloat16", choices=["bfloat16", "float32", "float16"])
+    return ap
+
+
+def main(argv=None) -> int:
+    args = build_parser().parse_args(argv)
+    if args.version:
+        from . import __version__
+        print(f"turboquant_cpp_amd v{__version__}")
+        return 0
+    if args.random_weights:
+        if not args.save:
+            print("--random-weights needs --save DIR", file=sys.stderr)
+            return 2
+        from .engine.model import write_random_model_dir
+        with open(args.random_weights) as f:
+            cfg = json.load(f)
+        out = write_random_model_dir(args.save, cfg, args.seed, args.std, args.norm_std, args.file_dtype)
+        print(f"wrote {out}", file=sys.stderr)
+        return 0
+    if not args.model:
+        build_parser().print_usage(sys.stderr)
+        return 2
+    if args.info:
+        from .config import config_from_dir
+        arch, cfg = config_from_dir(args.model)
+        print(f"architecture: {arch.name}")
+        for k, v in vars(cfg).items():
+            print(f"  {k}: {v}")
+        return 0
+
+    import torch
+    from .api import Model
+    t0 = time.time()
+    model = Model(args.model, temperature=args.temperature, top_p=args.top_p, max_tokens=args.max_tokens,
+                  context_length=args.ctx, dtype=args.dtype, seed=args.seed, rep_penalty=args.rep_penalty,
+                  max_batch=args.max_batch, stop_tokens=args.stop_id)
+    print(f"loaded {args.model} in {time.time() - t0:.1f}s ({args.dtype}, context {model.context_length})", file=sys.stderr)
+    if args.random_prompt:
+        g = torch.Generator().manual_seed(args.seed)
+        V = model.engine.vocab_size
+        prompts = [torch.randint(0, V, (int(n),), generator=g).tolist() for n in args.random_prompt.split(",")]
+    else:
+        prompts = parse_prompts(args.prompt if args.prompt is not None else "1")
+    torch.cuda.synchronize()
+    t1 = time.time()
+    results = model.generate_detailed(prompts)
+    torch.cuda.synchronize()
+    elapsed = time.time() - t1
+    n_generated = sum(len(r.tokens) for r in results)
+    if args.json:
+        print(json.dumps([{"tokens": r.tokens, "finish_reason": r.finish_reason} for r in results]))
+    else:
+        for i, r in enumerate(results):
+            print(f"[{i}] {' '.join(str(t) for t in r.tokens)}  ({r.finish_reason})")
+    if n_generated > 0 and elapsed > 0:
+        print(f"{n_generated} tokens in {elapsed:.1f}s ({n_generated / elapsed:.1f} tok/s, {len(prompts)} sequences, "
+              f"weights={args.dtype}, kv={args.dtype})", file=sys.stderr)
+    if args.profile:
+        eng = model.engine
+        slots = eng.open(len(prompts))
+        torch.cuda.synchronize()
+        t = time.time()
+        eng.step(slots, [list(p) for p in prompts])
+        torch.cuda.synchronize()
+        t_prompt = time.time() - t
+        t = time.time()
+        for _ in range(16):
+            eng.step(slots, [[1] for _ in prompts])
+        torch.cuda.synchronize()
+        t_dec = (time.time() - t) / 16
+        eng.close(slots)
+        print(f"profile: prompt step {t_prompt * 1e3:.2f} ms ({sum(len(p) for p in prompts)} tokens), "
+              f"decode step {t_dec * 1e3:.2f} ms ({len(prompts)} sequences)", file=sys.stderr)
+    model.close()
+    return 0

@@ -240,28 +240,39 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DT > 8 ? 2 :
   }
 }
 
-// Joins the runs of one (sequence, head) in order of position: grid (nh, B), block 64.
+// Joins the runs of one (sequence, head) in order of position: grid (nh, B), block 64.  The weights
+// exp(m_s - m) of the runs are worked out once, a lane per run, and kept in LDS; then every lane sums its
+// dimensions over the runs in order.
+#define MAX_RUNS_LDS 1024
 __global__ __launch_bounds__(64) void attn_join_kernel(AttnArgs a) {
-  const int h = blockIdx.x, b = blockIdx.y;
+  __shared__ float wgt[MAX_RUNS_LDS];
+  const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
   const int p = a.start[b];
   const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
   const int run_beg = lo / TILE / SPLIT, run_end = p / TILE / SPLIT + 1;
-  const float* part = a.partial + ((size_t)b * a.nh + h) * a.max_runs * (a.hd + 2);
+  const int stride = a.hd + 2;
+  const float* part = a.partial + ((size_t)b * a.nh + h) * a.max_runs * stride;
   float m = -INFINITY;
-  for (int s = run_beg; s < run_end; ++s) m = fmaxf(m, part[(size_t)s * (a.hd + 2) + a.hd]);
+  for (int s = run_beg + lane; s < run_end; s += 64) m = fmaxf(m, part[(size_t)s * stride + a.hd]);
+  m = wave_max(m);
   float l = 0.f;
-  for (int s = run_beg; s < run_end; ++s) {
-    const float* ps = part + (size_t)s * (a.hd + 2);
-    l += expf(ps[a.hd] - m) * ps[a.hd + 1];
+  for (int s0 = run_beg; s0 < run_end; s0 += 64) {     // denominators in run order, 64 runs at a time
+    const int s = s0 + lane;
+    float w = 0.f, wl = 0.f;
+    if (s < run_end) {
+      w = expf(part[(size_t)s * stride + a.hd] - m);
+      wl = w * part[(size_t)s * stride + a.hd + 1];
+      wgt[s - run_beg] = w;
+    }
+    l += wave_sum(wl);
   }
+  __builtin_amdgcn_wave_barrier();
   const float inv = 1.0f / l;
   bf16_t* orow = a.out + ((size_t)a.cu_seqlens[b] * a.nh + h) * a.hd;
-  for (int d = threadIdx.x; d < a.hd; d += 64) {
+  for (int d = lane; d < a.hd; d += 64) {
     float acc = 0.f;
-    for (int s = run_beg; s < run_end; ++s) {
-      const float* ps = part + (size_t)s * (a.hd + 2);
-      acc += expf(ps[a.hd] - m) * ps[d];
-    }
+#pragma unroll 8
+    for (int s = run_beg; s < run_end; ++s) acc = fmaf(wgt[s - run_beg], part[(size_t)s * stride + d], acc);
     orow[d] = f32_to_bf16(acc * inv);
   }
 }
@@ -294,6 +305,7 @@ TQ_API int tq_attention_mfma(const void* q, const void* k_pool, const void* v_po
   if (hd % 16 != 0 || hd < 16 || hd > 256 || page_size % TILE != 0 || nkv <= 0 || nh % nkv != 0)
     return TQ_ERR_UNSUPPORTED;
   if (nh > 65535 || B > 65535 || page_stride % 8 != 0) return TQ_ERR_UNSUPPORTED;
+  if (decode && (max_end + TILE * SPLIT - 1) / (TILE * SPLIT) > MAX_RUNS_LDS) return TQ_ERR_UNSUPPORTED;
   AttnArgs a{(const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, bt_stride, cu_seqlens, slots,
              start, page_size, page_stride, nh, nkv, hd, window, scale, (bf16_t*)out, partial,
              (max_end + TILE * SPLIT - 1) / (TILE * SPLIT)};

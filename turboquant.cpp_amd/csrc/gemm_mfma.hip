@@ -100,29 +100,27 @@ __global__ __launch_bounds__(1024) void gemm_stream_kernel(MfmaGemmArgs g) {
     acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
     if (DUAL) acc2[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
-  // Main part: U steps of 32 at a time with every load issued before the first product, so that a wave
-  // keeps U (2U with the gated pair) kilobytes of w in flight.  Rows that do not exist read row 0 instead;
-  // what they produce is never stored.
+  // U steps of 32 at a time, every load issued before the first product, so that a wave keeps U (2U with the
+  // gated pair) kilobytes of w in flight.  Rows that do not exist read row 0 instead (what they produce is never
+  // stored); steps beyond the wave's share or beyond K load nothing and multiply zeros.
   constexpr int U = (DUAL ? 4 : 8) / (MT == 4 ? 2 : 1);
-  int k = k_beg;
   {
     const bf16_t* wq = n_ok ? wp : g.w + (size_t)group * g.group_stride + c * 8;
     const bf16_t* vq = DUAL ? (n_ok ? vp : g.w2 + (size_t)group * g.group_stride + c * 8) : nullptr;
     const bf16_t* aq[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) aq[mt] = ap[mt] ? ap[mt] : g.a + c * 8;
-    const int k_main = k_beg + (min(k_end, g.K / 32 * 32) - k_beg) / (32 * U) * (32 * U);
-    for (; k < k_main; k += 32 * U) {
+    for (int k = k_beg; k < k_end; k += 32 * U) {
       bf16x8 wf[U], vf[DUAL ? U : 1], af[MT][U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        wf[u] = load8(wq + k + 32 * u);
-        if (DUAL) vf[u] = load8(vq + k + 32 * u);
+        const int ku = k + 32 * u;
+        const bool ok = ku < k_end && ku + c * 8 < g.K;   // K is a multiple of 8: a chunk of 8 is in or out as a whole
+        wf[u] = ok ? load8(wq + ku) : zero8();
+        if (DUAL) vf[u] = ok ? load8(vq + ku) : zero8();
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) af[mt][u] = ok ? load8(aq[mt] + ku) : zero8();
       }
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int u = 0; u < U; ++u) af[mt][u] = load8(aq[mt] + k + 32 * u);
 #pragma unroll
       for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -132,19 +130,7 @@ __global__ __launch_bounds__(1024) void gemm_stream_kernel(MfmaGemmArgs g) {
         }
     }
   }
-  // the rest, one step at a time with bounds checked
-  for (; k < k_end; k += 32) {
-    const bool k_ok = k + c * 8 < g.K;     // K is a multiple of 8: a chunk of 8 is inside or outside as a whole
-    const bf16x8 wf = n_ok && k_ok ? load8(wp + k) : zero8();
-    bf16x8 vf;
-    if (DUAL) vf = n_ok && k_ok ? load8(vp + k) : zero8();
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const bf16x8 af = ap[mt] && k_ok ? load8(ap[mt] + k) : zero8();
-      acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, wf, acc[mt], 0, 0, 0);
-      if (DUAL) acc2[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, vf, acc2[mt], 0, 0, 0);
-    }
-  }
+  // The waves' partial sums are added in wave order, every thread of the workgroup taking some of the outputs.
   constexpr int SETS = MT * (DUAL ? 2 : 1);
   if (nw > 1) {
 #pragma unroll
@@ -155,19 +141,21 @@ __global__ __launch_bounds__(1024) void gemm_stream_kernel(MfmaGemmArgs g) {
         if (DUAL) red[((wave * SETS + MT + mt) * 4 + v) * 64 + lane] = acc2[mt][v];
       }
     __syncthreads();
-    if (wave != 0) return;
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        float s = 0.f, s2 = 0.f;
-        for (int w = 0; w < nw; ++w) {     // partial sums in wave order
-          s += red[((w * SETS + mt) * 4 + v) * 64 + lane];
-          if (DUAL) s2 += red[((w * SETS + MT + mt) * 4 + v) * 64 + lane];
-        }
-        acc[mt][v] = s;
-        if (DUAL) acc2[mt][v] = s2;
+    for (int i = threadIdx.x; i < MT * 256; i += blockDim.x) {
+      const int ol = i % 64, v = (i / 64) % 4, mt = i / 256;
+      float s = 0.f, s2 = 0.f;
+      for (int w = 0; w < nw; ++w) {
+        s += red[((w * SETS + mt) * 4 + v) * 64 + ol];
+        if (DUAL) s2 += red[((w * SETS + MT + mt) * 4 + v) * 64 + ol];
       }
+      const int on = n0 + ol % 16, om = m0 + mt * 16 + 4 * (ol / 16) + v;
+      if (on >= g.N || om >= g.M) continue;
+      if (g.a_rows && g.a_rows[om] < 0) continue;
+      float o = s + bias_at(g, on);
+      if (DUAL) o = silu_f(o) * s2;
+      store_out<OUT_ACT>(g, om, on, o);
+    }
+    return;
   }
   if (!n_ok) return;
   const float b = bias_at(g, n);
@@ -203,7 +191,21 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(MfmaGemmArgs g) {
   bf16_t* As = (bf16_t*)smem;
   bf16_t* Ws = As + BM * TBK;
   bf16_t* Vs = Ws + TBN * TBK;
-  const int tile_m = blockIdx.x, tile_n = blockIdx.y;
+  // Which tile this workgroup takes.  Workgroups are dealt to the chip's 8 dies in turn (id % 8), and each die
+  // has its own L2: so the tiles are numbered such that one die gets a contiguous run of them, and a run goes
+  // through bands of 8 row tiles, down a band's column of row tiles first.  Workgroups that run at the same
+  // time on a die then share their tiles of `a` and of `w` in that die's L2.
+  int tile_m, tile_n;
+  {
+    const int gx = gridDim.x, gy = gridDim.y, total = gx * gy;
+    const int id = blockIdx.y * gx + blockIdx.x;
+    const int die = id % 8, q = total / 8, rem = total % 8;
+    const int logical = die * q + min(die, rem) + id / 8;
+    const int band = logical / (8 * gy), in_band = logical % (8 * gy);
+    const int bh = min(8, gx - band * 8);
+    tile_m = band * 8 + in_band % bh;
+    tile_n = in_band / bh;
+  }
   if (g.n_tiles && tile_m >= g.n_tiles[0]) return;
   const int group = g.tile_group ? g.tile_group[tile_m] : 0;
   const bf16_t* w = g.w + (size_t)group * g.group_stride;
@@ -327,18 +329,20 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(MfmaGemmArgs g) {
 }
 
 // ------------------------------------------------------------------------------------------ launch
-// Waves that split k in the streaming kernel: enough for about 2048 waves on the chip, a power of two,
-// each wave keeping at least 128 of k.  A function of N and K only.
-static int split_k_waves(int N, int K) {
+// Waves that split k in the streaming kernel: a power of two, enough for about 2048 waves on the chip when one
+// matrix is multiplied and for about 256 per matrix when there is one per expert, each wave keeping at least 256 of
+// k.  A function of N, K and of whether the product is over experts, never of the number of rows.
+static int split_k_waves(int N, int K, bool grouped) {
   const int n_tiles = (N + 15) / 16;
+  const int want = grouped ? 256 : 2048;
   int s = 1;
-  while (s < 16 && n_tiles * s < 2048 && K / (s * 2) >= 128) s *= 2;
+  while (s < 16 && n_tiles * s < want && K / (s * 2) >= 256) s *= 2;
   return s;
 }
 
 template <int MT>
 static int launch_stream(const MfmaGemmArgs& g, bool dual, bool out_act, int row_tiles, hipStream_t st) {
-  const int nw = split_k_waves(g.N, g.K);
+  const int nw = split_k_waves(g.N, g.K, g.tile_group != nullptr);
   const dim3 grid((g.N + 15) / 16, row_tiles);
   const size_t shmem = nw > 1 ? (size_t)nw * MT * (dual ? 2 : 1) * 4 * 64 * sizeof(float) : 0;
   if (shmem > 64 * 1024) return TQ_ERR_UNSUPPORTED;

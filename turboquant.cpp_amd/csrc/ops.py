@@ -35,7 +35,8 @@ _SIGNATURES = {
                         _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "tq_attention_generic": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_i64, _c_int, _c_int,
                              _c_int, _c_int, _c_int, _c_f32, _c_ptr, _c_ptr],
-    "tq_router_topk": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
+    "tq_router_topk": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
+                       _c_ptr],
     "tq_moe_align": [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
     "tq_argmax": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr],
     "tq_rep_penalty": [_c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_ptr, _c_f32, _c_ptr],
@@ -352,8 +353,10 @@ def router_topk(x32: torch.Tensor, router: torch.Tensor, shared_scale: torch.Ten
     ids = torch.empty((T, top_k), dtype=torch.int32, device=x32.device)
     weights = torch.empty((T, top_k), dtype=torch.float32, device=x32.device)
     gate = torch.empty((T,), dtype=torch.float32, device=x32.device) if shared_scale is not None else None
+    logits = torch.empty((T, E + (1 if shared_scale is not None else 0)), dtype=torch.float32, device=x32.device)
     _run(k, library(act).tq_router_topk(_ptr(x32), _ptr(router), _ptr(shared_scale), _WTYPE[router.dtype], E, top_k,
-                                        int(bool(renormalize)), _ptr(ids), _ptr(weights), _ptr(gate), T, H, _stream()))
+                                        int(bool(renormalize)), _ptr(ids), _ptr(weights), _ptr(gate), _ptr(logits),
+                                        T, H, _stream()))
     return ids, weights, gate
 
 

@@ -27,6 +27,7 @@ class StepBatch:
     start_dev: torch.Tensor           # int32 [B]
     want_rows: torch.Tensor           # int32 [R]: packed rows whose logits are wanted
     n_want: int
+    fixed_max_end: int | None = None  # set when launches must not depend on the sequences' true lengths
 
     @property
     def n_seqs(self) -> int:
@@ -42,6 +43,8 @@ class StepBatch:
 
     @property
     def max_end(self) -> int:
+        if self.fixed_max_end is not None:
+            return self.fixed_max_end
         return max(s + n for s, n in zip(self.start, self.n_new))
 
     def runs(self) -> dict:

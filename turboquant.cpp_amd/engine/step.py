@@ -14,6 +14,7 @@ import torch
 from ..cache.paged import CacheError
 from .batch import pack_step
 from .context import StepContext
+from .graph import DecodeGraphs
 from .model import CausalLM
 
 
@@ -25,11 +26,15 @@ class Engine:
     """A model with its cache.  ``max_tokens`` is the most positions that live sequences hold at once,
     each sequence rounded up to whole pages of ``page_size``."""
 
-    def __init__(self, model: CausalLM, max_tokens: int, page_size: int = 64, max_slots: int | None = None):
+    def __init__(self, model: CausalLM, max_tokens: int, page_size: int = 64, max_slots: int | None = None,
+                 use_graphs: bool = True):
         self.model = model
         self.cache = model.new_cache(max_tokens, page_size=page_size, max_slots=max_slots)
         self.device = model.device
         self.vocab_size = model.plan.vocab_size
+        # decode steps are replayed as HIP graphs where a GPU runs them
+        on_gpu = self.device is not None and self.device.type == "cuda"
+        self.graphs = DecodeGraphs(self) if use_graphs and on_gpu and all(p.graph_safe for p in model.parts()) else None
 
     # ------------------------------------------------------------ sequences
     def open(self, n: int = 1) -> list[int]:
@@ -82,9 +87,21 @@ class Engine:
                 s.reserved = 0
             raise
         self.cache.sync()
-        batch = pack_step(slots, starts, token_lists, wants, self.device)
-        ctx = StepContext(batch=batch, cache=self.cache, act=self.model.act, device=self.device)
-        logits = self.model.forward(ctx)
+        logits = None
+        if self.graphs is not None and all(len(t) == 1 for t in token_lists):
+            for i, w in enumerate(wants):
+                if any(x != 0 for x in w):
+                    raise ValueError(f"wanted place {w} is outside the 1 token that sequence {i} brings")
+            all_rows = self.graphs.run(slots, starts, [t[0] for t in token_lists])
+            if all_rows is not None:       # the graph gives every row; hand out a copy of the wanted ones
+                rows = [i for i, w in enumerate(wants) for _ in w]
+                logits = all_rows.clone() if rows == list(range(len(slots))) else \
+                    all_rows[torch.tensor(rows, dtype=torch.int64, device=self.device)] if rows else \
+                    torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
+        if logits is None:
+            batch = pack_step(slots, starts, token_lists, wants, self.device)
+            ctx = StepContext(batch=batch, cache=self.cache, act=self.model.act, device=self.device)
+            logits = self.model.forward(ctx)
         for slot in slots:
             self.cache.commit(slot)
         return logits

@@ -18,6 +18,7 @@ from .base import CacheNeed, ParamSpec, Part, build_part, register_part
 
 @register_part("mixer", "gqa_attention")
 class GroupedQueryAttention(Part):
+    graph_safe = True
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, position,
                  qkv_bias: bool = False, out_bias: bool = False, window: int | None = None,
                  scale: float | None = None):

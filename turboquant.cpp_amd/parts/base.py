@@ -57,6 +57,10 @@ class StateNeed:
 class Part:
     category: str = ""
     kind: str = ""
+    # True if forward() reads what changes from step to step (tokens, positions, slots, lengths) from the
+    # batch's device arrays only, so that a captured launch sequence can be replayed for other sequences.
+    # Decode steps of a model are replayed as graphs only if all its parts say so.
+    graph_safe: bool = False
 
     def param_specs(self) -> dict[str, ParamSpec]:
         return {}

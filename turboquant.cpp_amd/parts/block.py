@@ -12,6 +12,7 @@ from .base import Part, register_part
 
 @register_part("block", "prenorm")
 class PreNormBlock(Part):
+    graph_safe = True
     # the parts a layer of this arrangement is made of, and the registry each comes from
     slots = {"mixer_norm": "norm", "mixer": "mixer", "ffn_norm": "norm", "ffn": "ffn"}
 

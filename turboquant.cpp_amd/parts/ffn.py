@@ -15,6 +15,7 @@ from .base import ParamSpec, Part, register_part
 
 @register_part("ffn", "dense_swiglu")
 class DenseSwiGLU(Part):
+    graph_safe = True
     wants_f32 = False
 
     def __init__(self, hidden_size: int, inner_size: int):
@@ -33,6 +34,7 @@ class DenseSwiGLU(Part):
 
 @register_part("ffn", "moe_swiglu")
 class SparseMoE(Part):
+    graph_safe = True
     wants_f32 = True    # the router reads the normalised activations in float32
 
     def __init__(self, hidden_size: int, num_experts: int, top_k: int, expert_size: int, shared_size: int = 0,

@@ -11,6 +11,7 @@ from .base import ParamSpec, Part, register_part
 
 @register_part("norm", "rmsnorm")
 class RMSNorm(Part):
+    graph_safe = True
     def __init__(self, size: int, eps: float):
         self.size, self.eps = size, eps
         self.weight = None

@@ -23,6 +23,7 @@ PAIRINGS = {"half": 0, "interleaved": 1}
 
 @register_part("position", "rope")
 class RotaryEncoding(Part):
+    graph_safe = True
     def __init__(self, head_dim: int, rotary_dim: int, theta: float, pairing: str = "half"):
         if pairing not in PAIRINGS:
             raise ValueError(f"unknown pairing {pairing!r}; known: {sorted(PAIRINGS)}")
