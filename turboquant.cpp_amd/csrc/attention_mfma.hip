@@ -65,83 +65,109 @@ __device__ __forceinline__ float group_sum(float v) {
   return v + __shfl_xor(v, 32, 64);
 }
 
-// Runs the wave's 16 columns over tiles [tile_beg, tile_end).  DT: number of 16-wide blocks of hd held in
-// registers (hd <= 16 * DT).  p_q: position of this lane's column (-1: no such column), lo_q: first position
-// it may see.  qf: the column's query, 8 values of hd per 32-wide step at 8 * (l / 16).
-template <int DT>
-__device__ __forceinline__ void attend(f32x4 (&o)[DT], float& m_run, float& l_run, const bf16x8 (&qf)[(DT + 1) / 2],
-                                       const bf16_t* kh, const bf16_t* vh, const int* table, int page_size,
-                                       int64_t page_stride, int hd, int tile_beg, int tile_end, int p_q, int lo_q,
-                                       float scale) {
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// One tile of 64 positions for QG groups of 16 columns that share the tile's keys and values.  kt: the tile's
+// keys, row i at kt + i * k_stride; vt: the tile's values transposed, dimension d at vt + d * v_stride (memory or
+// LDS).  DT: number of 16-wide blocks of hd held in registers (hd <= 16 * DT).  p_q: position of this lane's
+// column in each group (-1: no such column), lo_q: first position it may see.  qf: the columns' queries, 8
+// values of hd per 32-wide step at 8 * (l / 16).  Every operand read from kt and vt serves all QG groups.
+template <int DT, int QG>
+__device__ __forceinline__ void tile_step(f32x4 (&o)[QG][DT], float (&m_run)[QG], float (&l_run)[QG],
+                                          const bf16x8 (&qf)[QG][(DT + 1) / 2], const bf16_t* kt, int k_stride,
+                                          const bf16_t* vt, int v_stride, int hd, int pos0, const int (&p_q)[QG],
+                                          const int (&lo_q)[QG], float scale) {
   constexpr int KS = (DT + 1) / 2;
   const int lane = threadIdx.x % 64, r = lane % 16, c = lane / 16;
   const int n_dt = hd / 16, n_ks = (hd + 31) / 32;
-  for (int tile = tile_beg; tile < tile_end; ++tile) {
-    const int pos0 = tile * TILE;
-    const int page = table[pos0 / page_size];
-    const int in_page = pos0 % page_size;
-    const bf16_t* kt = kh + (int64_t)page * page_stride + (int64_t)in_page * hd;      // [row][hd]
-    const bf16_t* vt = vh + (int64_t)page * page_stride + in_page;                     // [hd][row]
-    f32x4 s[4];
+  f32x4 s[QG][4];
 #pragma unroll
-    for (int jt = 0; jt < 4; ++jt) {
-      s[jt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int jt = 0; jt < 4; ++jt) {
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        if (ks < n_ks) {
-          const int d0 = 32 * ks + 8 * c;
-          const bf16x8 kf = d0 < hd ? ld16(kt + (16 * jt + r) * hd + d0) : zero16();
-          s[jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], s[jt], 0, 0, 0);
-        }
+    for (int g = 0; g < QG; ++g) s[g][jt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      if (ks < n_ks) {
+        const int d0 = 32 * ks + 8 * c;
+        const bf16x8 kf = d0 < hd ? ld16(kt + (16 * jt + r) * k_stride + d0) : zero16();
+#pragma unroll
+        for (int g = 0; g < QG; ++g) s[g][jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[g][ks], s[g][jt], 0, 0, 0);
       }
     }
-    // mask, running maximum, probabilities
+  }
+  // mask, running maximum, probabilities
+#pragma unroll
+  for (int g = 0; g < QG; ++g) {
     float m_tile = -INFINITY;
 #pragma unroll
     for (int jt = 0; jt < 4; ++jt)
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
         const int key = pos0 + 16 * jt + 4 * c + v;
-        const bool ok = key <= p_q && key >= lo_q;
-        s[jt][v] = ok ? s[jt][v] * scale : -INFINITY;
-        m_tile = fmaxf(m_tile, s[jt][v]);
+        const bool ok = key <= p_q[g] && key >= lo_q[g];
+        s[g][jt][v] = ok ? s[g][jt][v] * scale : -INFINITY;
+        m_tile = fmaxf(m_tile, s[g][jt][v]);
       }
     m_tile = group_max(m_tile);
-    const float m_new = fmaxf(m_run, m_tile);
+    const float m_new = fmaxf(m_run[g], m_tile);
     const bool any = m_new != -INFINITY;
-    const float alpha = any && m_run != -INFINITY ? expf(m_run - m_new) : (any ? 0.f : 1.f);
+    const float alpha = any && m_run[g] != -INFINITY ? expf(m_run[g] - m_new) : (any ? 0.f : 1.f);
     float l_tile = 0.f;
 #pragma unroll
     for (int jt = 0; jt < 4; ++jt)
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
-        const float p = any ? expf(s[jt][v] - m_new) : 0.f;      // exp(-inf) = 0 for masked keys
-        s[jt][v] = p;
+        const float p = any ? expf(s[g][jt][v] - m_new) : 0.f;      // exp(-inf) = 0 for masked keys
+        s[g][jt][v] = p;
         l_tile += p;
       }
-    l_run = l_run * alpha + group_sum(l_tile);
-    m_run = m_new;
+    l_run[g] = l_run[g] * alpha + group_sum(l_tile);
+    m_run[g] = m_new;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-      for (int v = 0; v < 4; ++v) o[dt][v] *= alpha;
-    // values
+      for (int v = 0; v < 4; ++v) o[g][dt][v] *= alpha;
+  }
+  // values
 #pragma unroll
-    for (int pr = 0; pr < 2; ++pr) {
-      const uint4 pw = make_uint4(pack2(s[2 * pr][0], s[2 * pr][1]), pack2(s[2 * pr][2], s[2 * pr][3]),
-                                  pack2(s[2 * pr + 1][0], s[2 * pr + 1][1]), pack2(s[2 * pr + 1][2], s[2 * pr + 1][3]));
-      const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
+  for (int pr = 0; pr < 2; ++pr) {
+    bf16x8 pf[QG];
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        if (dt < n_dt) {
-          const bf16_t* vr = vt + (int64_t)(16 * dt + r) * page_size + 32 * pr + 4 * c;
-          const uint2 a = *reinterpret_cast<const uint2*>(vr);
-          const uint2 b = *reinterpret_cast<const uint2*>(vr + 16);
-          const bf16x8 vf = __builtin_bit_cast(bf16x8, make_uint4(a.x, a.y, b.x, b.y));
-          o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[dt], 0, 0, 0);
-        }
+    for (int g = 0; g < QG; ++g) {
+      const u32x4 pw = {pack2(s[g][2 * pr][0], s[g][2 * pr][1]), pack2(s[g][2 * pr][2], s[g][2 * pr][3]),
+                        pack2(s[g][2 * pr + 1][0], s[g][2 * pr + 1][1]), pack2(s[g][2 * pr + 1][2], s[g][2 * pr + 1][3])};
+      pf[g] = __builtin_bit_cast(bf16x8, pw);
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      if (dt < n_dt) {
+        const bf16_t* vr = vt + (16 * dt + r) * v_stride + 32 * pr + 4 * c;
+        const u32x2 lo = *reinterpret_cast<const u32x2*>(vr);
+        const u32x2 hi = *reinterpret_cast<const u32x2*>(vr + 16);
+        const u32x4 both = {lo.x, lo.y, hi.x, hi.y};
+        const bf16x8 vf = __builtin_bit_cast(bf16x8, both);
+#pragma unroll
+        for (int g = 0; g < QG; ++g) o[g][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[g], o[g][dt], 0, 0, 0);
       }
     }
+  }
+}
+
+// Runs the wave's 16 columns over tiles [tile_beg, tile_end) straight from the cache pages.
+template <int DT>
+__device__ __forceinline__ void attend(f32x4 (&o)[1][DT], float (&m_run)[1], float (&l_run)[1],
+                                       const bf16x8 (&qf)[1][(DT + 1) / 2], const bf16_t* kh, const bf16_t* vh,
+                                       const int* table, int page_size, int64_t page_stride, int hd, int tile_beg,
+                                       int tile_end, int p_q, int lo_q, float scale) {
+  const int pq[1] = {p_q}, lq[1] = {lo_q};
+  for (int tile = tile_beg; tile < tile_end; ++tile) {
+    const int pos0 = tile * TILE;
+    const int page = table[pos0 / page_size];
+    const int in_page = pos0 % page_size;
+    const bf16_t* kt = kh + (int64_t)page * page_stride + (int64_t)in_page * hd;      // [row][hd]
+    const bf16_t* vt = vh + (int64_t)page * page_stride + in_page;                     // [hd][row]
+    tile_step<DT, 1>(o, m_run, l_run, qf, kt, hd, vt, page_size, hd, pos0, pq, lq, scale);
   }
 }
 
@@ -156,42 +182,84 @@ __device__ __forceinline__ void load_query(bf16x8 (&qf)[(DT + 1) / 2], const bf1
 }
 
 // ------------------------------------------------------------------------------------------ whole prompts
-// grid (ceil(longest run of new tokens / 64), nh, B), block 256: wave w takes tokens 64 x + 16 w .. + 15 of
-// sequence z.  The cache already holds the step's keys and values.
-template <int DT>
+// grid (ceil(longest run of new tokens / (64 QG)), nh, B), block 256: wave w takes tokens 16 QG (4 x + w) .. of
+// sequence z, QG groups of 16.  The cache already holds the step's keys and values.  The workgroup brings each
+// tile of keys and values into LDS once (key rows padded by KPAD, value rows VSTR long, so that the operand
+// reads do not collide) and its four waves read their operands from there.
+#define KPAD 8
+#define VSTR 68
+
+template <int DT, int QG>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_kernel(AttnArgs a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  bf16_t* Ks = (bf16_t*)smem_raw;                    // [TILE][hd + KPAD]
+  bf16_t* Vs = Ks + TILE * (a.hd + KPAD);            // [hd][VSTR]
+  constexpr int QW = 16 * QG;
   const int seq = blockIdx.z, h = blockIdx.y;
-  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, r = lane % 16, c = lane / 16;
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, r = lane % 16, c = lane / 16;
   const int t0 = a.cu_seqlens[seq], n = a.cu_seqlens[seq + 1] - t0;
-  const int q0 = blockIdx.x * 64 + wave * 16;
-  if (q0 >= n) return;
+  const int qb = blockIdx.x * 4 * QW;
+  if (qb >= n) return;
   const int start = a.start[seq];
-  const int qi = q0 + r;
-  const bool valid = qi < n;
-  const int p_q = valid ? start + qi : -1;
-  const int lo_q = a.window > 0 ? max(0, p_q - a.window + 1) : 0;
   const int kvh = h / (a.nh / a.nkv);
   const int64_t head_off = (int64_t)kvh * a.page_size * a.hd;
   const int* table = a.block_table + (size_t)a.slots[seq] * a.bt_stride;
 
-  bf16x8 qf[(DT + 1) / 2];
-  load_query<DT>(qf, a.q + ((size_t)(t0 + (valid ? qi : 0)) * a.nh + h) * a.hd, a.hd, valid);
-  f32x4 o[DT];
+  int p_q[QG], lo_q[QG];
+  bf16x8 qf[QG][(DT + 1) / 2];
+  f32x4 o[QG][DT];
+  float m_run[QG], l_run[QG];
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m_run = -INFINITY, l_run = 0.f;
-  const int p_first = start + q0, p_last = start + min(q0 + 15, n - 1);
-  const int lo_first = a.window > 0 ? max(0, p_first - a.window + 1) : 0;
-  attend<DT>(o, m_run, l_run, qf, a.k_pool + head_off, a.v_pool + head_off, table, a.page_size, a.page_stride, a.hd,
-             lo_first / TILE, p_last / TILE + 1, p_q, lo_q, a.scale);
-  if (!valid) return;
-  const float inv = 1.0f / l_run;
-  bf16_t* orow = a.out + ((size_t)(t0 + qi) * a.nh + h) * a.hd;
+  for (int g = 0; g < QG; ++g) {
+    const int qi = qb + wave * QW + g * 16 + r;
+    const bool valid = qi < n;
+    p_q[g] = valid ? start + qi : -1;
+    lo_q[g] = a.window > 0 ? max(0, p_q[g] - a.window + 1) : 0;
+    load_query<DT>(qf[g], a.q + ((size_t)(t0 + (valid ? qi : 0)) * a.nh + h) * a.hd, a.hd, valid);
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) {
-    if (16 * dt < a.hd) {
-      const uint2 w = make_uint2(pack2(o[dt][0] * inv, o[dt][1] * inv), pack2(o[dt][2] * inv, o[dt][3] * inv));
-      *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * c) = w;
+    for (int dt = 0; dt < DT; ++dt) o[g][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    m_run[g] = -INFINITY;
+    l_run[g] = 0.f;
+  }
+  // tiles the workgroup goes through, and those among them that this wave's tokens can see
+  const int wg_first = start + qb, wg_last = start + min(qb + 4 * QW, n) - 1;
+  const int tile_beg = (a.window > 0 ? max(0, wg_first - a.window + 1) : 0) / TILE, tile_end = wg_last / TILE + 1;
+  const int wq0 = qb + wave * QW;
+  const bool wave_has = wq0 < n;
+  const int wave_first = start + wq0, wave_last = start + min(wq0 + QW, n) - 1;
+  const int wave_beg = (a.window > 0 ? max(0, wave_first - a.window + 1) : 0) / TILE;
+  const int wave_end = wave_has ? wave_last / TILE + 1 : 0;
+  const int hd = a.hd, kcpr = hd / 8;
+  for (int tile = tile_beg; tile < tile_end; ++tile) {
+    const int pos0 = tile * TILE;
+    const int page = table[pos0 / a.page_size];
+    const int in_page = pos0 % a.page_size;
+    const bf16_t* kg = a.k_pool + head_off + (int64_t)page * a.page_stride + (int64_t)in_page * hd;
+    const bf16_t* vg = a.v_pool + head_off + (int64_t)page * a.page_stride + in_page;
+    for (int i = tid; i < TILE * kcpr; i += 256) {
+      const int row = i / kcpr, ch = i % kcpr;
+      *reinterpret_cast<u32x4*>(Ks + row * (hd + KPAD) + ch * 8) = *reinterpret_cast<const u32x4*>(kg + row * hd + ch * 8);
+    }
+    for (int i = tid; i < hd * 16; i += 256) {
+      const int d = i / 16, ch = i % 16;
+      *reinterpret_cast<u32x2*>(Vs + d * VSTR + ch * 4) = *reinterpret_cast<const u32x2*>(vg + (int64_t)d * a.page_size + ch * 4);
+    }
+    __syncthreads();
+    if (tile >= wave_beg && tile < wave_end)
+      tile_step<DT, QG>(o, m_run, l_run, qf, Ks, hd + KPAD, Vs, VSTR, hd, pos0, p_q, lo_q, a.scale);
+    __syncthreads();
+  }
+#pragma unroll
+  for (int g = 0; g < QG; ++g) {
+    if (p_q[g] < 0) continue;
+    const float inv = 1.0f / l_run[g];
+    bf16_t* orow = a.out + ((size_t)(t0 + p_q[g] - start) * a.nh + h) * a.hd;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      if (16 * dt < a.hd) {
+        const u32x2 w = {pack2(o[g][dt][0] * inv, o[g][dt][1] * inv), pack2(o[g][dt][2] * inv, o[g][dt][3] * inv)};
+        *reinterpret_cast<u32x2*>(orow + 16 * dt + 4 * c) = w;
+      }
     }
   }
 }
@@ -217,12 +285,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DT > 8 ? 2 :
   const int* table = a.block_table + (size_t)a.slots[b] * a.bt_stride;
   const int t = a.cu_seqlens[b];
 
-  bf16x8 qf[(DT + 1) / 2];
-  load_query<DT>(qf, a.q + ((size_t)t * a.nh + h) * a.hd, a.hd, valid);
-  f32x4 o[DT];
+  bf16x8 qf[1][(DT + 1) / 2];
+  load_query<DT>(qf[0], a.q + ((size_t)t * a.nh + h) * a.hd, a.hd, valid);
+  f32x4 o[1][DT];
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m_run = -INFINITY, l_run = 0.f;
+  for (int dt = 0; dt < DT; ++dt) o[0][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run[1] = {-INFINITY}, l_run[1] = {0.f};
   attend<DT>(o, m_run, l_run, qf, a.k_pool + head_off, a.v_pool + head_off, table, a.page_size, a.page_stride, a.hd,
              tile_beg, tile_end, valid ? p : -1, lo, a.scale);
   if (!valid) return;
@@ -231,12 +299,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DT > 8 ? 2 :
   for (int dt = 0; dt < DT; ++dt) {
     if (16 * dt < a.hd) {
 #pragma unroll
-      for (int v = 0; v < 4; ++v) out[16 * dt + 4 * c + v] = o[dt][v];
+      for (int v = 0; v < 4; ++v) out[16 * dt + 4 * c + v] = o[0][dt][v];
     }
   }
   if (c == 0) {
-    out[a.hd] = m_run;
-    out[a.hd + 1] = l_run;
+    out[a.hd] = m_run[0];
+    out[a.hd + 1] = l_run[0];
   }
 }
 
@@ -278,9 +346,13 @@ __global__ __launch_bounds__(64) void attn_join_kernel(AttnArgs a) {
 }
 
 // ------------------------------------------------------------------------------------------ launch
-template <int DT>
+template <int DT, int QG>
 static void launch_prefill(const AttnArgs& a, int B, int max_new, hipStream_t st) {
-  hipLaunchKernelGGL(attn_prefill_kernel<DT>, dim3((max_new + 63) / 64, a.nh, B), dim3(256), 0, st, a);
+  const size_t shmem = ((size_t)TILE * (a.hd + KPAD) + (size_t)a.hd * VSTR) * sizeof(bf16_t);
+  if (shmem > 48 * 1024)
+    hipFuncSetAttribute((const void*)attn_prefill_kernel<DT, QG>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+  hipLaunchKernelGGL((attn_prefill_kernel<DT, QG>), dim3((max_new + 64 * QG - 1) / (64 * QG), a.nh, B), dim3(256), shmem,
+                     st, a);
 }
 template <int DT>
 static void launch_decode(const AttnArgs& a, int B, hipStream_t st) {
@@ -316,9 +388,10 @@ TQ_API int tq_attention_mfma(const void* q, const void* k_pool, const void* v_po
     else if (dt <= 8) launch_decode<8>(a, B, st);
     else launch_decode<16>(a, B, st);
   } else {
-    if (dt <= 4) launch_prefill<4>(a, B, max_new, st);
-    else if (dt <= 8) launch_prefill<8>(a, B, max_new, st);
-    else launch_prefill<16>(a, B, max_new, st);
+    // two groups of 16 tokens per wave when the runs are long enough to fill them and registers allow
+    if (dt <= 4) { if (max_new > 64) launch_prefill<4, 2>(a, B, max_new, st); else launch_prefill<4, 1>(a, B, max_new, st); }
+    else if (dt <= 8) { if (max_new > 64) launch_prefill<8, 2>(a, B, max_new, st); else launch_prefill<8, 1>(a, B, max_new, st); }
+    else launch_prefill<16, 1>(a, B, max_new, st);
   }
   TQ_LAUNCH_CHECK();
   return 0;

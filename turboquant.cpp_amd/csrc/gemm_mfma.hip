@@ -10,8 +10,9 @@
 //    add their partial sums in wave order through LDS, so that even a narrow matrix gives the chip enough
 //    waves and bytes in flight.  How k is split depends on N and K only, never on the number of rows.
 //  * gemm_tile_kernel, for many rows (prompts): tiles of BM x 128 outputs with 64 of k at a time staged
-//    through LDS (16-byte chunks, XOR-swizzled by row so that the operand reads of
-//    v_mfma_f32_32x32x16_bf16 do not collide), the next tile prefetched into registers meanwhile.
+//    through two LDS buffers (16-byte chunks, XOR-swizzled by row so that the operand reads of
+//    v_mfma_f32_32x32x16_bf16 do not collide); while one buffer is multiplied the next tile is written into
+//    the other and the one after that is on its way from memory.
 //
 // Operand layouts (wave of 64 lanes): 16x16x32: A lane l = row l%16, k 8*(l/16)..+7; B lane l = column l%16,
 // same k; D lane l = column l%16, rows 4*(l/16)+v, v<4.  32x32x16: A lane l = row l%32, k 8*(l/32)..+7;
@@ -21,6 +22,7 @@
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 struct MfmaGemmArgs {
   const bf16_t* a;
@@ -188,6 +190,8 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(MfmaGemmArgs g) {
   constexpr int A_CH = BM * 8 / 256;             // 16-byte chunks of the a tile per thread
   constexpr int W_CH = TBN * 8 / 256;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  // two buffers, each a tile of `a`, one of `w` and (gated pair) one of `w2`
+  constexpr int BUF = (BM + TBN * (DUAL ? 2 : 1)) * TBK;
   bf16_t* As = (bf16_t*)smem;
   bf16_t* Ws = As + BM * TBK;
   bf16_t* Vs = Ws + TBN * TBK;
@@ -251,48 +255,58 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(MfmaGemmArgs g) {
         if (DUAL) acc2[mi][ni][v] = 0.f;
       }
 
-  uint4 pa[A_CH], pw[W_CH], pv[DUAL ? W_CH : 1];
-  const uint4 z = make_uint4(0, 0, 0, 0);
-  auto fetch = [&](int k0) {
-    const bool k_ok = k0 + ch_of_thread * 8 < g.K;
-#pragma unroll
-    for (int i = 0; i < A_CH; ++i) pa[i] = a_src[i] && k_ok ? *reinterpret_cast<const uint4*>(a_src[i] + k0) : z;
-#pragma unroll
-    for (int i = 0; i < W_CH; ++i) {
-      pw[i] = w_src[i] && k_ok ? *reinterpret_cast<const uint4*>(w_src[i] + k0) : z;
-      if (DUAL) pv[i] = v_src[i] && k_ok ? *reinterpret_cast<const uint4*>(v_src[i] + k0) : z;
-    }
-  };
-  auto stage = [&]() {
-#pragma unroll
-    for (int i = 0; i < A_CH; ++i) *reinterpret_cast<uint4*>(As + a_dst[i]) = pa[i];
-#pragma unroll
-    for (int i = 0; i < W_CH; ++i) {
-      *reinterpret_cast<uint4*>(Ws + w_dst[i]) = pw[i];
-      if (DUAL) *reinterpret_cast<uint4*>(Vs + w_dst[i]) = pv[i];
-    }
-  };
+  u32x4 pa[A_CH], pw[W_CH], pv[DUAL ? W_CH : 1];
+  const u32x4 z = {0u, 0u, 0u, 0u};
+  // FETCH: the thread's chunks of the tile at k0 into registers.  STAGE: registers into LDS.  (Written as macros
+  // so that the small arrays above are only ever indexed by constants and stay in registers.)
+#define TQ_FETCH(k0)                                                                                          \
+  do {                                                                                                        \
+    const bool k_ok = (k0) + ch_of_thread * 8 < g.K;                                                          \
+    _Pragma("unroll") for (int i = 0; i < A_CH; ++i)                                                          \
+        pa[i] = a_src[i] && k_ok ? *reinterpret_cast<const u32x4*>(a_src[i] + (k0)) : z;                      \
+    _Pragma("unroll") for (int i = 0; i < W_CH; ++i) {                                                        \
+      pw[i] = w_src[i] && k_ok ? *reinterpret_cast<const u32x4*>(w_src[i] + (k0)) : z;                        \
+      if (DUAL) pv[i] = v_src[i] && k_ok ? *reinterpret_cast<const u32x4*>(v_src[i] + (k0)) : z;              \
+    }                                                                                                         \
+  } while (0)
+#define TQ_STAGE(off)                                                                                         \
+  do {                                                                                                        \
+    _Pragma("unroll") for (int i = 0; i < A_CH; ++i) *reinterpret_cast<u32x4*>(As + (off) + a_dst[i]) = pa[i]; \
+    _Pragma("unroll") for (int i = 0; i < W_CH; ++i) {                                                        \
+      *reinterpret_cast<u32x4*>(Ws + (off) + w_dst[i]) = pw[i];                                               \
+      if (DUAL) *reinterpret_cast<u32x4*>(Vs + (off) + w_dst[i]) = pv[i];                                     \
+    }                                                                                                         \
+  } while (0)
 
-  fetch(0);
-  stage();
+  // Tile t is computed from buffer t % 2 while tile t + 1 goes from registers into the other buffer and tile
+  // t + 2 is on its way from memory into registers: one barrier per step of 64 of k.
+  TQ_FETCH(0);
+  TQ_STAGE(0);
+  if (TBK < g.K) TQ_FETCH(TBK);
   __syncthreads();
   const int lr = lane % 32, lc = lane / 32;
-  for (int k0 = 0; k0 < g.K; k0 += TBK) {
-    const bool more = k0 + TBK < g.K;
-    if (more) fetch(k0 + TBK);
+  int cur = 0;
+  for (int k0 = 0; k0 < g.K; k0 += TBK, cur ^= BUF) {
+    if (k0 + TBK < g.K) {
+      TQ_STAGE(cur ^ BUF);
+      if (k0 + 2 * TBK < g.K) TQ_FETCH(k0 + 2 * TBK);
+    }
+    const bf16_t* Ac = As + cur;
+    const bf16_t* Wc = Ws + cur;
+    const bf16_t* Vc = Vs + cur;
 #pragma unroll
     for (int j = 0; j < TBK / 16; ++j) {
       bf16x8 af[MI], wf[NI], vf[DUAL ? NI : 1];
 #pragma unroll
       for (int mi = 0; mi < MI; ++mi) {
         const int row = wm * 64 + mi * 32 + lr;
-        af[mi] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(As + swz<BM>(row, 2 * j + lc)));
+        af[mi] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(Ac + swz<BM>(row, 2 * j + lc)));
       }
 #pragma unroll
       for (int ni = 0; ni < NI; ++ni) {
         const int row = wn * (NI * 32) + ni * 32 + lr;
-        wf[ni] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(Ws + swz<BM>(row, 2 * j + lc)));
-        if (DUAL) vf[ni] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(Vs + swz<BM>(row, 2 * j + lc)));
+        wf[ni] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(Wc + swz<BM>(row, 2 * j + lc)));
+        if (DUAL) vf[ni] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(Vc + swz<BM>(row, 2 * j + lc)));
       }
 #pragma unroll
       for (int mi = 0; mi < MI; ++mi)
@@ -303,11 +317,9 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(MfmaGemmArgs g) {
         }
     }
     __syncthreads();
-    if (more) {
-      stage();
-      __syncthreads();
-    }
   }
+#undef TQ_FETCH
+#undef TQ_STAGE
 
 #pragma unroll
   for (int ni = 0; ni < NI; ++ni) {
@@ -360,7 +372,7 @@ static int launch_stream(const MfmaGemmArgs& g, bool dual, bool out_act, int row
 template <int BM>
 static int launch_tile(const MfmaGemmArgs& g, bool dual, bool out_act, hipStream_t st) {
   const dim3 grid((g.M + BM - 1) / BM, (g.N + TBN - 1) / TBN);
-  const size_t shmem = (size_t)(BM + TBN * (dual ? 2 : 1)) * TBK * sizeof(bf16_t);
+  const size_t shmem = (size_t)2 * (BM + TBN * (dual ? 2 : 1)) * TBK * sizeof(bf16_t);
 #define TQ_TILE(D, O)                                                                                          \
   do {                                                                                                         \
     if (shmem > 48 * 1024)                                                                                     \

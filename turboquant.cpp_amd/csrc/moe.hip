@@ -30,48 +30,74 @@ __device__ __forceinline__ void load8(const bf16_t* p, float (&w)[8]) {
   }
 }
 
-template <class W>
+template <int TG>
+__device__ __forceinline__ void router_chunk(const float* xs, int H, int j, const float (&w)[8], float (&s)[TG]) {
+#pragma unroll
+  for (int r = 0; r < TG; ++r) {
+    const float4 a = *reinterpret_cast<const float4*>(xs + r * H + j);
+    const float4 b = *reinterpret_cast<const float4*>(xs + r * H + j + 4);
+    s[r] = fmaf(a.x, w[0], s[r]);
+    s[r] = fmaf(a.y, w[1], s[r]);
+    s[r] = fmaf(a.z, w[2], s[r]);
+    s[r] = fmaf(a.w, w[3], s[r]);
+    s[r] = fmaf(b.x, w[4], s[r]);
+    s[r] = fmaf(b.y, w[5], s[r]);
+    s[r] = fmaf(b.z, w[6], s[r]);
+    s[r] = fmaf(b.w, w[7], s[r]);
+  }
+}
+
+// TG: tokens per workgroup (tokens beyond T are zeros in LDS and are not stored).
+template <class W, int TG>
 __global__ __launch_bounds__(256) void router_logits_kernel(const float* __restrict__ x, const W* __restrict__ wr,
                                                             const W* __restrict__ shared_w, int rows, int E,
-                                                            float* __restrict__ logits, int T, int H, int tg) {
-  extern __shared__ float xs[];      // [tg][H]
-  const int t0 = blockIdx.x * tg;
-  const int nt = min(tg, T - t0);
+                                                            float* __restrict__ logits, int T, int H) {
+  extern __shared__ float xs[];      // [TG][H]
+  const int t0 = blockIdx.x * TG;
+  const int nt = min(TG, T - t0);
   const int wave = threadIdx.x / TQ_WAVE, lane = threadIdx.x % TQ_WAVE;
-  for (int i = threadIdx.x; i < nt * H; i += blockDim.x) xs[i] = x[(size_t)t0 * H + i];
-  __syncthreads();
   const bool vec = H % 8 == 0;
-  for (int e = blockIdx.y * 4 + wave; e < rows; e += gridDim.y * 4) {
+  if (vec) {
+    const float4* src = reinterpret_cast<const float4*>(x + (size_t)t0 * H);
+    float4* dst = reinterpret_cast<float4*>(xs);
+    for (int i = threadIdx.x; i < TG * H / 4; i += blockDim.x) dst[i] = i < nt * H / 4 ? src[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+  } else {
+    for (int i = threadIdx.x; i < TG * H; i += blockDim.x) xs[i] = i < nt * H ? x[(size_t)t0 * H + i] : 0.f;
+  }
+  __syncthreads();
+  // workgroups start at different rows, so that they do not all ask for the same row at once
+  const int rot = (blockIdx.x * 5) % rows;
+  const int h_quad = H / (TQ_WAVE * 8 * 4) * (TQ_WAVE * 8 * 4);     // the part of a row that goes four chunks at a time
+  for (int idx = blockIdx.y * 4 + wave; idx < rows; idx += gridDim.y * 4) {
+    const int e = idx + rot < rows ? idx + rot : idx + rot - rows;
     const W* row = e < E ? wr + (size_t)e * H : shared_w;
-    float s[RT];
+    float s[TG];
 #pragma unroll
-    for (int r = 0; r < RT; ++r) s[r] = 0.f;
+    for (int r = 0; r < TG; ++r) s[r] = 0.f;
     if (vec) {
-      for (int j = lane * 8; j < H; j += TQ_WAVE * 8) {
+      for (int j0 = lane * 8; j0 < h_quad; j0 += TQ_WAVE * 8 * 4) {   // four chunks asked for before the first is used
+        float w[4][8];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) load8(row + j0 + c * TQ_WAVE * 8, w[c]);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) router_chunk<TG>(xs, H, j0 + c * TQ_WAVE * 8, w[c], s);
+      }
+      for (int j = h_quad + lane * 8; j < H; j += TQ_WAVE * 8) {
         float w[8];
         load8(row + j, w);
-#pragma unroll
-        for (int r = 0; r < RT; ++r) {
-          if (r < nt) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) s[r] = fmaf(xs[r * H + j + i], w[i], s[r]);
-          }
-        }
+        router_chunk<TG>(xs, H, j, w, s);
       }
     } else {
       for (int j = lane; j < H; j += TQ_WAVE) {
         const float w = to_f32(row[j]);
 #pragma unroll
-        for (int r = 0; r < RT; ++r)
-          if (r < nt) s[r] = fmaf(xs[r * H + j], w, s[r]);
+        for (int r = 0; r < TG; ++r) s[r] = fmaf(xs[r * H + j], w, s[r]);
       }
     }
 #pragma unroll
-    for (int r = 0; r < RT; ++r) {
-      if (r < nt) {
-        const float v = wave_sum(s[r]);
-        if (lane == 0) logits[(size_t)(t0 + r) * rows + e] = v;
-      }
+    for (int r = 0; r < TG; ++r) {
+      const float v = wave_sum(s[r]);
+      if (lane == 0 && r < nt) logits[(size_t)(t0 + r) * rows + e] = v;
     }
   }
 }
@@ -143,7 +169,7 @@ TQ_API int tq_router_topk(const float* x, const void* wr, const void* shared_w, 
   if (T <= 0) return 0;
   if (topk < 1 || topk > 64 || topk > E || E > 8192) return TQ_ERR_UNSUPPORTED;
   int tg = RT;
-  while (tg > 1 && (size_t)tg * H * sizeof(float) > 128 * 1024) tg /= 2;
+  while (tg > 1 && (size_t)tg * H * sizeof(float) > 32 * 1024) tg /= 2;   // small enough for several workgroups per CU
   const size_t shmem = (size_t)tg * H * sizeof(float);
   if (shmem > 160 * 1024) return TQ_ERR_UNSUPPORTED;
   const int rows = E + (shared_w ? 1 : 0);
@@ -151,12 +177,21 @@ TQ_API int tq_router_topk(const float* x, const void* wr, const void* shared_w, 
   // with few groups of tokens the rows are dealt over more workgroups
   int row_groups = 256 / groups;
   row_groups = row_groups < 1 ? 1 : (row_groups > (rows + 3) / 4 ? (rows + 3) / 4 : row_groups);
+#define TQ_ROUTER(TGV)                                                                                              \
+  do {                                                                                                              \
+    if (shmem > 48 * 1024)                                                                                          \
+      hipFuncSetAttribute((const void*)router_logits_kernel<W, TGV>, hipFuncAttributeMaxDynamicSharedMemorySize,    \
+                          (int)shmem);                                                                              \
+    hipLaunchKernelGGL((router_logits_kernel<W, TGV>), dim3(groups, row_groups), dim3(256), shmem, st, x,           \
+                       (const W*)wr, (const W*)shared_w, rows, E, logits, T, H);                                    \
+  } while (0)
   TQ_DISPATCH_W(wtype, {
-    if (shmem > 48 * 1024)
-      hipFuncSetAttribute((const void*)router_logits_kernel<W>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
-    hipLaunchKernelGGL(router_logits_kernel<W>, dim3(groups, row_groups), dim3(256), shmem, st, x, (const W*)wr,
-                       (const W*)shared_w, rows, E, logits, T, H, tg);
+    if (tg == 8) TQ_ROUTER(8);
+    else if (tg == 4) TQ_ROUTER(4);
+    else if (tg == 2) TQ_ROUTER(2);
+    else TQ_ROUTER(1);
   });
+#undef TQ_ROUTER
   TQ_LAUNCH_CHECK();
   hipLaunchKernelGGL(router_select_kernel, dim3((T + 3) / 4), dim3(256), (size_t)4 * E * sizeof(float), st, logits,
                      rows, E, topk, renorm, ids, weights, shared_gate, T);
