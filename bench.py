@@ -73,6 +73,7 @@ def main() -> int:
     ap.add_argument("--points-context", type=int, default=2048)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true")
+    ap.add_argument("--prefill-only", action="store_true", help="time only the prompt step (for profiles)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single device)")
@@ -152,6 +153,11 @@ def main() -> int:
         return min(times[1:])
 
     pf = run_prefill(PREFILL_TOKENS)
+    if args.prefill_only:
+        print(json.dumps({"metric": f"prefill tok/s at {PREFILL_TOKENS} tokens", "value": round(PREFILL_TOKENS / pf, 1),
+                          "unit": "tok/s", "ms": round(pf * 1e3, 3), "layers": args.layers, "dtype": short,
+                          "frac": round(prefill_flops(cfg, args.layers, PREFILL_TOKENS) / pf / PEAK_FLOPS[short], 4)}))
+        return 0
     sec, mean_ctx = run_decode(args.batch, args.context, args.steps, args.warmup)
     value = args.batch / sec
     read = decode_bytes(cfg, args.layers, args.batch, mean_ctx, 2 if act == "bfloat16" else 4)

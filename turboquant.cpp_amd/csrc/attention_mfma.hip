@@ -5,14 +5,15 @@
 // share keys and values and runs over tiles of 64 cache positions (a page, or a quarter of one):
 //
 //   S^T = K Q^T     v_mfma_f32_16x16x32_bf16 with A = 16 keys x 32 of hd (16 bytes per lane straight from the
-//                   page, keys lie [row][hd]) and B = the columns' queries, kept in registers.  Lane l then
-//                   holds, for column l % 16, the scores of keys 4 * (l / 16) + v of each 16-key block.
+//                   page, keys lie [row][hd]) and B = the columns' queries, kept in registers.  The 16 rows of
+//                   block jt are not 16 consecutive keys: row i is key 32 (jt / 2) + 8 (i / 4) + 4 (jt % 2) + i % 4,
+//                   so that lane l, which holds rows 4 (l / 16) + v of every block for column l % 16, holds 8
+//                   consecutive keys across the two blocks of a pair.
 //   softmax         per column, that is per lane: maxima and sums over a lane's registers and over the four
 //                   lanes l % 16 + 16 c; all in float, running maximum across tiles.
-//   O^T += V^T P^T  A = 16 of hd x 32 keys (values lie transposed in the page, [hd][row], so a lane reads 4
-//                   consecutive keys of one dimension with 8 bytes) and B = the probabilities exactly as the
-//                   lane already holds them: the 32 keys of one product are the lane group's 4 keys of two
-//                   16-key blocks.  No transpose through LDS anywhere.
+//   O^T += V^T P^T  A = 16 of hd x 32 keys (values lie transposed in the page, [hd][row], so a lane reads its 8
+//                   consecutive keys of one dimension with 16 bytes) and B = the probabilities exactly as the
+//                   lane already holds them.  No transpose through LDS anywhere.
 //
 // Two entry points share this: whole prompts (columns = 16 consecutive tokens of a sequence, one head; four
 // waves per workgroup) and decoding (columns = the query heads that share one kv head, one token; the cache is
@@ -90,7 +91,7 @@ __device__ __forceinline__ void tile_step(f32x4 (&o)[QG][DT], float (&m_run)[QG]
     for (int ks = 0; ks < KS; ++ks) {
       if (ks < n_ks) {
         const int d0 = 32 * ks + 8 * c;
-        const bf16x8 kf = d0 < hd ? ld16(kt + (16 * jt + r) * k_stride + d0) : zero16();
+        const bf16x8 kf = d0 < hd ? ld16(kt + (32 * (jt / 2) + 8 * (r / 4) + 4 * (jt % 2) + r % 4) * k_stride + d0) : zero16();
 #pragma unroll
         for (int g = 0; g < QG; ++g) s[g][jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[g][ks], s[g][jt], 0, 0, 0);
       }
@@ -104,7 +105,7 @@ __device__ __forceinline__ void tile_step(f32x4 (&o)[QG][DT], float (&m_run)[QG]
     for (int jt = 0; jt < 4; ++jt)
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
-        const int key = pos0 + 16 * jt + 4 * c + v;
+        const int key = pos0 + 32 * (jt / 2) + 8 * c + 4 * (jt % 2) + v;
         const bool ok = key <= p_q[g] && key >= lo_q[g];
         s[g][jt][v] = ok ? s[g][jt][v] * scale : -INFINITY;
         m_tile = fmaxf(m_tile, s[g][jt][v]);
@@ -142,11 +143,7 @@ __device__ __forceinline__ void tile_step(f32x4 (&o)[QG][DT], float (&m_run)[QG]
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       if (dt < n_dt) {
-        const bf16_t* vr = vt + (16 * dt + r) * v_stride + 32 * pr + 4 * c;
-        const u32x2 lo = *reinterpret_cast<const u32x2*>(vr);
-        const u32x2 hi = *reinterpret_cast<const u32x2*>(vr + 16);
-        const u32x4 both = {lo.x, lo.y, hi.x, hi.y};
-        const bf16x8 vf = __builtin_bit_cast(bf16x8, both);
+        const bf16x8 vf = ld16(vt + (16 * dt + r) * v_stride + 32 * pr + 8 * c);
 #pragma unroll
         for (int g = 0; g < QG; ++g) o[g][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[g], o[g][dt], 0, 0, 0);
       }
@@ -187,7 +184,7 @@ __device__ __forceinline__ void load_query(bf16x8 (&qf)[(DT + 1) / 2], const bf1
 // tile of keys and values into LDS once (key rows padded by KPAD, value rows VSTR long, so that the operand
 // reads do not collide) and its four waves read their operands from there.
 #define KPAD 8
-#define VSTR 68
+#define VSTR 72
 
 template <int DT, int QG>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_kernel(AttnArgs a) {
@@ -240,9 +237,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
       const int row = i / kcpr, ch = i % kcpr;
       *reinterpret_cast<u32x4*>(Ks + row * (hd + KPAD) + ch * 8) = *reinterpret_cast<const u32x4*>(kg + row * hd + ch * 8);
     }
-    for (int i = tid; i < hd * 16; i += 256) {
-      const int d = i / 16, ch = i % 16;
-      *reinterpret_cast<u32x2*>(Vs + d * VSTR + ch * 4) = *reinterpret_cast<const u32x2*>(vg + (int64_t)d * a.page_size + ch * 4);
+    for (int i = tid; i < hd * 8; i += 256) {
+      const int d = i / 8, ch = i % 8;
+      *reinterpret_cast<u32x4*>(Vs + d * VSTR + ch * 8) = *reinterpret_cast<const u32x4*>(vg + (int64_t)d * a.page_size + ch * 8);
     }
     __syncthreads();
     if (tile >= wave_beg && tile < wave_end)

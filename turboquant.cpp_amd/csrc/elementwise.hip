@@ -139,21 +139,26 @@ TQ_API int tq_rope_kv_write(const float* qkv, const int* positions, const int* s
 // out[t] = sum_j weights[t][j] * y[slot[t][j]]   (j ascending: the order in which experts were selected,
 //          /root/reference/src/engine/tq_moe.c:720,864-999)
 //        + gate[t] * sum_s shared[s][t]           (shared expert last, tq_moe.c:1005-1058)
-__global__ void moe_combine_kernel(const float* __restrict__ y, const int* __restrict__ pair_slot,
-                                   const float* __restrict__ weights, int topk, const float* __restrict__ shared,
-                                   int S, size_t shared_stride, const float* __restrict__ gate,
-                                   float* __restrict__ out, int H) {
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y, const int* __restrict__ pair_slot,
+                                                          const float* __restrict__ weights, int topk,
+                                                          const float* __restrict__ shared, int S, size_t shared_stride,
+                                                          const float* __restrict__ gate, float* __restrict__ out, int H) {
+  __shared__ int slot[64];
+  __shared__ float wgt[64];
   const int t = blockIdx.x;
+  if (threadIdx.x < topk) {      // the token's rows and weights once, not once per element
+    slot[threadIdx.x] = pair_slot[t * topk + threadIdx.x];
+    wgt[threadIdx.x] = weights[t * topk + threadIdx.x];
+  }
+  __syncthreads();
+  const float g = gate ? gate[t] : 1.0f;
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     float acc = 0.f;
-    for (int j = 0; j < topk; ++j) {
-      const int p = pair_slot[t * topk + j];
-      acc += weights[t * topk + j] * y[(size_t)p * H + i];
-    }
+    for (int j = 0; j < topk; ++j) acc += wgt[j] * y[(size_t)slot[j] * H + i];
     if (shared) {
       float sh = 0.f;
       for (int s = 0; s < S; ++s) sh += shared[s * shared_stride + (size_t)t * H + i];
-      acc += (gate ? gate[t] : 1.0f) * sh;
+      acc += g * sh;
     }
     out[(size_t)t * H + i] = acc;
   }
@@ -163,6 +168,7 @@ TQ_API int tq_moe_combine(const float* y, const int* pair_slot, const float* wei
                           const float* shared, int S, int64_t shared_stride, const float* gate, float* out, int T,
                           int H, hipStream_t st) {
   if (T <= 0) return 0;
+  if (topk < 1 || topk > 64) return TQ_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(256), 0, st, y, pair_slot, weights, topk, shared, S,
                      (size_t)shared_stride, gate, out, H);
   TQ_LAUNCH_CHECK();

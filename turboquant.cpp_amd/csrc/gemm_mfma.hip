@@ -180,8 +180,11 @@ __global__ __launch_bounds__(1024) void gemm_stream_kernel(MfmaGemmArgs g) {
 #define TBN 128
 #define TBK 64
 
+// Where 16-byte chunk `chunk` of row `row` lies in a tile: rows of 128 bytes, the chunk index XOR-ed with bits 1..3
+// of the row.  Measured with ds_read_b128 in the operand layout (lane l reads row l % 32): this runs at the full
+// 128 bytes per clock; XOR with bits 0..2 at 107, no swizzle at 31.
 template <int BM>
-__device__ __forceinline__ int swz(int row, int chunk) { return row * TBK + ((chunk ^ (row & 7)) << 3); }
+__device__ __forceinline__ int swz(int row, int chunk) { return row * TBK + ((chunk ^ ((row >> 1) & 7)) << 3); }
 
 template <int BM, bool DUAL, bool OUT_ACT>
 __global__ __launch_bounds__(256) void gemm_tile_kernel(MfmaGemmArgs g) {

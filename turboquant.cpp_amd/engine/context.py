@@ -15,10 +15,23 @@ class StepContext:
     cache: PagedCache
     act: str                          # "float32" or "bfloat16": the type of activations and cache
     device: torch.device
+    side_stream: "torch.cuda.Stream | None" = None   # a second stream for work that does not depend on the main line
 
     def kv(self, entry: int) -> KVView:
         """Keys and values of the schedule entry (or of the entry whose cache it reads)."""
         return self.cache.kv(entry)
+
+    def fork(self):
+        """Lets the side stream start from where the current stream is; returns it (None: run in line)."""
+        if self.side_stream is None:
+            return None
+        self.side_stream.wait_stream(torch.cuda.current_stream())
+        return self.side_stream
+
+    def join(self) -> None:
+        """The current stream waits for what the side stream has been given."""
+        if self.side_stream is not None:
+            torch.cuda.current_stream().wait_stream(self.side_stream)
 
     def state(self, entry: int) -> torch.Tensor:
         """The entry's fixed-size state, [slots, ...]; row ``slot`` belongs to the sequence in that slot."""

@@ -64,7 +64,8 @@ class DecodeGraph:
     def capture(self, slots, starts, tokens) -> torch.Tensor:
         self.fill(slots, starts, tokens)
         e = self.engine
-        ctx = StepContext(batch=self.batch(slots, starts), cache=e.cache, act=e.model.act, device=e.device)
+        ctx = StepContext(batch=self.batch(slots, starts), cache=e.cache, act=e.model.act, device=e.device,
+                          side_stream=e.side_stream)
         torch.cuda.synchronize()
         with torch.cuda.graph(self.graph, pool=self.pool):
             self.logits = e.model.forward(ctx)

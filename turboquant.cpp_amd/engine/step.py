@@ -34,6 +34,7 @@ class Engine:
         self.vocab_size = model.plan.vocab_size
         # decode steps are replayed as HIP graphs where a GPU runs them
         on_gpu = self.device is not None and self.device.type == "cuda"
+        self.side_stream = torch.cuda.Stream(device=self.device) if on_gpu else None     # default priority
         self.graphs = DecodeGraphs(self) if use_graphs and on_gpu and all(p.graph_safe for p in model.parts()) else None
 
     # ------------------------------------------------------------ sequences
@@ -100,7 +101,8 @@ class Engine:
                     torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
         if logits is None:
             batch = pack_step(slots, starts, token_lists, wants, self.device)
-            ctx = StepContext(batch=batch, cache=self.cache, act=self.model.act, device=self.device)
+            ctx = StepContext(batch=batch, cache=self.cache, act=self.model.act, device=self.device,
+                              side_stream=self.side_stream)
             logits = self.model.forward(ctx)
         for slot in slots:
             self.cache.commit(slot)

@@ -9,6 +9,8 @@ the reference's softmax over the chosen logits.
 """
 from __future__ import annotations
 
+import torch
+
 from ..csrc import ops
 from .base import ParamSpec, Part, register_part
 
@@ -61,6 +63,15 @@ class SparseMoE(Part):
 
     def forward(self, normed, normed32, ctx):
         T = normed.shape[0]
+        # the shared expert needs nothing from the router: it runs on a second stream beside the routed experts
+        shared, side = None, None
+        if self.shared_size > 0:
+            side = ctx.fork() if hasattr(ctx, "fork") else None
+            if side is not None:
+                with torch.cuda.stream(side):
+                    shared = self._shared(normed, ctx)
+            else:
+                shared = self._shared(normed, ctx)
         ids, weights, gate = ops.router_topk(normed32, self.router, self.shared_scale if self.shared_gated else None,
                                              self.top_k, self.renormalize, ctx.act)
         unit = 16 if T * self.top_k <= 16 * self.num_experts else 64
@@ -69,8 +80,10 @@ class SparseMoE(Part):
                      tile_group=tile_expert, n_tiles=n_tiles, tile_rows=unit)
         y = ops.gemm(h, self.expert_down, ctx.act, a_rows=sorted_token, tile_group=tile_expert, n_tiles=n_tiles,
                      tile_rows=unit, gather=False)
-        shared = None
-        if self.shared_size > 0:
-            hs = ops.gemm(normed, self.shared_gate, ctx.act, w2=self.shared_up, out_act=True)
-            shared = ops.gemm(hs, self.shared_down, ctx.act).unsqueeze(0)
+        if side is not None:
+            ctx.join()
         return ops.moe_combine(y, pair_slot, weights, shared, gate, ctx.act)
+
+    def _shared(self, normed, ctx):
+        hs = ops.gemm(normed, self.shared_gate, ctx.act, w2=self.shared_up, out_act=True)
+        return ops.gemm(hs, self.shared_down, ctx.act).unsqueeze(0)
