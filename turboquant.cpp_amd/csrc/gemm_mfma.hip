@@ -9,7 +9,7 @@
 //    `a` are read the same way and stay in cache.  The waves of a workgroup split k among them and
 //    add their partial sums in wave order through LDS, so that even a narrow matrix gives the chip enough
 //    waves and bytes in flight.  How k is split depends on N and K only, never on the number of rows.
-//  * gemm_tile_kernel, for many rows (prompts): tiles of BM x 128 outputs with 64 of k at a time staged
+//  * gemm_tile_kernel, for many rows (prompts): tiles of BM x 128 outputs by eight waves, 64 of k at a time staged
 //    through two LDS buffers (16-byte chunks, XOR-swizzled by row so that the operand reads of
 //    v_mfma_f32_32x32x16_bf16 do not collide); while one buffer is multiplied the next tile is written into
 //    the other and the one after that is on its way from memory.
@@ -175,23 +175,25 @@ __global__ __launch_bounds__(1024) void gemm_stream_kernel(MfmaGemmArgs g) {
 }
 
 // ------------------------------------------------------------------------------------------ many rows
-// grid (row tiles of BM, ceil(N / 128)); block 256.  BM = 64: waves side by side along n, each 64 x 32;
-// BM = 128: waves 2 x 2, each 64 x 64.
+// grid (row tiles of BM, ceil(N / 128)); block of 8 waves laid WM x WN over the tile: BM = 128 as 4 x 2 (a wave
+// owns 32 x 64 outputs), BM = 64 as 2 x 4 (32 x 32).  Eight waves of small tiles beat four of large ones here:
+// the step is bound by the way through LDS, and twice the waves hide twice the latency.
 #define TBN 128
 #define TBK 64
 
 // Where 16-byte chunk `chunk` of row `row` lies in a tile: rows of 128 bytes, the chunk index XOR-ed with bits 1..3
 // of the row.  Measured with ds_read_b128 in the operand layout (lane l reads row l % 32): this runs at the full
 // 128 bytes per clock; XOR with bits 0..2 at 107, no swizzle at 31.
-template <int BM>
 __device__ __forceinline__ int swz(int row, int chunk) { return row * TBK + ((chunk ^ ((row >> 1) & 7)) << 3); }
 
-template <int BM, bool DUAL, bool OUT_ACT>
-__global__ __launch_bounds__(256) void gemm_tile_kernel(MfmaGemmArgs g) {
-  constexpr int NI = BM == 128 ? 2 : 1;          // 32-wide column tiles per wave
-  constexpr int MI = 2;                          // 32-high row tiles per wave
-  constexpr int A_CH = BM * 8 / 256;             // 16-byte chunks of the a tile per thread
-  constexpr int W_CH = TBN * 8 / 256;
+template <int BM, int WM, int WN, bool DUAL, bool OUT_ACT>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g) {
+  constexpr int NT = 64 * WM * WN;
+  constexpr int MI = BM / WM / 32;               // 32-high row tiles per wave
+  constexpr int NI = TBN / WN / 32;              // 32-wide column tiles per wave
+  constexpr int A_CH = BM * 8 / NT;              // 16-byte chunks of the a tile per thread
+  constexpr int W_CH = TBN * 8 / NT;
+  static_assert(MI >= 1 && NI >= 1 && A_CH >= 1 && W_CH >= 1 && BM * 8 % NT == 0 && TBN * 8 % NT == 0, "tile layout");
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   // two buffers, each a tile of `a`, one of `w` and (gated pair) one of `w2`
   constexpr int BUF = (BM + TBN * (DUAL ? 2 : 1)) * TBK;
@@ -219,33 +221,32 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(MfmaGemmArgs g) {
   const bf16_t* w2 = DUAL ? g.w2 + (size_t)group * g.group_stride : nullptr;
   const int m0 = tile_m * BM, n0 = tile_n * TBN;
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
-  const int wm = BM == 128 ? wave / 2 : 0, wn = BM == 128 ? wave % 2 : wave;
+  const int wm = wave / WN, wn = wave % WN;
 
-  // what this thread fetches of each tile: chunk `ch` of row `row`
+  // What this thread fetches of each tile: chunk `ch` of row `row`.  Rows past the end of `a` or `w`, and rows
+  // of padding in an expert's tile, read some valid row instead: an output depends on its own row of `a` and
+  // of `w` only, and those outputs are never stored.  So the loads need no predicate.
   const bf16_t* a_src[A_CH];
   int a_dst[A_CH], w_dst[W_CH];
   const bf16_t *w_src[W_CH], *v_src[W_CH];
 #pragma unroll
   for (int i = 0; i < A_CH; ++i) {
-    const int idx = tid + i * 256, row = idx / 8, ch = idx % 8;
-    const int m = m0 + row;
-    int src = -1;
-    if (m < g.M) {
-      src = g.a_rows ? g.a_rows[m] : m;
-      if (src >= 0 && !g.a_gather) src = m;
-    }
-    a_src[i] = src >= 0 ? g.a + (size_t)src * g.lda + ch * 8 : nullptr;
-    a_dst[i] = swz<BM>(row, ch);
+    const int idx = tid + i * NT, row = idx / 8, ch = idx % 8;
+    const int m = min(m0 + row, g.M - 1);
+    int src = m;
+    if (g.a_rows && g.a_gather) src = max(g.a_rows[m], 0);
+    a_src[i] = g.a + (size_t)src * g.lda + ch * 8;
+    a_dst[i] = swz(row, ch);
   }
 #pragma unroll
   for (int i = 0; i < W_CH; ++i) {
-    const int idx = tid + i * 256, row = idx / 8, ch = idx % 8;
-    const int n = n0 + row;
-    w_src[i] = n < g.N ? w + (size_t)n * g.K + ch * 8 : nullptr;
-    v_src[i] = DUAL && n < g.N ? w2 + (size_t)n * g.K + ch * 8 : nullptr;
-    w_dst[i] = swz<BM>(row, ch);
+    const int idx = tid + i * NT, row = idx / 8, ch = idx % 8;
+    const int n = min(n0 + row, g.N - 1);
+    w_src[i] = w + (size_t)n * g.K + ch * 8;
+    v_src[i] = DUAL ? w2 + (size_t)n * g.K + ch * 8 : nullptr;
+    w_dst[i] = swz(row, ch);
   }
-  const int ch_of_thread = tid % 8;     // (tid + i * 256) % 8
+  const int ch_of_thread = tid % 8;     // (tid + i * NT) % 8
 
   f32x16 acc[MI][NI], acc2[DUAL ? MI : 1][DUAL ? NI : 1];
 #pragma unroll
@@ -260,16 +261,26 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(MfmaGemmArgs g) {
 
   u32x4 pa[A_CH], pw[W_CH], pv[DUAL ? W_CH : 1];
   const u32x4 z = {0u, 0u, 0u, 0u};
-  // FETCH: the thread's chunks of the tile at k0 into registers.  STAGE: registers into LDS.  (Written as macros
-  // so that the small arrays above are only ever indexed by constants and stay in registers.)
+  // FETCH: the thread's chunks of the tile at k0 into registers; only the last tile of a K that is no multiple
+  // of 64 needs zeros past the end.  STAGE: registers into LDS.  (Written as macros so that the small arrays
+  // above are only ever indexed by constants and stay in registers.)
 #define TQ_FETCH(k0)                                                                                          \
   do {                                                                                                        \
-    const bool k_ok = (k0) + ch_of_thread * 8 < g.K;                                                          \
-    _Pragma("unroll") for (int i = 0; i < A_CH; ++i)                                                          \
-        pa[i] = a_src[i] && k_ok ? *reinterpret_cast<const u32x4*>(a_src[i] + (k0)) : z;                      \
-    _Pragma("unroll") for (int i = 0; i < W_CH; ++i) {                                                        \
-      pw[i] = w_src[i] && k_ok ? *reinterpret_cast<const u32x4*>(w_src[i] + (k0)) : z;                        \
-      if (DUAL) pv[i] = v_src[i] && k_ok ? *reinterpret_cast<const u32x4*>(v_src[i] + (k0)) : z;              \
+    if ((k0) + TBK <= g.K) {                                                                                  \
+      _Pragma("unroll") for (int i = 0; i < A_CH; ++i)                                                        \
+          pa[i] = *reinterpret_cast<const u32x4*>(a_src[i] + (k0));                                           \
+      _Pragma("unroll") for (int i = 0; i < W_CH; ++i) {                                                      \
+        pw[i] = *reinterpret_cast<const u32x4*>(w_src[i] + (k0));                                             \
+        if (DUAL) pv[i] = *reinterpret_cast<const u32x4*>(v_src[i] + (k0));                                   \
+      }                                                                                                       \
+    } else {                                                                                                  \
+      const bool k_ok = (k0) + ch_of_thread * 8 < g.K;                                                        \
+      _Pragma("unroll") for (int i = 0; i < A_CH; ++i)                                                        \
+          pa[i] = k_ok ? *reinterpret_cast<const u32x4*>(a_src[i] + (k0)) : z;                                \
+      _Pragma("unroll") for (int i = 0; i < W_CH; ++i) {                                                      \
+        pw[i] = k_ok ? *reinterpret_cast<const u32x4*>(w_src[i] + (k0)) : z;                                  \
+        if (DUAL) pv[i] = k_ok ? *reinterpret_cast<const u32x4*>(v_src[i] + (k0)) : z;                        \
+      }                                                                                                       \
     }                                                                                                         \
   } while (0)
 #define TQ_STAGE(off)                                                                                         \
@@ -302,14 +313,14 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(MfmaGemmArgs g) {
       bf16x8 af[MI], wf[NI], vf[DUAL ? NI : 1];
 #pragma unroll
       for (int mi = 0; mi < MI; ++mi) {
-        const int row = wm * 64 + mi * 32 + lr;
-        af[mi] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(Ac + swz<BM>(row, 2 * j + lc)));
+        const int row = wm * (MI * 32) + mi * 32 + lr;
+        af[mi] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(Ac + swz(row, 2 * j + lc)));
       }
 #pragma unroll
       for (int ni = 0; ni < NI; ++ni) {
         const int row = wn * (NI * 32) + ni * 32 + lr;
-        wf[ni] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(Wc + swz<BM>(row, 2 * j + lc)));
-        if (DUAL) vf[ni] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(Vc + swz<BM>(row, 2 * j + lc)));
+        wf[ni] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(Wc + swz(row, 2 * j + lc)));
+        if (DUAL) vf[ni] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(Vc + swz(row, 2 * j + lc)));
       }
 #pragma unroll
       for (int mi = 0; mi < MI; ++mi)
@@ -333,7 +344,7 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(MfmaGemmArgs g) {
     for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int m = m0 + wm * 64 + mi * 32 + 8 * (v / 4) + 4 * lc + (v % 4);
+        const int m = m0 + wm * (MI * 32) + mi * 32 + 8 * (v / 4) + 4 * lc + (v % 4);
         if (m >= g.M) continue;
         if (g.a_rows && g.a_rows[m] < 0) continue;
         float o = acc[mi][ni][v] + b;
@@ -372,16 +383,16 @@ static int launch_stream(const MfmaGemmArgs& g, bool dual, bool out_act, int row
   return 0;
 }
 
-template <int BM>
+template <int BM, int WM, int WN>
 static int launch_tile(const MfmaGemmArgs& g, bool dual, bool out_act, hipStream_t st) {
   const dim3 grid((g.M + BM - 1) / BM, (g.N + TBN - 1) / TBN);
   const size_t shmem = (size_t)2 * (BM + TBN * (dual ? 2 : 1)) * TBK * sizeof(bf16_t);
-#define TQ_TILE(D, O)                                                                                          \
-  do {                                                                                                         \
-    if (shmem > 48 * 1024)                                                                                     \
-      hipFuncSetAttribute((const void*)gemm_tile_kernel<BM, D, O>, hipFuncAttributeMaxDynamicSharedMemorySize, \
-                          (int)shmem);                                                                         \
-    hipLaunchKernelGGL((gemm_tile_kernel<BM, D, O>), grid, dim3(256), shmem, st, g);                           \
+#define TQ_TILE(D, O)                                                                                  \
+  do {                                                                                                 \
+    if (shmem > 48 * 1024)                                                                             \
+      hipFuncSetAttribute((const void*)gemm_tile_kernel<BM, WM, WN, D, O>,                             \
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);                     \
+    hipLaunchKernelGGL((gemm_tile_kernel<BM, WM, WN, D, O>), grid, dim3(64 * WM * WN), shmem, st, g);  \
   } while (0)
   if (dual && out_act)
     TQ_TILE(true, true);
@@ -414,7 +425,7 @@ TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gat
       rc = launch_stream<1>(g, dual, out_act, M / 16, st);
     } else if (tile_rows == 64) {
       if ((N + TBN - 1) / TBN > 65535) return TQ_ERR_UNSUPPORTED;
-      rc = launch_tile<64>(g, dual, out_act, st);
+      rc = launch_tile<64, 2, 4>(g, dual, out_act, st);
     } else {
       return TQ_ERR_BAD_ARG;
     }
@@ -426,7 +437,7 @@ TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gat
     rc = launch_stream<4>(g, dual, out_act, 1, st);
   } else {
     if ((N + TBN - 1) / TBN > 65535) return TQ_ERR_UNSUPPORTED;
-    rc = M <= 64 * 16 && !dual ? launch_tile<64>(g, dual, out_act, st) : launch_tile<128>(g, dual, out_act, st);
+    rc = M <= 64 * 16 && !dual ? launch_tile<64, 2, 4>(g, dual, out_act, st) : launch_tile<128, 4, 2>(g, dual, out_act, st);
   }
   if (rc) return rc;
   TQ_LAUNCH_CHECK();
