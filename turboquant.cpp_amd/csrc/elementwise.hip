@@ -83,43 +83,58 @@ TQ_API int tq_add_rmsnorm(float* x, const float* delta, int S, int64_t delta_str
 // sequence: page = block_table[seq][pos / page_size], row pos % page_size of kv head h.  After the
 // layer's own offset (already added to k_pool / v_pool) keys lie [page][kv head][row][hd] and values
 // transposed, [page][kv head][hd][row].
-__global__ void rope_kv_write_kernel(const float* __restrict__ qkv, const int* __restrict__ positions,
+// A workgroup of four waves takes `spb` heads of one token (grid (T, ceil(heads / spb))); a wave takes every
+// fourth of them and turns pair i of all its heads with one sine and cosine.
+__global__ __launch_bounds__(256) void rope_kv_write_kernel(const float* __restrict__ qkv, const int* __restrict__ positions,
                                      const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
                                      int bt_stride, const float* __restrict__ inv_freq, int pairing, int rot,
                                      act_t* __restrict__ q_out, act_t* __restrict__ k_pool,
                                      act_t* __restrict__ v_pool, int page_size, int64_t page_stride, int nh,
-                                     int nkv, int hd, int write_kv) {
+                                     int nkv, int hd, int write_kv, int spb) {
   const int t = blockIdx.x;
-  const int slot = blockIdx.y;          // 0..nh-1 query heads, then key heads, then value heads
+  const int wave = threadIdx.x / TQ_WAVE, lane = threadIdx.x % TQ_WAVE;
+  const int heads = nh + 2 * nkv;       // 0..nh-1 query heads, then key heads, then value heads
+  const int s0 = blockIdx.y * spb + wave, s1 = min(blockIdx.y * spb + spb, heads);
+  if (s0 >= s1) return;
   const int pos = positions[t];
-  const float* src = qkv + ((size_t)t * (nh + 2 * nkv) + slot) * hd;
-  act_t* dst;
-  if (slot < nh) {
-    dst = q_out + ((size_t)t * nh + slot) * hd;
-  } else {
-    if (!write_kv) return;
-    const int kvh = (slot - nh) % nkv;
-    const bool is_v = slot >= nh + nkv;
+  const float* src_t = qkv + (size_t)t * heads * hd;
+  act_t* q_t = q_out + (size_t)t * nh * hd;
+  act_t *k_t = nullptr, *v_t = nullptr;      // the token's row of kv head 0 in its page
+  if (write_kv && s1 > nh) {
     const int page = block_table[(size_t)seq_of_token[t] * bt_stride + pos / page_size];
-    if (is_v) {   // values lie transposed, [hd][row], so that a dimension's values over positions are contiguous
-      act_t* col = v_pool + (size_t)page * page_stride + (size_t)kvh * page_size * hd + pos % page_size;
-      for (int i = threadIdx.x; i < hd; i += blockDim.x) col[(size_t)i * page_size] = from_f32<act_t>(src[i]);
-      return;
-    }
-    dst = k_pool + (size_t)page * page_stride + ((size_t)kvh * page_size + pos % page_size) * hd;
+    const int row = pos % page_size;
+    k_t = k_pool + (size_t)page * page_stride + (size_t)row * hd;
+    v_t = v_pool + (size_t)page * page_stride + row;
   }
+  const int rot_end = write_kv ? min(s1, nh + nkv) : min(s1, nh);     // heads below this are rotated
+  const size_t kv_head_stride = (size_t)page_size * hd;
   const int half = rot / 2;
-  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+  for (int i = lane; i < half; i += TQ_WAVE) {
     const float theta = (float)pos * inv_freq[i];
     float sn, cs;
     sincosf(theta, &sn, &cs);
     const int ia = pairing == 0 ? i : 2 * i;
     const int ib = pairing == 0 ? i + half : 2 * i + 1;
-    const float a = src[ia], b = src[ib];
-    dst[ia] = from_f32<act_t>(a * cs - b * sn);
-    dst[ib] = from_f32<act_t>(a * sn + b * cs);
+    for (int s = s0; s < rot_end; s += 4) {
+      const float* src = src_t + (size_t)s * hd;
+      act_t* dst = s < nh ? q_t + (size_t)s * hd : k_t + (size_t)(s - nh) * kv_head_stride;
+      const float a = src[ia], b = src[ib];
+      dst[ia] = from_f32<act_t>(a * cs - b * sn);
+      dst[ib] = from_f32<act_t>(a * sn + b * cs);
+    }
   }
-  for (int i = rot + threadIdx.x; i < hd; i += blockDim.x) dst[i] = from_f32<act_t>(src[i]);
+  for (int s = s0; s < rot_end; s += 4) {      // dimensions from rot on pass through
+    const float* src = src_t + (size_t)s * hd;
+    act_t* dst = s < nh ? q_t + (size_t)s * hd : k_t + (size_t)(s - nh) * kv_head_stride;
+    for (int i = rot + lane; i < hd; i += TQ_WAVE) dst[i] = from_f32<act_t>(src[i]);
+  }
+  if (!write_kv) return;
+  for (int s = s0; s < s1; s += 4) {           // values lie transposed, [hd][row]
+    if (s < nh + nkv) continue;
+    const float* src = src_t + (size_t)s * hd;
+    act_t* col = v_t + (size_t)(s - nh - nkv) * kv_head_stride;
+    for (int i = lane; i < hd; i += TQ_WAVE) col[(size_t)i * page_size] = from_f32<act_t>(src[i]);
+  }
 }
 
 TQ_API int tq_rope_kv_write(const float* qkv, const int* positions, const int* seq_of_token,
@@ -128,9 +143,14 @@ TQ_API int tq_rope_kv_write(const float* qkv, const int* positions, const int* s
                             int nh, int nkv, int hd, int write_kv, hipStream_t st) {
   if (T <= 0) return 0;
   if (rot < 0 || rot > hd || (rot & 1) || (pairing != 0 && pairing != 1)) return TQ_ERR_BAD_ARG;
-  hipLaunchKernelGGL(rope_kv_write_kernel, dim3(T, nh + 2 * nkv), dim3(64), 0, st, qkv, positions, seq_of_token,
-                     block_table, bt_stride, inv_freq, pairing, rot, (act_t*)q_out, (act_t*)k_pool, (act_t*)v_pool,
-                     page_size, page_stride, nh, nkv, hd, write_kv);
+  const int heads = nh + 2 * nkv;
+  // few tokens: a head per wave, so that the chip sees many small workgroups; many: all heads of a token in one
+  int spb = 4;
+  while (spb < heads && (int64_t)T * ((heads + spb - 1) / spb) > 4096) spb *= 2;
+  if ((heads + spb - 1) / spb > 65535) return TQ_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(rope_kv_write_kernel, dim3(T, (heads + spb - 1) / spb), dim3(256), 0, st, qkv, positions,
+                     seq_of_token, block_table, bt_stride, inv_freq, pairing, rot, (act_t*)q_out, (act_t*)k_pool,
+                     (act_t*)v_pool, page_size, page_stride, nh, nkv, hd, write_kv, spb);
   TQ_LAUNCH_CHECK();
   return 0;
 }

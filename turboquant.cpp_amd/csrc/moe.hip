@@ -5,9 +5,9 @@
 // ---------------------------------------------------------------- router
 // Two kernels.  router_logits: logit[t][e] = sum_j x[t][j] * wr[e][j] in float
 // (/root/reference/src/engine/tq_moe.c:611-618), with the shared expert's gate vector as one more row.  A
-// wave takes one row of wr at a time for a group of up to 8 tokens whose activations wait in LDS; lane l sums
-// the elements j = 8 * (64 i + l) .. + 7 for i = 0, 1, ... and the lanes' sums are added by a butterfly: one
-// order for every token, whatever else is in the batch.  Rows are dealt over a second grid dimension when
+// wave takes one row of wr (or a few) at a time for a group of up to 8 tokens whose activations wait in LDS; lane l sums
+// a fixed share of the elements and the lanes' sums are added by a butterfly: one order for every token,
+// whatever else is in the batch.  Rows are dealt over a second grid dimension when
 // there are few tokens, so that decoding does not leave the chip to eight waves.
 // router_select, one wave per token: top-k by logit, k rounds of a search in which >= lets the highest index
 // win among equal logits, so ids come out by descending logit (tq_moe.c:626-645).  Weights:
@@ -15,90 +15,115 @@
 //   renorm == 0: softmax over all experts, the selected probabilities kept as they are.
 // shared_gate[t] = 1 / (1 + exp(-(x . shared_w)))  (tq_moe.c:1012-1018, with an exact exponential).
 #define RT 8   // most tokens per workgroup of router_logits
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ void load8(const float* p, float (&w)[8]) {
-  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
-  w[0] = a.x; w[1] = a.y; w[2] = a.z; w[3] = a.w; w[4] = b.x; w[5] = b.y; w[6] = b.z; w[7] = b.w;
+__device__ __forceinline__ void load4(const float* p, float* w) {
+  const f32x4 a = *reinterpret_cast<const f32x4*>(p);
+  w[0] = a.x; w[1] = a.y; w[2] = a.z; w[3] = a.w;
 }
-__device__ __forceinline__ void load8(const bf16_t* p, float (&w)[8]) {
-  const uint4 v = *reinterpret_cast<const uint4*>(p);
-  const uint32_t u[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    w[2 * i] = __uint_as_float(u[i] << 16);
-    w[2 * i + 1] = __uint_as_float(u[i] & 0xffff0000u);
-  }
-}
-
-template <int TG>
-__device__ __forceinline__ void router_chunk(const float* xs, int H, int j, const float (&w)[8], float (&s)[TG]) {
-#pragma unroll
-  for (int r = 0; r < TG; ++r) {
-    const float4 a = *reinterpret_cast<const float4*>(xs + r * H + j);
-    const float4 b = *reinterpret_cast<const float4*>(xs + r * H + j + 4);
-    s[r] = fmaf(a.x, w[0], s[r]);
-    s[r] = fmaf(a.y, w[1], s[r]);
-    s[r] = fmaf(a.z, w[2], s[r]);
-    s[r] = fmaf(a.w, w[3], s[r]);
-    s[r] = fmaf(b.x, w[4], s[r]);
-    s[r] = fmaf(b.y, w[5], s[r]);
-    s[r] = fmaf(b.z, w[6], s[r]);
-    s[r] = fmaf(b.w, w[7], s[r]);
-  }
+__device__ __forceinline__ void load4(const bf16_t* p, float* w) {
+  const uint2 v = *reinterpret_cast<const uint2*>(p);
+  w[0] = __uint_as_float(v.x << 16);
+  w[1] = __uint_as_float(v.x & 0xffff0000u);
+  w[2] = __uint_as_float(v.y << 16);
+  w[3] = __uint_as_float(v.y & 0xffff0000u);
 }
 
-// TG: tokens per workgroup (tokens beyond T are zeros in LDS and are not stored).
-template <class W, int TG>
+// TG: tokens per workgroup (tokens beyond T are zeros in LDS and are not stored).  RW: rows of wr that a wave
+// takes at a time, so that one read of the activations from LDS serves RW rows.  Neither changes the order in
+// which a logit is summed: of every 512 elements lane l sums 4 l .. 4 l + 3 and 256 + 4 l .. 256 + 4 l + 3 (its
+// 16-byte reads from LDS then lie side by side with its neighbours'), block after block.  In LDS a token's row is
+// filled with zeros up to a multiple of 512, so the last block needs no predicate: there the weights are read
+// from the row's last elements instead, and multiplied by zeros.
+template <class W, int TG, int RW>
 __global__ __launch_bounds__(256) void router_logits_kernel(const float* __restrict__ x, const W* __restrict__ wr,
                                                             const W* __restrict__ shared_w, int rows, int E,
                                                             float* __restrict__ logits, int T, int H) {
-  extern __shared__ float xs[];      // [TG][H]
+  extern __shared__ __attribute__((aligned(16))) float xs[];      // [TG][Hp]
+  const int Hp = (H + 511) / 512 * 512;
   const int t0 = blockIdx.x * TG;
   const int nt = min(TG, T - t0);
   const int wave = threadIdx.x / TQ_WAVE, lane = threadIdx.x % TQ_WAVE;
-  const bool vec = H % 8 == 0;
+  const bool vec = H % 4 == 0;
   if (vec) {
-    const float4* src = reinterpret_cast<const float4*>(x + (size_t)t0 * H);
-    float4* dst = reinterpret_cast<float4*>(xs);
-    for (int i = threadIdx.x; i < TG * H / 4; i += blockDim.x) dst[i] = i < nt * H / 4 ? src[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+    const int Hp4 = Hp / 4, H4 = H / 4;
+    f32x4* dst = reinterpret_cast<f32x4*>(xs);
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+    for (int i = threadIdx.x; i < TG * Hp4; i += blockDim.x) {
+      const int k = i / Hp4, j = i % Hp4;
+      dst[i] = k < nt && j < H4 ? reinterpret_cast<const f32x4*>(x + (size_t)(t0 + k) * H)[j] : zero;
+    }
   } else {
-    for (int i = threadIdx.x; i < TG * H; i += blockDim.x) xs[i] = i < nt * H ? x[(size_t)t0 * H + i] : 0.f;
+    for (int i = threadIdx.x; i < TG * Hp; i += blockDim.x) {
+      const int k = i / Hp, j = i % Hp;
+      xs[i] = k < nt && j < H ? x[(size_t)(t0 + k) * H + j] : 0.f;
+    }
   }
   __syncthreads();
   // workgroups start at different rows, so that they do not all ask for the same row at once
   const int rot = (blockIdx.x * 5) % rows;
-  const int h_quad = H / (TQ_WAVE * 8 * 4) * (TQ_WAVE * 8 * 4);     // the part of a row that goes four chunks at a time
-  for (int idx = blockIdx.y * 4 + wave; idx < rows; idx += gridDim.y * 4) {
-    const int e = idx + rot < rows ? idx + rot : idx + rot - rows;
-    const W* row = e < E ? wr + (size_t)e * H : shared_w;
-    float s[TG];
+  for (int idx = (blockIdx.y * 4 + wave) * RW; idx < rows; idx += gridDim.y * 4 * RW) {
+    const W* row[RW];
+    int e[RW];
 #pragma unroll
-    for (int r = 0; r < TG; ++r) s[r] = 0.f;
+    for (int r = 0; r < RW; ++r) {
+      const int i = min(idx + r, rows - 1) + rot;
+      e[r] = i < rows ? i : i - rows;
+      row[r] = e[r] < E ? wr + (size_t)e[r] * H : shared_w;
+    }
+    float s[RW][TG];
+#pragma unroll
+    for (int r = 0; r < RW; ++r)
+#pragma unroll
+      for (int k = 0; k < TG; ++k) s[r][k] = 0.f;
     if (vec) {
-      for (int j0 = lane * 8; j0 < h_quad; j0 += TQ_WAVE * 8 * 4) {   // four chunks asked for before the first is used
-        float w[4][8];
+      const f32x4* xv = reinterpret_cast<const f32x4*>(xs);
+      const int Hp4 = Hp / 4;
+#pragma unroll(RW >= 4 ? 2 : 4)
+      for (int b = 0; b < Hp; b += 512) {
+        const int g0 = min(b + 4 * lane, H - 4), g1 = min(b + 256 + 4 * lane, H - 4);
+        float w[RW][8];
 #pragma unroll
-        for (int c = 0; c < 4; ++c) load8(row + j0 + c * TQ_WAVE * 8, w[c]);
+        for (int r = 0; r < RW; ++r) {
+          load4(row[r] + g0, &w[r][0]);
+          load4(row[r] + g1, &w[r][4]);
+        }
 #pragma unroll
-        for (int c = 0; c < 4; ++c) router_chunk<TG>(xs, H, j0 + c * TQ_WAVE * 8, w[c], s);
-      }
-      for (int j = h_quad + lane * 8; j < H; j += TQ_WAVE * 8) {
-        float w[8];
-        load8(row + j, w);
-        router_chunk<TG>(xs, H, j, w, s);
+        for (int k = 0; k < TG; ++k) {
+          const f32x4 a = xv[k * Hp4 + b / 4 + lane];
+          const f32x4 c = xv[k * Hp4 + b / 4 + 64 + lane];
+#pragma unroll
+          for (int r = 0; r < RW; ++r) {
+            float v = s[r][k];
+            v = fmaf(a.x, w[r][0], v);
+            v = fmaf(a.y, w[r][1], v);
+            v = fmaf(a.z, w[r][2], v);
+            v = fmaf(a.w, w[r][3], v);
+            v = fmaf(c.x, w[r][4], v);
+            v = fmaf(c.y, w[r][5], v);
+            v = fmaf(c.z, w[r][6], v);
+            v = fmaf(c.w, w[r][7], v);
+            s[r][k] = v;
+          }
+        }
       }
     } else {
       for (int j = lane; j < H; j += TQ_WAVE) {
-        const float w = to_f32(row[j]);
 #pragma unroll
-        for (int r = 0; r < TG; ++r) s[r] = fmaf(xs[r * H + j], w, s[r]);
+        for (int r = 0; r < RW; ++r) {
+          const float w = to_f32(row[r][j]);
+#pragma unroll
+          for (int k = 0; k < TG; ++k) s[r][k] = fmaf(xs[k * Hp + j], w, s[r][k]);
+        }
       }
     }
 #pragma unroll
-    for (int r = 0; r < TG; ++r) {
-      const float v = wave_sum(s[r]);
-      if (lane == 0 && r < nt) logits[(size_t)(t0 + r) * rows + e] = v;
-    }
+    for (int r = 0; r < RW; ++r)
+#pragma unroll
+      for (int k = 0; k < TG; ++k) {
+        const float v = wave_sum(s[r][k]);
+        if (lane == 0 && k < nt && idx + r < rows) logits[(size_t)(t0 + k) * rows + e[r]] = v;
+      }
   }
 }
 
@@ -169,28 +194,39 @@ TQ_API int tq_router_topk(const float* x, const void* wr, const void* shared_w, 
   if (T <= 0) return 0;
   if (topk < 1 || topk > 64 || topk > E || E > 8192) return TQ_ERR_UNSUPPORTED;
   int tg = RT;
-  while (tg > 1 && (size_t)tg * H * sizeof(float) > 32 * 1024) tg /= 2;   // small enough for several workgroups per CU
-  const size_t shmem = (size_t)tg * H * sizeof(float);
+  const size_t hp = ((size_t)H + 511) / 512 * 512;      // a token's row in LDS
+  while (tg > 1 && (size_t)tg * hp * sizeof(float) > 32 * 1024) tg /= 2;   // small enough for several workgroups per CU
+  const size_t shmem = (size_t)tg * hp * sizeof(float);
   if (shmem > 160 * 1024) return TQ_ERR_UNSUPPORTED;
   const int rows = E + (shared_w ? 1 : 0);
   const int groups = (T + tg - 1) / tg;
-  // with few groups of tokens the rows are dealt over more workgroups
-  int row_groups = 256 / groups;
+  // The rows are dealt over so many workgroups that the chip holds about 2048 of them: what a wave does is a
+  // chain of loads, and only many waves hide it.  A wave takes 1, 2 or 4 rows at a time.
+  int row_groups = 2048 / groups;
   row_groups = row_groups < 1 ? 1 : (row_groups > (rows + 3) / 4 ? (rows + 3) / 4 : row_groups);
-#define TQ_ROUTER(TGV)                                                                                              \
+  const int rows_per_wave = (rows + row_groups * 4 - 1) / (row_groups * 4);
+  const int rw = rows_per_wave >= 4 ? 4 : (rows_per_wave >= 2 ? 2 : 1);
+#define TQ_ROUTER(TGV, RWV)                                                                                         \
   do {                                                                                                              \
     if (shmem > 48 * 1024)                                                                                          \
-      hipFuncSetAttribute((const void*)router_logits_kernel<W, TGV>, hipFuncAttributeMaxDynamicSharedMemorySize,    \
-                          (int)shmem);                                                                              \
-    hipLaunchKernelGGL((router_logits_kernel<W, TGV>), dim3(groups, row_groups), dim3(256), shmem, st, x,           \
+      hipFuncSetAttribute((const void*)router_logits_kernel<W, TGV, RWV>,                                           \
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);                                  \
+    hipLaunchKernelGGL((router_logits_kernel<W, TGV, RWV>), dim3(groups, row_groups), dim3(256), shmem, st, x,      \
                        (const W*)wr, (const W*)shared_w, rows, E, logits, T, H);                                    \
   } while (0)
+#define TQ_ROUTER_RW(TGV)          \
+  do {                             \
+    if (rw == 4) TQ_ROUTER(TGV, 4); \
+    else if (rw == 2) TQ_ROUTER(TGV, 2); \
+    else TQ_ROUTER(TGV, 1);        \
+  } while (0)
   TQ_DISPATCH_W(wtype, {
-    if (tg == 8) TQ_ROUTER(8);
-    else if (tg == 4) TQ_ROUTER(4);
-    else if (tg == 2) TQ_ROUTER(2);
-    else TQ_ROUTER(1);
+    if (tg == 8) TQ_ROUTER_RW(8);
+    else if (tg == 4) TQ_ROUTER_RW(4);
+    else if (tg == 2) TQ_ROUTER_RW(2);
+    else TQ_ROUTER_RW(1);
   });
+#undef TQ_ROUTER_RW
 #undef TQ_ROUTER
   TQ_LAUNCH_CHECK();
   hipLaunchKernelGGL(router_select_kernel, dim3((T + 3) / 4), dim3(256), (size_t)4 * E * sizeof(float), st, logits,
@@ -208,8 +244,8 @@ TQ_API int tq_router_topk(const float* x, const void* wr, const void* shared_w, 
 //   pair_slot[i]     row of pair i
 //   tile_expert[j]   expert of row tile j (tiles of `unit` rows), n_tiles[0] tiles in all
 // One workgroup of 16 waves does all of it.  Wave w owns the w-th sixteenth of the pairs: it goes through
-// them 64 at a time, and for every expert present among the 64 (found leader by leader with ballots) gives
-// the lanes of that expert their rank in order of lane and adds their number to its count of the expert.
+// them 64 at a time, finds for every lane the lanes that hold the same expert (a ballot per bit of the expert's
+// number), gives it its rank among them in order of lane and adds their number to its count of the expert.
 // After a barrier the counts of all waves give every expert's first row and every wave's first row within
 // the expert, and each pair's row is that plus its rank.
 #define AW 16   // waves
@@ -233,19 +269,18 @@ __global__ __launch_bounds__(64 * AW) void moe_align_kernel(const int* __restric
     const int i = b + lane;
     const bool valid = i < seg_end;
     const int e = valid ? ids[i] : -1;
-    int rank = 0;
-    unsigned long long rest = __ballot(valid);
-    while (rest) {
-      const int leader = __ffsll((long long)rest) - 1;
-      const int e0 = __shfl(e, leader, TQ_WAVE);
-      const unsigned long long m = __ballot(valid && e == e0);
-      const int base = mine[e0];
-      if (e == e0 && valid) rank = base + __popcll(m & ((1ull << lane) - 1ull));
-      __builtin_amdgcn_wave_barrier();
-      if (lane == leader) mine[e0] = base + __popcll(m);
-      __builtin_amdgcn_wave_barrier();
-      rest &= ~m;
+    // the lanes that hold the same expert: one ballot per bit of the expert's number
+    unsigned long long same = __ballot(valid);
+    for (int bit = 0; (1 << bit) < E; ++bit) {
+      const unsigned long long set = __ballot(valid && ((e >> bit) & 1));
+      same &= ((e >> bit) & 1) ? set : ~set;
     }
+    const unsigned long long lower = same & ((1ull << lane) - 1ull);
+    const int base = mine[valid ? e : 0];
+    const int rank = base + __popcll(lower);
+    __builtin_amdgcn_wave_barrier();       // every lane has read its count before the expert's first lane adds to it
+    if (valid && lower == 0) mine[e] = base + __popcll(same);
+    __builtin_amdgcn_wave_barrier();
     if (valid) pair_slot[i] = rank;      // rank within (wave, expert) for now
   }
   __syncthreads();
