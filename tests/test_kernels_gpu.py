@@ -424,7 +424,9 @@ def test_sample_topp_distribution(ops):
 # ------------------------------------------------------------------------------------------------ tiled attention
 @pytest.mark.parametrize("nh,nkv,hd,window,page", [(4, 4, 16, None, 64), (6, 2, 48, 24, 64), (3, 1, 80, 70, 128),
                                                      (16, 16, 128, None, 64), (40, 2, 32, 200, 64), (2, 1, 256, None, 64),
-                                                     (5, 5, 96, 1, 64)])
+                                                     (5, 5, 96, 1, 64), (8, 2, 64, 100, 64),
+                                                     # enough heads for two token groups per wave
+                                                     (48, 6, 128, None, 64), (48, 4, 64, 100, 64), (44, 4, 48, 30, 64)])
 def test_attention_tiled(ops, nh, nkv, hd, window, page):
     """The matrix-core kernels (whole runs of tokens, and one token per sequence split over the cache) against the
     plain attention: unequal lengths, a sequence that goes on from a cached prefix, groups of more than 16 heads."""

@@ -26,6 +26,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define TILE 64
+#define LOG2E 1.4426950408889634f
 #define SPLIT 4          // tiles per run when decoding: 256 positions
 
 struct AttnArgs {
@@ -54,8 +55,10 @@ __device__ __forceinline__ bf16x8 zero16() {
   const uint4 v = make_uint4(0, 0, 0, 0);
   return __builtin_bit_cast(bf16x8, v);
 }
-__device__ __forceinline__ uint32_t pack2(float a, float b) {
-  return (uint32_t)f32_to_bf16(a).bits | ((uint32_t)f32_to_bf16(b).bits << 16);
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack2(float a, float b) {      // round to nearest even, one instruction for the pair
+  const bf16x2 v = {(__bf16)a, (__bf16)b};
+  return __builtin_bit_cast(uint32_t, v);
 }
 __device__ __forceinline__ float group_max(float v) {     // over the four lanes that share l % 16
   v = fmaxf(v, __shfl_xor(v, 16, 64));
@@ -72,16 +75,20 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 // One tile of 64 positions for QG groups of 16 columns that share the tile's keys and values.  kt: the tile's
 // keys, row i at kt + i * k_stride; vt: the tile's values transposed, dimension d at vt + d * v_stride (memory or
 // LDS).  DT: number of 16-wide blocks of hd held in registers (hd <= 16 * DT).  p_q: position of this lane's
-// column in each group (-1: no such column), lo_q: first position it may see.  qf: the columns' queries, 8
-// values of hd per 32-wide step at 8 * (l / 16).  Every operand read from kt and vt serves all QG groups.
-template <int DT, int QG>
+// column in each group (-1: no such column), lo_q: first position it may see; masked: whether any column of the
+// wave has a key in this tile that it may not see (if not, the comparisons are left out).  qf: the columns'
+// queries, 8 values of hd per 32-wide step at 8 * (l / 16).  Every operand read from kt and vt serves all QG
+// groups.  EXACT: hd is exactly 16 DT and DT is even.  scale2 = scale * log2(e) > 0: maxima are kept in that unit and probabilities are 2^(s * scale2 - m),
+// which is exp(s * scale - max) with one instruction for the power.
+template <int DT, int QG, bool EXACT>
 __device__ __forceinline__ void tile_step(f32x4 (&o)[QG][DT], float (&m_run)[QG], float (&l_run)[QG],
                                           const bf16x8 (&qf)[QG][(DT + 1) / 2], const bf16_t* kt, int k_stride,
                                           const bf16_t* vt, int v_stride, int hd, int pos0, const int (&p_q)[QG],
-                                          const int (&lo_q)[QG], float scale) {
+                                          const int (&lo_q)[QG], float scale2, bool masked) {
   constexpr int KS = (DT + 1) / 2;
   const int lane = threadIdx.x % 64, r = lane % 16, c = lane / 16;
-  const int n_dt = hd / 16, n_ks = (hd + 31) / 32;
+  // EXACT: hd == 16 DT with DT even, so nothing below depends on hd and every product is unconditional
+  const int n_dt = EXACT ? DT : hd / 16, n_ks = EXACT ? KS : (hd + 31) / 32;
   f32x4 s[QG][4];
 #pragma unroll
   for (int jt = 0; jt < 4; ++jt) {
@@ -91,7 +98,7 @@ __device__ __forceinline__ void tile_step(f32x4 (&o)[QG][DT], float (&m_run)[QG]
     for (int ks = 0; ks < KS; ++ks) {
       if (ks < n_ks) {
         const int d0 = 32 * ks + 8 * c;
-        const bf16x8 kf = d0 < hd ? ld16(kt + (32 * (jt / 2) + 8 * (r / 4) + 4 * (jt % 2) + r % 4) * k_stride + d0) : zero16();
+        const bf16x8 kf = EXACT || d0 < hd ? ld16(kt + (32 * (jt / 2) + 8 * (r / 4) + 4 * (jt % 2) + r % 4) * k_stride + d0) : zero16();
 #pragma unroll
         for (int g = 0; g < QG; ++g) s[g][jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[g][ks], s[g][jt], 0, 0, 0);
       }
@@ -101,25 +108,33 @@ __device__ __forceinline__ void tile_step(f32x4 (&o)[QG][DT], float (&m_run)[QG]
 #pragma unroll
   for (int g = 0; g < QG; ++g) {
     float m_tile = -INFINITY;
+    if (masked) {
 #pragma unroll
-    for (int jt = 0; jt < 4; ++jt)
+      for (int jt = 0; jt < 4; ++jt)
 #pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        const int key = pos0 + 32 * (jt / 2) + 8 * c + 4 * (jt % 2) + v;
-        const bool ok = key <= p_q[g] && key >= lo_q[g];
-        s[g][jt][v] = ok ? s[g][jt][v] * scale : -INFINITY;
-        m_tile = fmaxf(m_tile, s[g][jt][v]);
-      }
-    m_tile = group_max(m_tile);
+        for (int v = 0; v < 4; ++v) {
+          const int key = pos0 + 32 * (jt / 2) + 8 * c + 4 * (jt % 2) + v;
+          const bool ok = key <= p_q[g] && key >= lo_q[g];
+          s[g][jt][v] = ok ? s[g][jt][v] : -INFINITY;
+          m_tile = fmaxf(m_tile, s[g][jt][v]);
+        }
+    } else {
+#pragma unroll
+      for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) m_tile = fmaxf(m_tile, s[g][jt][v]);
+    }
+    m_tile = group_max(m_tile) * scale2;
     const float m_new = fmaxf(m_run[g], m_tile);
     const bool any = m_new != -INFINITY;
-    const float alpha = any && m_run[g] != -INFINITY ? expf(m_run[g] - m_new) : (any ? 0.f : 1.f);
+    const float alpha = any && m_run[g] != -INFINITY ? __builtin_amdgcn_exp2f(m_run[g] - m_new) : (any ? 0.f : 1.f);
+    const float m_use = any ? m_new : 0.f;       // 2^(-inf - 0) = 0 for masked keys, also when all are masked
     float l_tile = 0.f;
 #pragma unroll
     for (int jt = 0; jt < 4; ++jt)
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
-        const float p = any ? expf(s[g][jt][v] - m_new) : 0.f;      // exp(-inf) = 0 for masked keys
+        const float p = __builtin_amdgcn_exp2f(fmaf(s[g][jt][v], scale2, -m_use));
         s[g][jt][v] = p;
         l_tile += p;
       }
@@ -152,19 +167,20 @@ __device__ __forceinline__ void tile_step(f32x4 (&o)[QG][DT], float (&m_run)[QG]
 }
 
 // Runs the wave's 16 columns over tiles [tile_beg, tile_end) straight from the cache pages.
-template <int DT>
+template <int DT, bool EXACT>
 __device__ __forceinline__ void attend(f32x4 (&o)[1][DT], float (&m_run)[1], float (&l_run)[1],
                                        const bf16x8 (&qf)[1][(DT + 1) / 2], const bf16_t* kh, const bf16_t* vh,
                                        const int* table, int page_size, int64_t page_stride, int hd, int tile_beg,
-                                       int tile_end, int p_q, int lo_q, float scale) {
-  const int pq[1] = {p_q}, lq[1] = {lo_q};
+                                       int tile_end, int p, bool valid, int lo_q, float scale2) {
+  const int pq[1] = {valid ? p : -1}, lq[1] = {lo_q};
   for (int tile = tile_beg; tile < tile_end; ++tile) {
     const int pos0 = tile * TILE;
     const int page = table[pos0 / page_size];
     const int in_page = pos0 % page_size;
     const bf16_t* kt = kh + (int64_t)page * page_stride + (int64_t)in_page * hd;      // [row][hd]
     const bf16_t* vt = vh + (int64_t)page * page_stride + in_page;                     // [hd][row]
-    tile_step<DT, 1>(o, m_run, l_run, qf, kt, hd, vt, page_size, hd, pos0, pq, lq, scale);
+    const bool masked = pos0 + TILE - 1 > p || pos0 < lo_q;      // the same for all lanes
+    tile_step<DT, 1, EXACT>(o, m_run, l_run, qf, kt, hd, vt, page_size, hd, pos0, pq, lq, scale2, masked);
   }
 }
 
@@ -179,27 +195,35 @@ __device__ __forceinline__ void load_query(bf16x8 (&qf)[(DT + 1) / 2], const bf1
 }
 
 // ------------------------------------------------------------------------------------------ whole prompts
-// grid (ceil(longest run of new tokens / (64 QG)), nh, B), block 256: wave w takes tokens 16 QG (4 x + w) .. of
-// sequence z, QG groups of 16.  The cache already holds the step's keys and values.  The workgroup brings each
-// tile of keys and values into LDS once (key rows padded by KPAD, value rows VSTR long, so that the operand
-// reads do not collide) and its four waves read their operands from there.
+// grid (blocks of 64 QG new tokens x heads x sequences), block 256: wave w takes tokens 16 QG w .. of its block,
+// QG groups of 16.  The cache already holds the step's keys and values.  Blocks are numbered from the end of the
+// sequences: a block attends to everything before it, so the longest ones start first and the short ones fill
+// the gaps that they leave.  The workgroup brings each tile of keys and values into one of two LDS buffers
+// (key rows padded by KPAD, value rows VSTR long, so that the operand reads do not collide) while it works on
+// the other, and the tile after that is on its way from memory into registers meanwhile: one barrier per tile.
 #define KPAD 8
 #define VSTR 72
 
-template <int DT, int QG>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_kernel(AttnArgs a) {
+template <int DT, int QG, bool EXACT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_kernel(AttnArgs a, int n_blocks, int B) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  bf16_t* Ks = (bf16_t*)smem_raw;                    // [TILE][hd + KPAD]
-  bf16_t* Vs = Ks + TILE * (a.hd + KPAD);            // [hd][VSTR]
   constexpr int QW = 16 * QG;
-  const int seq = blockIdx.z, h = blockIdx.y;
+  constexpr int KCH = (TILE * 2 * DT + 255) / 256;      // 16-byte chunks of a key tile per thread
+  constexpr int VCH = (16 * DT * 8 + 255) / 256;        // and of a value tile
+  const int hd = EXACT ? 16 * DT : a.hd, kcpr = hd / 8;
+  const int buf = TILE * (hd + KPAD) + hd * VSTR;       // elements of one buffer: keys [TILE][hd + KPAD], values [hd][VSTR]
+  bf16_t* Ks = (bf16_t*)smem_raw;
+  bf16_t* Vs = Ks + TILE * (hd + KPAD);
+  const int per_block = a.nh * B;
+  const int blk = n_blocks - 1 - (int)blockIdx.x / per_block;
+  const int h = (int)blockIdx.x % per_block % a.nh, seq = (int)blockIdx.x % per_block / a.nh;
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, r = lane % 16, c = lane / 16;
   const int t0 = a.cu_seqlens[seq], n = a.cu_seqlens[seq + 1] - t0;
-  const int qb = blockIdx.x * 4 * QW;
+  const int qb = blk * 4 * QW;
   if (qb >= n) return;
   const int start = a.start[seq];
   const int kvh = h / (a.nh / a.nkv);
-  const int64_t head_off = (int64_t)kvh * a.page_size * a.hd;
+  const int64_t head_off = (int64_t)kvh * a.page_size * hd;
   const int* table = a.block_table + (size_t)a.slots[seq] * a.bt_stride;
 
   int p_q[QG], lo_q[QG];
@@ -212,7 +236,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     const bool valid = qi < n;
     p_q[g] = valid ? start + qi : -1;
     lo_q[g] = a.window > 0 ? max(0, p_q[g] - a.window + 1) : 0;
-    load_query<DT>(qf[g], a.q + ((size_t)(t0 + (valid ? qi : 0)) * a.nh + h) * a.hd, a.hd, valid);
+    load_query<DT>(qf[g], a.q + ((size_t)(t0 + (valid ? qi : 0)) * a.nh + h) * hd, hd, valid);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[g][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     m_run[g] = -INFINITY;
@@ -224,36 +248,72 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   const int wq0 = qb + wave * QW;
   const bool wave_has = wq0 < n;
   const int wave_first = start + wq0, wave_last = start + min(wq0 + QW, n) - 1;
+  const int wave_lo_last = a.window > 0 ? max(0, wave_last - a.window + 1) : 0;     // first key of the wave's last token
   const int wave_beg = (a.window > 0 ? max(0, wave_first - a.window + 1) : 0) / TILE;
   const int wave_end = wave_has ? wave_last / TILE + 1 : 0;
-  const int hd = a.hd, kcpr = hd / 8;
-  for (int tile = tile_beg; tile < tile_end; ++tile) {
-    const int pos0 = tile * TILE;
-    const int page = table[pos0 / a.page_size];
-    const int in_page = pos0 % a.page_size;
-    const bf16_t* kg = a.k_pool + head_off + (int64_t)page * a.page_stride + (int64_t)in_page * hd;
-    const bf16_t* vg = a.v_pool + head_off + (int64_t)page * a.page_stride + in_page;
-    for (int i = tid; i < TILE * kcpr; i += 256) {
-      const int row = i / kcpr, ch = i % kcpr;
-      *reinterpret_cast<u32x4*>(Ks + row * (hd + KPAD) + ch * 8) = *reinterpret_cast<const u32x4*>(kg + row * hd + ch * 8);
+
+  // what this thread carries of every tile: where its chunks lie in the tile in memory and in LDS (a thread
+  // past the end of a small tile carries the last chunk once more)
+  int k_g[KCH], k_l[KCH], v_g[VCH], v_l[VCH];
+#pragma unroll
+  for (int j = 0; j < KCH; ++j) {
+    const int i = min(tid + j * 256, TILE * kcpr - 1), row = i / kcpr, ch = i % kcpr;
+    k_g[j] = row * hd + ch * 8;
+    k_l[j] = row * (hd + KPAD) + ch * 8;
+  }
+#pragma unroll
+  for (int j = 0; j < VCH; ++j) {
+    const int i = min(tid + j * 256, hd * 8 - 1), d = i / 8, ch = i % 8;
+    v_g[j] = d * a.page_size + ch * 8;
+    v_l[j] = d * VSTR + ch * 8;
+  }
+  u32x4 pk[KCH], pv[VCH];
+  const int tiles_per_page = a.page_size / TILE;
+  int page_next = table[tile_beg / tiles_per_page];     // page of the tile that the next fetch takes
+#define TQ_FETCH(tile)                                                                                      \
+  do {                                                                                                      \
+    const int64_t base = head_off + (int64_t)page_next * a.page_stride;                                     \
+    const int in_page = ((tile) % tiles_per_page) * TILE;                                                   \
+    const bf16_t* kg = a.k_pool + base + (int64_t)in_page * hd;                                             \
+    const bf16_t* vg = a.v_pool + base + in_page;                                                           \
+    _Pragma("unroll") for (int j = 0; j < KCH; ++j) pk[j] = *reinterpret_cast<const u32x4*>(kg + k_g[j]);   \
+    _Pragma("unroll") for (int j = 0; j < VCH; ++j) pv[j] = *reinterpret_cast<const u32x4*>(vg + v_g[j]);   \
+    if ((tile) + 1 < tile_end) page_next = table[((tile) + 1) / tiles_per_page];                            \
+  } while (0)
+#define TQ_STAGE(off)                                                                                       \
+  do {                                                                                                      \
+    _Pragma("unroll") for (int j = 0; j < KCH; ++j) *reinterpret_cast<u32x4*>(Ks + (off) + k_l[j]) = pk[j]; \
+    _Pragma("unroll") for (int j = 0; j < VCH; ++j) *reinterpret_cast<u32x4*>(Vs + (off) + v_l[j]) = pv[j]; \
+  } while (0)
+
+  TQ_FETCH(tile_beg);
+  TQ_STAGE(0);
+  if (tile_beg + 1 < tile_end) TQ_FETCH(tile_beg + 1);
+  __syncthreads();
+  int cur = 0;
+  for (int tile = tile_beg; tile < tile_end; ++tile, cur ^= buf) {
+    if (tile + 1 < tile_end) {
+      TQ_STAGE(cur ^ buf);
+      if (tile + 2 < tile_end) TQ_FETCH(tile + 2);
     }
-    for (int i = tid; i < hd * 8; i += 256) {
-      const int d = i / 8, ch = i % 8;
-      *reinterpret_cast<u32x4*>(Vs + d * VSTR + ch * 8) = *reinterpret_cast<const u32x4*>(vg + (int64_t)d * a.page_size + ch * 8);
+    if (tile >= wave_beg && tile < wave_end) {
+      const int pos0 = tile * TILE;
+      const bool masked = pos0 + TILE - 1 > wave_first || pos0 < wave_lo_last;
+      tile_step<DT, QG, EXACT>(o, m_run, l_run, qf, Ks + cur, hd + KPAD, Vs + cur, VSTR, hd, pos0, p_q, lo_q,
+                        a.scale * LOG2E, masked);
     }
-    __syncthreads();
-    if (tile >= wave_beg && tile < wave_end)
-      tile_step<DT, QG>(o, m_run, l_run, qf, Ks, hd + KPAD, Vs, VSTR, hd, pos0, p_q, lo_q, a.scale);
     __syncthreads();
   }
+#undef TQ_FETCH
+#undef TQ_STAGE
 #pragma unroll
   for (int g = 0; g < QG; ++g) {
     if (p_q[g] < 0) continue;
     const float inv = 1.0f / l_run[g];
-    bf16_t* orow = a.out + ((size_t)(t0 + p_q[g] - start) * a.nh + h) * a.hd;
+    bf16_t* orow = a.out + ((size_t)(t0 + p_q[g] - start) * a.nh + h) * hd;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-      if (16 * dt < a.hd) {
+      if (16 * dt < hd) {
         const u32x2 w = {pack2(o[g][dt][0] * inv, o[g][dt][1] * inv), pack2(o[g][dt][2] * inv, o[g][dt][3] * inv)};
         *reinterpret_cast<u32x2*>(orow + 16 * dt + 4 * c) = w;
       }
@@ -265,7 +325,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 // One new token per sequence at position start[b].  grid (max_runs, nkv * ceil(g / 16), B), block 64: the wave
 // takes run x (tiles SPLIT x .. SPLIT x + SPLIT - 1) for up to 16 of the g = nh / nkv heads of one kv head and
 // writes their unnormalised sums with maximum and denominator.
-template <int DT>
+template <int DT, bool EXACT>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DT > 8 ? 2 : 3))) void attn_decode_kernel(AttnArgs a) {
   const int b = blockIdx.z, run = blockIdx.x;
   const int g = a.nh / a.nkv, ngc = (g + 15) / 16;
@@ -288,8 +348,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DT > 8 ? 2 :
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) o[0][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m_run[1] = {-INFINITY}, l_run[1] = {0.f};
-  attend<DT>(o, m_run, l_run, qf, a.k_pool + head_off, a.v_pool + head_off, table, a.page_size, a.page_stride, a.hd,
-             tile_beg, tile_end, valid ? p : -1, lo, a.scale);
+  attend<DT, EXACT>(o, m_run, l_run, qf, a.k_pool + head_off, a.v_pool + head_off, table, a.page_size, a.page_stride, a.hd,
+             tile_beg, tile_end, p, valid, lo, a.scale * LOG2E);
   if (!valid) return;
   float* out = a.partial + (((size_t)b * a.nh + h) * a.max_runs + run) * (a.hd + 2);
 #pragma unroll
@@ -306,7 +366,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DT > 8 ? 2 :
 }
 
 // Joins the runs of one (sequence, head) in order of position: grid (nh, B), block 64.  The weights
-// exp(m_s - m) of the runs are worked out once, a lane per run, and kept in LDS; then every lane sums its
+// 2^(m_s - m) of the runs are worked out once, a lane per run, and kept in LDS; then every lane sums its
 // dimensions over the runs in order.
 #define MAX_RUNS_LDS 1024
 __global__ __launch_bounds__(64) void attn_join_kernel(AttnArgs a) {
@@ -325,7 +385,7 @@ __global__ __launch_bounds__(64) void attn_join_kernel(AttnArgs a) {
     const int s = s0 + lane;
     float w = 0.f, wl = 0.f;
     if (s < run_end) {
-      w = expf(part[(size_t)s * stride + a.hd] - m);
+      w = __builtin_amdgcn_exp2f(part[(size_t)s * stride + a.hd] - m);      // maxima are in units of log2
       wl = w * part[(size_t)s * stride + a.hd + 1];
       wgt[s - run_beg] = w;
     }
@@ -343,18 +403,20 @@ __global__ __launch_bounds__(64) void attn_join_kernel(AttnArgs a) {
 }
 
 // ------------------------------------------------------------------------------------------ launch
-template <int DT, int QG>
-static void launch_prefill(const AttnArgs& a, int B, int max_new, hipStream_t st) {
-  const size_t shmem = ((size_t)TILE * (a.hd + KPAD) + (size_t)a.hd * VSTR) * sizeof(bf16_t);
+template <int DT, int QG, bool EXACT>
+static int launch_prefill(const AttnArgs& a, int B, int max_new, hipStream_t st) {
+  const size_t shmem = 2 * ((size_t)TILE * (a.hd + KPAD) + (size_t)a.hd * VSTR) * sizeof(bf16_t);
   if (shmem > 48 * 1024)
-    hipFuncSetAttribute((const void*)attn_prefill_kernel<DT, QG>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
-  hipLaunchKernelGGL((attn_prefill_kernel<DT, QG>), dim3((max_new + 64 * QG - 1) / (64 * QG), a.nh, B), dim3(256), shmem,
-                     st, a);
+    hipFuncSetAttribute((const void*)attn_prefill_kernel<DT, QG, EXACT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+  const int n_blocks = (max_new + 64 * QG - 1) / (64 * QG);
+  if ((int64_t)n_blocks * a.nh * B > 0x7fffffff) return TQ_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL((attn_prefill_kernel<DT, QG, EXACT>), dim3(n_blocks * a.nh * B), dim3(256), shmem, st, a, n_blocks, B);
+  return 0;
 }
-template <int DT>
+template <int DT, bool EXACT>
 static void launch_decode(const AttnArgs& a, int B, hipStream_t st) {
   const int g = a.nh / a.nkv;
-  hipLaunchKernelGGL(attn_decode_kernel<DT>, dim3(a.max_runs, a.nkv * ((g + 15) / 16), B), dim3(64), 0, st, a);
+  hipLaunchKernelGGL((attn_decode_kernel<DT, EXACT>), dim3(a.max_runs, a.nkv * ((g + 15) / 16), B), dim3(64), 0, st, a);
   hipLaunchKernelGGL(attn_join_kernel, dim3(a.nh, B), dim3(64), 0, st, a);
 }
 
@@ -373,22 +435,33 @@ TQ_API int tq_attention_mfma(const void* q, const void* k_pool, const void* v_po
   if (B <= 0) return 0;
   if (hd % 16 != 0 || hd < 16 || hd > 256 || page_size % TILE != 0 || nkv <= 0 || nh % nkv != 0)
     return TQ_ERR_UNSUPPORTED;
-  if (nh > 65535 || B > 65535 || page_stride % 8 != 0) return TQ_ERR_UNSUPPORTED;
+  if (nh > 65535 || B > 65535 || page_stride % 8 != 0 || !(scale > 0.f)) return TQ_ERR_UNSUPPORTED;
   if (decode && (max_end + TILE * SPLIT - 1) / (TILE * SPLIT) > MAX_RUNS_LDS) return TQ_ERR_UNSUPPORTED;
   AttnArgs a{(const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, bt_stride, cu_seqlens, slots,
              start, page_size, page_stride, nh, nkv, hd, window, scale, (bf16_t*)out, partial,
              (max_end + TILE * SPLIT - 1) / (TILE * SPLIT)};
   const int dt = hd / 16;
+  // head sizes 64, 128 and 256 have kernels of their own in which nothing depends on hd at run time
   if (decode) {
     if (!partial) return TQ_ERR_BAD_ARG;
-    if (dt <= 4) launch_decode<4>(a, B, st);
-    else if (dt <= 8) launch_decode<8>(a, B, st);
-    else launch_decode<16>(a, B, st);
+    if (dt == 4) launch_decode<4, true>(a, B, st);
+    else if (dt == 8) launch_decode<8, true>(a, B, st);
+    else if (dt == 16) launch_decode<16, true>(a, B, st);
+    else if (dt < 4) launch_decode<4, false>(a, B, st);
+    else if (dt < 8) launch_decode<8, false>(a, B, st);
+    else launch_decode<16, false>(a, B, st);
   } else {
-    // two groups of 16 tokens per wave when the runs are long enough to fill them and registers allow
-    if (dt <= 4) { if (max_new > 64) launch_prefill<4, 2>(a, B, max_new, st); else launch_prefill<4, 1>(a, B, max_new, st); }
-    else if (dt <= 8) { if (max_new > 64) launch_prefill<8, 2>(a, B, max_new, st); else launch_prefill<8, 1>(a, B, max_new, st); }
-    else launch_prefill<16, 1>(a, B, max_new, st);
+    // two groups of 16 tokens per wave, which halves the reads from LDS per product, when that still leaves
+    // the chip two workgroups per compute unit and registers allow; else one group
+    const bool two = (int64_t)((max_new + 127) / 128) * nh * B >= 512;
+    int rc;
+    if (dt == 4) rc = two ? launch_prefill<4, 2, true>(a, B, max_new, st) : launch_prefill<4, 1, true>(a, B, max_new, st);
+    else if (dt == 8) rc = two ? launch_prefill<8, 2, true>(a, B, max_new, st) : launch_prefill<8, 1, true>(a, B, max_new, st);
+    else if (dt == 16) rc = launch_prefill<16, 1, true>(a, B, max_new, st);
+    else if (dt < 4) rc = two ? launch_prefill<4, 2, false>(a, B, max_new, st) : launch_prefill<4, 1, false>(a, B, max_new, st);
+    else if (dt < 8) rc = two ? launch_prefill<8, 2, false>(a, B, max_new, st) : launch_prefill<8, 1, false>(a, B, max_new, st);
+    else rc = launch_prefill<16, 1, false>(a, B, max_new, st);
+    if (rc) return rc;
   }
   TQ_LAUNCH_CHECK();
   return 0;

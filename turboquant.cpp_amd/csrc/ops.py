@@ -311,7 +311,7 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, lay
     esz = k_pages.element_size()
     lib = library(act)
     if (runs is not None and dtype_name(act) == "bfloat16" and hasattr(lib, "tq_attention_mfma")
-            and head_dim % 16 == 0 and head_dim <= 256 and page_size % 64 == 0 and page_stride % 8 == 0):
+            and head_dim % 16 == 0 and head_dim <= 256 and page_size % 64 == 0 and page_stride % 8 == 0 and scale > 0):
         B = runs["slots"].numel()
         _check(runs["cu_seqlens"], k, "cu_seqlens", torch.int32, (B + 1,))
         _check(runs["slots"], k, "slots", torch.int32, (B,))
