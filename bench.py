@@ -40,11 +40,13 @@ def layer_weight_elems(c, experts_used: float) -> float:
     return attn + moe + 2 * H
 
 
-def decode_bytes(c, layers: int, batch: int, context: float, wbytes: int = 2) -> float:
-    """Bytes a decode step has to read: every weight it uses once (the experts that a batch of random tokens
-    reaches, in expectation) and the keys and values of the live requests."""
+def decode_bytes(c, layers: int, batch: int, context: float, wbytes: int = 2, used: float | None = None) -> float:
+    """Bytes a decode step has to read: every weight it uses once (`used` experts a layer, counted in a step of
+    the run; without a count, what a batch of uniformly routed tokens reaches in expectation) and the keys and
+    values of the live requests."""
     E, k = c["num_experts"], c["num_experts_per_tok"]
-    used = E * (1.0 - (1.0 - k / E) ** batch)
+    if used is None:
+        used = E * (1.0 - (1.0 - k / E) ** batch)
     hd = c["hidden_size"] // c["num_attention_heads"]
     w = layers * layer_weight_elems(c, used) + c["vocab_size"] * c["hidden_size"] + c["hidden_size"]
     kv = batch * context * layers * 2 * c["num_key_value_heads"] * hd
@@ -122,7 +124,22 @@ def main() -> int:
             lg = engine.step(slots, [[t] for t in tokens])
             return ops.argmax(lg, act).tolist()
 
-        for _ in range(warmup):
+        # the first warm-up step (which runs eagerly) also counts the distinct experts that each layer's router picks
+        picked = []
+        router_topk = ops.router_topk
+
+        def counting_router(*a, **k):
+            out = router_topk(*a, **k)
+            picked.append(int(torch.unique(out[0]).numel()))
+            return out
+
+        ops.router_topk = counting_router
+        try:
+            tokens = one_step(tokens)
+        finally:
+            ops.router_topk = router_topk
+        experts_used = sum(picked) / max(len(picked), 1)
+        for _ in range(warmup - 1):
             tokens = one_step(tokens)
         torch.cuda.synchronize()
         t = time.perf_counter()
@@ -134,7 +151,7 @@ def main() -> int:
         engine.close(slots)
         del engine
         torch.cuda.empty_cache()
-        return dt / steps, mean_ctx
+        return dt / steps, mean_ctx, experts_used
 
     def run_prefill(T: int):
         engine = Engine(model, max_tokens=T + 64, page_size=64, max_slots=1)
@@ -158,14 +175,14 @@ def main() -> int:
                           "unit": "tok/s", "ms": round(pf * 1e3, 3), "layers": args.layers, "dtype": short,
                           "frac": round(prefill_flops(cfg, args.layers, PREFILL_TOKENS) / pf / PEAK_FLOPS[short], 4)}))
         return 0
-    sec, mean_ctx = run_decode(args.batch, args.context, args.steps, args.warmup)
+    sec, mean_ctx, experts_used = run_decode(args.batch, args.context, args.steps, args.warmup)
     value = args.batch / sec
-    read = decode_bytes(cfg, args.layers, args.batch, mean_ctx, 2 if act == "bfloat16" else 4)
+    read = decode_bytes(cfg, args.layers, args.batch, mean_ctx, 2 if act == "bfloat16" else 4, experts_used)
     achieved = read / sec / 1e9
     points = {}
     if not args.no_points:
         for b in (1, 64):
-            s, _ = run_decode(b, args.points_context, 32, 4)
+            s, _, _ = run_decode(b, args.points_context, 32, 4)
             points[f"decode_b{b}"] = round(b / s, 1)
     out = {
         "metric": "decode tok/s at batch 8, context 8192 (Qwen1.5-MoE-A2.7B layer sizes, random weights)",
@@ -180,6 +197,7 @@ def main() -> int:
             "shared_inner": cfg["shared_expert_intermediate_size"], "global_batch": args.batch,
             "seq_len": args.context, "parallelism": "single GPU", "points_context": args.points_context,
             "prefill_tokens": PREFILL_TOKENS, "weights": "random N(0,0.02) seed 2", "kv_cache": short,
+            "experts_read_per_layer": round(experts_used, 1),
         },
         "prefill": {"value": round(PREFILL_TOKENS / pf, 1), "tokens": PREFILL_TOKENS, "ms": round(pf * 1e3, 3),
                     "frac": round(prefill_flops(cfg, args.layers, PREFILL_TOKENS) / pf / PEAK_FLOPS[short], 4)},

@@ -20,6 +20,8 @@ def embed(tokens, table, act):
 
 
 def add_rmsnorm(x, delta, weight, eps, act, rows=None, want_act=True, want_f32=False):
+    if hasattr(delta, "pair_slot"):      # a sum over experts that is still to be done
+        delta = moe_combine(delta.y, delta.pair_slot, delta.weights, delta.dense, delta.gate, act)
     v = x if delta is None else x + delta.sum(dim=0)
     if rows is None:
         x.copy_(v)

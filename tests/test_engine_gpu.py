@@ -347,7 +347,15 @@ def test_feed_forward_parts_alone(act):
         assert moe.wants_f32 and ("shared_scale" in moe.param_specs()) == (shared > 0)
         w = {n: rnd(s.shape, act, 50 + i, 0.3) for i, (n, s) in enumerate(moe.param_specs().items())}
         moe.set_params({n: t.to(DEV) for n, t in w.items()})
-        y = moe.forward(x.to(DEV), x.float().to(DEV), ctx)[0].cpu().double()
+        unsummed = moe.forward(x.to(DEV), x.float().to(DEV), ctx)
+        y = unsummed.materialize(act)[0].cpu().double()
+        # the next norm sums it in its own pass: the same bits as summing first
+        norm = build_part("norm", PartSpec("rmsnorm", dict(size=H, eps=1e-5)))
+        norm.set_params({"weight": rnd((H,), act, 77, 0.5).to(DEV)})
+        stream_a, stream_b = x.float().to(DEV).clone(), x.float().to(DEV).clone()
+        fused = norm.forward(stream_a, unsummed, ctx, want_f32=True)[1]
+        apart = norm.forward(stream_b, unsummed.materialize(act), ctx, want_f32=True)[1]
+        assert torch.equal(fused, apart) and torch.equal(stream_a, stream_b)
         pw = {"router": w["router"].double(),
               "experts": [{"gate": w["expert_gate"][e].double(), "up": w["expert_up"][e].double(),
                            "down": w["expert_down"][e].double()} for e in range(7)]}

@@ -172,6 +172,24 @@ def test_moe_combine(ops, act):
     assert (out.double() - ref).abs().max() < 1e-5
     out2 = ops.moe_combine(y.to(DEV), slot.to(DEV), wts.to(DEV), None, None, act).cpu()[0]
     assert (out2.double() - (wts[:, :, None].double() * y[slot.long()].double()).sum(1)).abs().max() < 1e-5
+    # the same sum left to the norm: against the plain formula, for all rows and for chosen rows
+    x = rnd((T, H), torch.float32, 53)
+    w = rnd((H,), adt(act), 54)
+    eps = 1e-5
+    for dense, gt in ((shared, gate), (None, None)):
+        v = x.double() + (wts[:, :, None].double() * y[slot.long()].double()).sum(1)
+        if dense is not None:
+            v = v + gt[:, None].double() * dense.double().sum(0)
+        want = v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps) * w.double()
+        unsummed = ops.GatheredSum(y.to(DEV), slot.to(DEV), wts.to(DEV), None if dense is None else dense.to(DEV),
+                                   None if gt is None else gt.to(DEV))
+        xs = x.to(DEV).clone()
+        got = ops.add_rmsnorm(xs, unsummed, w.to(DEV), eps, act, want_act=False, want_f32=True)[1].cpu()
+        assert (got.double() - want).abs().max() < 1e-4 and (xs.cpu().double() - v).abs().max() < 1e-5
+        rows = torch.tensor([4, 1], dtype=torch.int32)
+        xs = x.to(DEV).clone()
+        got = ops.add_rmsnorm(xs, unsummed, w.to(DEV), eps, act, rows=rows.to(DEV), want_act=False, want_f32=True)[1].cpu()
+        assert (got.double() - want[rows.long()]).abs().max() < 1e-4 and torch.equal(xs.cpu(), x)
 
 
 # ------------------------------------------------------------------------------------------------ router

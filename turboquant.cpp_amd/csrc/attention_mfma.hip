@@ -72,15 +72,27 @@ __device__ __forceinline__ float group_sum(float v) {
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
+// Where the workgroup's tiles lie in LDS when the head size is 64, 128 or 256 (rows of 8, 16 or 32 chunks of 16
+// bytes, no padding): chunk ch of key row `row` at chunk ch ^ g(row), where g numbers the 16 rows that one
+// operand read touches (rows r % 4 + 8 (r / 4) + const) 0..15, or 0..7 twice for rows of 8 chunks; chunk ch of value
+// row d (64 positions, 8 chunks) at chunk ch ^ (d & 7).  Measured: such reads run at about 210 bytes per clock
+// and compute unit, rows padded by 16 bytes at about 120.
+template <int DT>
+__device__ __forceinline__ int k_swz(int row, int ch) {
+  const int g = DT == 4 ? (((row >> 1) & 1) | (((row >> 3) & 3) << 1)) : ((row & 3) | (((row >> 3) & 3) << 2));
+  return row * (16 * DT) + ((ch ^ g) << 3);
+}
+__device__ __forceinline__ int v_swz(int d, int ch) { return d * TILE + ((ch ^ (d & 7)) << 3); }
+
 // One tile of 64 positions for QG groups of 16 columns that share the tile's keys and values.  kt: the tile's
 // keys, row i at kt + i * k_stride; vt: the tile's values transposed, dimension d at vt + d * v_stride (memory or
 // LDS).  DT: number of 16-wide blocks of hd held in registers (hd <= 16 * DT).  p_q: position of this lane's
 // column in each group (-1: no such column), lo_q: first position it may see; masked: whether any column of the
 // wave has a key in this tile that it may not see (if not, the comparisons are left out).  qf: the columns'
 // queries, 8 values of hd per 32-wide step at 8 * (l / 16).  Every operand read from kt and vt serves all QG
-// groups.  EXACT: hd is exactly 16 DT and DT is even.  scale2 = scale * log2(e) > 0: maxima are kept in that unit and probabilities are 2^(s * scale2 - m),
+// groups.  EXACT: hd is exactly 16 DT and DT is even.  SWZ: kt and vt are tiles in LDS laid out by k_swz, v_swz.  scale2 = scale * log2(e) > 0: maxima are kept in that unit and probabilities are 2^(s * scale2 - m),
 // which is exp(s * scale - max) with one instruction for the power.
-template <int DT, int QG, bool EXACT>
+template <int DT, int QG, bool EXACT, bool SWZ = false>
 __device__ __forceinline__ void tile_step(f32x4 (&o)[QG][DT], float (&m_run)[QG], float (&l_run)[QG],
                                           const bf16x8 (&qf)[QG][(DT + 1) / 2], const bf16_t* kt, int k_stride,
                                           const bf16_t* vt, int v_stride, int hd, int pos0, const int (&p_q)[QG],
@@ -98,7 +110,9 @@ __device__ __forceinline__ void tile_step(f32x4 (&o)[QG][DT], float (&m_run)[QG]
     for (int ks = 0; ks < KS; ++ks) {
       if (ks < n_ks) {
         const int d0 = 32 * ks + 8 * c;
-        const bf16x8 kf = EXACT || d0 < hd ? ld16(kt + (32 * (jt / 2) + 8 * (r / 4) + 4 * (jt % 2) + r % 4) * k_stride + d0) : zero16();
+        const int krow = 32 * (jt / 2) + 8 * (r / 4) + 4 * (jt % 2) + r % 4;
+        const bf16x8 kf = SWZ ? ld16(kt + k_swz<DT>(krow, 4 * ks + c))
+                              : (EXACT || d0 < hd ? ld16(kt + krow * k_stride + d0) : zero16());
 #pragma unroll
         for (int g = 0; g < QG; ++g) s[g][jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[g][ks], s[g][jt], 0, 0, 0);
       }
@@ -158,7 +172,7 @@ __device__ __forceinline__ void tile_step(f32x4 (&o)[QG][DT], float (&m_run)[QG]
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       if (dt < n_dt) {
-        const bf16x8 vf = ld16(vt + (16 * dt + r) * v_stride + 32 * pr + 8 * c);
+        const bf16x8 vf = SWZ ? ld16(vt + v_swz(16 * dt + r, 4 * pr + c)) : ld16(vt + (16 * dt + r) * v_stride + 32 * pr + 8 * c);
 #pragma unroll
         for (int g = 0; g < QG; ++g) o[g][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[g], o[g][dt], 0, 0, 0);
       }
@@ -199,7 +213,7 @@ __device__ __forceinline__ void load_query(bf16x8 (&qf)[(DT + 1) / 2], const bf1
 // QG groups of 16.  The cache already holds the step's keys and values.  Blocks are numbered from the end of the
 // sequences: a block attends to everything before it, so the longest ones start first and the short ones fill
 // the gaps that they leave.  The workgroup brings each tile of keys and values into one of two LDS buffers
-// (key rows padded by KPAD, value rows VSTR long, so that the operand reads do not collide) while it works on
+// (swizzled for head sizes 64, 128, 256; else key rows padded by KPAD and value rows VSTR long) while it works on
 // the other, and the tile after that is on its way from memory into registers meanwhile: one barrier per tile.
 #define KPAD 8
 #define VSTR 72
@@ -211,9 +225,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   constexpr int KCH = (TILE * 2 * DT + 255) / 256;      // 16-byte chunks of a key tile per thread
   constexpr int VCH = (16 * DT * 8 + 255) / 256;        // and of a value tile
   const int hd = EXACT ? 16 * DT : a.hd, kcpr = hd / 8;
-  const int buf = TILE * (hd + KPAD) + hd * VSTR;       // elements of one buffer: keys [TILE][hd + KPAD], values [hd][VSTR]
+  // elements of one buffer: keys [TILE][hd + KPAD], values [hd][VSTR]; swizzled instead of padded when EXACT
+  const int kstr = EXACT ? hd : hd + KPAD, vstr = EXACT ? TILE : VSTR;
+  const int buf = TILE * kstr + hd * vstr;
   bf16_t* Ks = (bf16_t*)smem_raw;
-  bf16_t* Vs = Ks + TILE * (hd + KPAD);
+  bf16_t* Vs = Ks + TILE * kstr;
   const int per_block = a.nh * B;
   const int blk = n_blocks - 1 - (int)blockIdx.x / per_block;
   const int h = (int)blockIdx.x % per_block % a.nh, seq = (int)blockIdx.x % per_block / a.nh;
@@ -259,13 +275,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
   for (int j = 0; j < KCH; ++j) {
     const int i = min(tid + j * 256, TILE * kcpr - 1), row = i / kcpr, ch = i % kcpr;
     k_g[j] = row * hd + ch * 8;
-    k_l[j] = row * (hd + KPAD) + ch * 8;
+    k_l[j] = EXACT ? k_swz<DT>(row, ch) : row * kstr + ch * 8;
   }
 #pragma unroll
   for (int j = 0; j < VCH; ++j) {
     const int i = min(tid + j * 256, hd * 8 - 1), d = i / 8, ch = i % 8;
     v_g[j] = d * a.page_size + ch * 8;
-    v_l[j] = d * VSTR + ch * 8;
+    v_l[j] = EXACT ? v_swz(d, ch) : d * vstr + ch * 8;
   }
   u32x4 pk[KCH], pv[VCH];
   const int tiles_per_page = a.page_size / TILE;
@@ -299,8 +315,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     if (tile >= wave_beg && tile < wave_end) {
       const int pos0 = tile * TILE;
       const bool masked = pos0 + TILE - 1 > wave_first || pos0 < wave_lo_last;
-      tile_step<DT, QG, EXACT>(o, m_run, l_run, qf, Ks + cur, hd + KPAD, Vs + cur, VSTR, hd, pos0, p_q, lo_q,
-                        a.scale * LOG2E, masked);
+      tile_step<DT, QG, EXACT, EXACT>(o, m_run, l_run, qf, Ks + cur, kstr, Vs + cur, vstr, hd, pos0, p_q, lo_q,
+                                      a.scale * LOG2E, masked);
     }
     __syncthreads();
   }
@@ -405,7 +421,7 @@ __global__ __launch_bounds__(64) void attn_join_kernel(AttnArgs a) {
 // ------------------------------------------------------------------------------------------ launch
 template <int DT, int QG, bool EXACT>
 static int launch_prefill(const AttnArgs& a, int B, int max_new, hipStream_t st) {
-  const size_t shmem = 2 * ((size_t)TILE * (a.hd + KPAD) + (size_t)a.hd * VSTR) * sizeof(bf16_t);
+  const size_t shmem = 2 * (EXACT ? (size_t)2 * TILE * a.hd : (size_t)TILE * (a.hd + KPAD) + (size_t)a.hd * VSTR) * sizeof(bf16_t);
   if (shmem > 48 * 1024)
     hipFuncSetAttribute((const void*)attn_prefill_kernel<DT, QG, EXACT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
   const int n_blocks = (max_new + 64 * QG - 1) / (64 * QG);

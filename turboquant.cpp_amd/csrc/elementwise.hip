@@ -24,25 +24,52 @@ TQ_API int tq_embed(const int* tokens, const void* table, int wtype, float* x, i
 
 // ---------------------------------------------------------------- residual sum + RMS norm
 // For row r (token rows[r], or r itself when rows is null):
-//   v = x[row] + sum_s delta[s][row]            (the residual sum, in float, s ascending)
+//   v = x[row] + d[row]                         (the residual sum, in float)
 //   x[row] = v                                  (only when rows is null)
 //   ss = sum v^2 / H + eps ; out = (v * (1/sqrt(ss))) * w
-// Formula and product order of /root/reference/src/engine/tq_ops.c:1373-1410.
+// Formula and product order of /root/reference/src/engine/tq_ops.c:1373-1410.  What is added, d, is either
+//   the partial sums delta[s][row] one after the other, s ascending (each added to v in turn), or, with y set,
+//   the experts' outputs that nobody has summed yet, as moe_combine below would:
+//   d = sum_j weights[row][j] * y[pair_slot[row][j]] (j ascending) + gate[row] * sum_s delta[s][row].
 // The sum of squares is taken in a fixed order that does not depend on the number of rows.
 template <class W>
 __global__ void add_rmsnorm_kernel(float* __restrict__ x, const float* __restrict__ delta, int S,
-                                   size_t delta_stride, const W* __restrict__ w, float eps,
+                                   size_t delta_stride, const float* __restrict__ y,
+                                   const int* __restrict__ pair_slot, const float* __restrict__ weights, int topk,
+                                   const float* __restrict__ gate, const W* __restrict__ w, float eps,
                                    const int* __restrict__ rows, act_t* __restrict__ out,
                                    float* __restrict__ out32, int H) {
   extern __shared__ float v[];       // H floats, then one float per wave
+  __shared__ int slot[64];
+  __shared__ float wgt[64];
   float* red = v + H;
   const int r = blockIdx.x;
   const int row = rows ? rows[r] : r;
   float* xr = x + (size_t)row * H;
+  float g = 1.0f;
+  if (y) {
+    if (threadIdx.x < topk) {      // the token's rows and weights once, not once per element
+      slot[threadIdx.x] = pair_slot[(size_t)row * topk + threadIdx.x];
+      wgt[threadIdx.x] = weights[(size_t)row * topk + threadIdx.x];
+    }
+    if (gate) g = gate[row];
+    __syncthreads();
+  }
   float ss = 0.f;
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     float a = xr[i];
-    for (int s = 0; s < S; ++s) a += delta[s * delta_stride + (size_t)row * H + i];
+    if (y) {
+      float acc = 0.f;
+      for (int j = 0; j < topk; ++j) acc += wgt[j] * y[(size_t)slot[j] * H + i];
+      if (S > 0) {
+        float sh = 0.f;
+        for (int s = 0; s < S; ++s) sh += delta[s * delta_stride + (size_t)row * H + i];
+        acc += g * sh;
+      }
+      a += acc;
+    } else {
+      for (int s = 0; s < S; ++s) a += delta[s * delta_stride + (size_t)row * H + i];
+    }
     v[i] = a;
     if (!rows) xr[i] = a;
     ss += a * a;
@@ -57,17 +84,20 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const float* __restric
   }
 }
 
-TQ_API int tq_add_rmsnorm(float* x, const float* delta, int S, int64_t delta_stride, const void* w, int wtype,
-                          float eps, const int* rows, int R, void* out, float* out32, int H, hipStream_t st) {
+TQ_API int tq_add_rmsnorm(float* x, const float* delta, int S, int64_t delta_stride, const float* y,
+                          const int* pair_slot, const float* weights, int topk, const float* gate, const void* w,
+                          int wtype, float eps, const int* rows, int R, void* out, float* out32, int H,
+                          hipStream_t st) {
   if (R <= 0) return 0;
+  if (y && (topk < 1 || topk > 64 || !pair_slot || !weights)) return TQ_ERR_BAD_ARG;
   const int threads = 256;
   const size_t shmem = (size_t)(H + threads / TQ_WAVE) * sizeof(float);
-  if (shmem > 160 * 1024) return TQ_ERR_UNSUPPORTED;
+  if (shmem > 150 * 1024) return TQ_ERR_UNSUPPORTED;
   TQ_DISPATCH_W(wtype, {
     if (shmem > 48 * 1024)
       hipFuncSetAttribute((const void*)add_rmsnorm_kernel<W>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
-    hipLaunchKernelGGL(add_rmsnorm_kernel<W>, dim3(R), dim3(threads), shmem, st, x, delta, S, (size_t)delta_stride,
-                       (const W*)w, eps, rows, (act_t*)out, out32, H);
+    hipLaunchKernelGGL(add_rmsnorm_kernel<W>, dim3(R), dim3(threads), shmem, st, x, delta, S, (size_t)delta_stride, y,
+                       pair_slot, weights, topk, gate, (const W*)w, eps, rows, (act_t*)out, out32, H);
   });
   TQ_LAUNCH_CHECK();
   return 0;

@@ -49,10 +49,10 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float* __restr
     const int Hp4 = Hp / 4, H4 = H / 4;
     f32x4* dst = reinterpret_cast<f32x4*>(xs);
     const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-    for (int i = threadIdx.x; i < TG * Hp4; i += blockDim.x) {
-      const int k = i / Hp4, j = i % Hp4;
-      dst[i] = k < nt && j < H4 ? reinterpret_cast<const f32x4*>(x + (size_t)(t0 + k) * H)[j] : zero;
-    }
+#pragma unroll
+    for (int k = 0; k < TG; ++k)
+      for (int j = threadIdx.x; j < Hp4; j += blockDim.x)
+        dst[k * Hp4 + j] = k < nt && j < H4 ? reinterpret_cast<const f32x4*>(x + (size_t)(t0 + k) * H)[j] : zero;
   } else {
     for (int i = threadIdx.x; i < TG * Hp; i += blockDim.x) {
       const int k = i / Hp, j = i % Hp;
@@ -79,31 +79,41 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float* __restr
     if (vec) {
       const f32x4* xv = reinterpret_cast<const f32x4*>(xs);
       const int Hp4 = Hp / 4;
-#pragma unroll(RW >= 4 ? 2 : 4)
-      for (int b = 0; b < Hp; b += 512) {
-        const int g0 = min(b + 4 * lane, H - 4), g1 = min(b + 256 + 4 * lane, H - 4);
-        float w[RW][8];
+      constexpr int NB = RW >= 4 ? 2 : 4;      // blocks whose weights are asked for before the first is used
+      for (int b0 = 0; b0 < Hp; b0 += NB * 512) {
+        float w[NB][RW][8];
 #pragma unroll
-        for (int r = 0; r < RW; ++r) {
-          load4(row[r] + g0, &w[r][0]);
-          load4(row[r] + g1, &w[r][4]);
-        }
-#pragma unroll
-        for (int k = 0; k < TG; ++k) {
-          const f32x4 a = xv[k * Hp4 + b / 4 + lane];
-          const f32x4 c = xv[k * Hp4 + b / 4 + 64 + lane];
+        for (int u = 0; u < NB; ++u) {
+          const int b = b0 + u * 512;
+          const int g0 = min(b + 4 * lane, H - 4), g1 = min(b + 256 + 4 * lane, H - 4);
 #pragma unroll
           for (int r = 0; r < RW; ++r) {
-            float v = s[r][k];
-            v = fmaf(a.x, w[r][0], v);
-            v = fmaf(a.y, w[r][1], v);
-            v = fmaf(a.z, w[r][2], v);
-            v = fmaf(a.w, w[r][3], v);
-            v = fmaf(c.x, w[r][4], v);
-            v = fmaf(c.y, w[r][5], v);
-            v = fmaf(c.z, w[r][6], v);
-            v = fmaf(c.w, w[r][7], v);
-            s[r][k] = v;
+            load4(row[r] + g0, &w[u][r][0]);
+            load4(row[r] + g1, &w[u][r][4]);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+          const int b = b0 + u * 512;
+          if (b < Hp) {
+#pragma unroll
+            for (int k = 0; k < TG; ++k) {
+              const f32x4 a = xv[k * Hp4 + b / 4 + lane];
+              const f32x4 c = xv[k * Hp4 + b / 4 + 64 + lane];
+#pragma unroll
+              for (int r = 0; r < RW; ++r) {
+                float v = s[r][k];
+                v = fmaf(a.x, w[u][r][0], v);
+                v = fmaf(a.y, w[u][r][1], v);
+                v = fmaf(a.z, w[u][r][2], v);
+                v = fmaf(a.w, w[u][r][3], v);
+                v = fmaf(c.x, w[u][r][4], v);
+                v = fmaf(c.y, w[u][r][5], v);
+                v = fmaf(c.z, w[u][r][6], v);
+                v = fmaf(c.w, w[u][r][7], v);
+                s[r][k] = v;
+              }
+            }
           }
         }
       }

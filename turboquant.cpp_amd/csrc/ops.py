@@ -8,6 +8,7 @@ the compiled library, they raise.
 from __future__ import annotations
 
 import ctypes
+import dataclasses
 import math
 
 import torch
@@ -27,7 +28,8 @@ _c_int, _c_i64, _c_f32, _c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, c
 
 _SIGNATURES = {
     "tq_embed": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr],
-    "tq_add_rmsnorm": [_c_ptr, _c_ptr, _c_int, _c_i64, _c_ptr, _c_int, _c_f32, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr],
+    "tq_add_rmsnorm": [_c_ptr, _c_ptr, _c_int, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_f32,
+                       _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr],
     "tq_rope_kv_write": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
                          _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "tq_moe_combine": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
@@ -138,15 +140,45 @@ def embed(tokens: torch.Tensor, table: torch.Tensor, act) -> torch.Tensor:
     return x
 
 
-def add_rmsnorm(x: torch.Tensor, delta: torch.Tensor | None, weight: torch.Tensor, eps: float, act,
+@dataclasses.dataclass
+class GatheredSum:
+    """A part's output that nobody has summed yet:
+    ``out[t] = sum_j weights[t, j] * y[pair_slot[t, j]] + gate[t] * sum_s dense[s, t]`` (j ascending; ``dense``
+    and ``gate`` may be None).  The next norm adds it into the residual stream in the pass that normalises;
+    ``materialize`` gives it as a float32 [1, T, H] tensor to whoever needs it earlier."""
+    y: torch.Tensor                      # float32 [rows, H]
+    pair_slot: torch.Tensor              # int32 [T, k]
+    weights: torch.Tensor                # float32 [T, k]
+    dense: torch.Tensor | None = None    # float32 [S, T, H]
+    gate: torch.Tensor | None = None     # float32 [T]
+
+    def materialize(self, act) -> torch.Tensor:
+        return moe_combine(self.y, self.pair_slot, self.weights, self.dense, self.gate, act)
+
+
+def add_rmsnorm(x: torch.Tensor, delta, weight: torch.Tensor, eps: float, act,
                 rows: torch.Tensor | None = None, want_act: bool = True, want_f32: bool = False):
-    """x += sum_s delta[s] (in place, unless ``rows`` picks rows); returns rmsnorm(x) * weight as
-    (activation-typed or None, float32 or None), one row per entry of ``rows`` (all rows if None)."""
+    """x += delta (in place, unless ``rows`` picks rows), where delta is None, float32 partial sums [S, T, H] added
+    one after the other, or a GatheredSum; returns rmsnorm(x) * weight as (activation-typed or None, float32 or
+    None), one row per entry of ``rows`` (all rows if None)."""
     k = "add_rmsnorm"
     _check(x, k, "x", torch.float32)
     _need(x.dim() == 2, k, "x must be [T, H]")
     T, H = x.shape
     _check(weight, k, "weight", tuple(_WTYPE), (H,))
+    y = pair_slot = weights = gate = None
+    topk = 0
+    if isinstance(delta, GatheredSum):
+        y, pair_slot, weights, gate, delta = delta.y, delta.pair_slot, delta.weights, delta.gate, delta.dense
+        _check(y, k, "y", torch.float32)
+        _need(y.dim() == 2 and y.shape[1] == H, k, f"y must be [rows, {H}]")
+        _check(pair_slot, k, "pair_slot", torch.int32)
+        _need(pair_slot.dim() == 2 and pair_slot.shape[0] == T, k, f"pair_slot must be [{T}, k]")
+        topk = pair_slot.shape[1]
+        _need(1 <= topk <= 64, k, f"{topk} experts per token is beyond the 64 this kernel takes")
+        _check(weights, k, "weights", torch.float32, (T, topk))
+        if gate is not None:
+            _check(gate, k, "gate", torch.float32, (T,))
     S, stride = 0, 0
     if delta is not None:
         _check(delta, k, "delta", torch.float32)
@@ -160,8 +192,9 @@ def add_rmsnorm(x: torch.Tensor, delta: torch.Tensor | None, weight: torch.Tenso
     adt = ACT_DTYPES[dtype_name(act)]
     out = torch.empty((R, H), dtype=adt, device=x.device) if want_act else None
     out32 = torch.empty((R, H), dtype=torch.float32, device=x.device) if want_f32 else None
-    _run(k, library(act).tq_add_rmsnorm(_ptr(x), _ptr(delta), S, stride, _ptr(weight), _WTYPE[weight.dtype],
-                                        float(eps), _ptr(rows), R, _ptr(out), _ptr(out32), H, _stream()))
+    _run(k, library(act).tq_add_rmsnorm(_ptr(x), _ptr(delta), S, stride, _ptr(y), _ptr(pair_slot), _ptr(weights), topk,
+                                        _ptr(gate), _ptr(weight), _WTYPE[weight.dtype], float(eps), _ptr(rows), R,
+                                        _ptr(out), _ptr(out32), H, _stream()))
     return out, out32
 
 

@@ -18,7 +18,9 @@ Interfaces (``ctx`` is the :class:`~..engine.context.StepContext` of the running
 * block     ``forward(x, pending, ctx, entry) -> pending``: the arrangement of norms, mixer and ffn around
             the residual stream.
 
-``delta`` is always float32 [S, T, H]: S partial results that the next norm adds to the stream in order.
+``delta`` is float32 [S, T, H], S partial results that the next norm adds to the stream in order, or a
+``csrc.ops.GatheredSum``: a weighted sum over rows of a matrix (the experts' outputs) that is left to the next
+norm, whose ``materialize`` gives the tensor to an arrangement that needs it earlier.
 """
 from __future__ import annotations
 

@@ -82,7 +82,8 @@ class SparseMoE(Part):
                      tile_rows=unit, gather=False)
         if side is not None:
             ctx.join()
-        return ops.moe_combine(y, pair_slot, weights, shared, gate, ctx.act)
+        # the weighted sum over the chosen experts and the shared expert is left to the next norm
+        return ops.GatheredSum(y, pair_slot, weights, shared, gate)
 
     def _shared(self, normed, ctx):
         hs = ops.gemm(normed, self.shared_gate, ctx.act, w2=self.shared_up, out_act=True)
