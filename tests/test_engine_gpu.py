@@ -492,6 +492,126 @@ def test_a_mixer_with_state_of_its_own_is_registered_built_and_stepped():
         unregister_part("mixer", "toy_decay")
 
 
+def test_a_feed_forward_with_routing_and_another_position_encoding_defined_here():
+    """Two more parts defined in the test and registered from here: a feed-forward that sends each token to one of
+    four small experts (chosen by the largest of four router scores, relu inside), and a position encoding whose
+    angles grow linearly with the pair index and turn only half of each head, in interleaved pairs.  The library's
+    attention part takes the encoding by its table alone; layer 1 uses the library's own encoding and a window.
+    Whole prompts, token by token and a batch must agree with a plain loop."""
+    import plain_qwen2moe as P
+    from turboquant_cpp_amd.config import LayerSpec, ModelPlan, PartSpec, ScheduleEntry, Source
+    from turboquant_cpp_amd.engine.model import CausalLM
+    from turboquant_cpp_amd.engine.step import Engine
+    from turboquant_cpp_amd.parts import ParamSpec, Part, register_part, unregister_part
+    from turboquant_cpp_amd.weights import TensorDict
+
+    H, V, NH, NKV, HD, E, I, L = 40, 70, 4, 2, 16, 4, 24, 2
+    ROT, F0, F1 = 8, 0.9, 0.05
+
+    class ToyLinearAngles(Part):
+        pairing = "interleaved"
+        pairing_code = 1
+
+        def __init__(self, rotary_dim, first, last):
+            self.rotary_dim, self.first, self.last = rotary_dim, first, last
+
+        def table(self, device):
+            return torch.linspace(self.first, self.last, self.rotary_dim // 2, dtype=torch.float32).to(device)
+
+    class ToyOneOfFour(Part):
+        wants_f32 = False
+
+        def __init__(self, hidden_size, experts, inner_size):
+            self.hidden_size, self.experts, self.inner_size = hidden_size, experts, inner_size
+            self.router = self.w1 = self.w2 = None
+
+        def param_specs(self):
+            return {"router": ParamSpec((self.experts, self.hidden_size)),
+                    "w1": ParamSpec((self.experts, self.inner_size, self.hidden_size)),
+                    "w2": ParamSpec((self.experts, self.hidden_size, self.inner_size))}
+
+        def forward(self, normed, normed32, ctx):
+            x = normed.float()
+            pick = (x @ self.router.float().T).argmax(dim=-1)
+            h = torch.relu(torch.einsum("th,tih->ti", x, self.w1.float()[pick]))
+            return torch.einsum("ti,thi->th", h, self.w2.float()[pick]).unsqueeze(0)
+
+    register_part("position", "toy_linear")(ToyLinearAngles)
+    register_part("ffn", "toy_one_of_four")(ToyOneOfFour)
+    try:
+        def norm(name):
+            return PartSpec("rmsnorm", dict(size=H, eps=1e-6), {"weight": Source.single(name)})
+        positions = [PartSpec("toy_linear", dict(rotary_dim=ROT, first=F0, last=F1)),
+                     PartSpec("rope", dict(head_dim=HD, rotary_dim=HD, theta=100.0, pairing="half"))]
+        windows = [None, 5]
+        layers = [LayerSpec("prenorm", {
+            "mixer_norm": norm(f"l{l}.n1"), "ffn_norm": norm(f"l{l}.n2"),
+            "mixer": PartSpec("gqa_attention", dict(hidden_size=H, num_heads=NH, num_kv_heads=NKV, head_dim=HD,
+                                                    position=positions[l], window=windows[l]),
+                              {"qkv_weight": Source.concat([f"l{l}.q", f"l{l}.k", f"l{l}.v"]), "out_weight": Source.single(f"l{l}.o")}),
+            "ffn": PartSpec("toy_one_of_four", dict(hidden_size=H, experts=E, inner_size=I),
+                            {n: Source.single(f"l{l}.{n}") for n in ("router", "w1", "w2")})}) for l in range(L)]
+        plan = ModelPlan("ToyRoutedLM", V, H, layers, [ScheduleEntry(l) for l in range(L)], norm("final"),
+                         Source.single("embed"), None, max_positions=256)
+        model = CausalLM(plan, "float32")
+        g = torch.Generator().manual_seed(80)
+        tensors = {n: (torch.ones(s) if role == "scale" else 0.4 * torch.randn(s, generator=g))
+                   for n, (s, role) in model.tensor_table().items()}
+        model.load(TensorDict(tensors), DEV)
+        eng = Engine(model, max_tokens=64 * 6, max_slots=3)
+        assert eng.graphs is None          # parts that do not declare themselves safe for replay switch it off
+        assert len(eng.cache.groups) == 2  # the windowed layer has storage of its own
+
+        def turn(x, angles_per_step, pairing, rot):      # x [T, heads, hd]
+            T = x.shape[0]
+            ang = (torch.arange(T, dtype=torch.float32)[:, None] * angles_per_step[None, :]).double()
+            cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+            out = x.clone()
+            if pairing == "interleaved":
+                a, b = x[..., 0:rot:2], x[..., 1:rot:2]
+                out[..., 0:rot:2], out[..., 1:rot:2] = a * cos - b * sin, a * sin + b * cos
+            else:
+                a, b = x[..., :rot // 2], x[..., rot // 2:rot]
+                out[..., :rot // 2], out[..., rot // 2:rot] = a * cos - b * sin, a * sin + b * cos
+            return out
+
+        def plain(tokens):
+            t = {n: v.double() for n, v in tensors.items()}
+            x = t["embed"][tokens]
+            T = len(tokens)
+            tables = [torch.linspace(F0, F1, ROT // 2, dtype=torch.float32), torch.from_numpy(P.rope_frequencies(HD, 100.0))]
+            for l in range(L):
+                xb = P.rmsnorm(x, t[f"l{l}.n1"], 1e-6)
+                q = (xb @ t[f"l{l}.q"].T).view(T, NH, HD)
+                k = (xb @ t[f"l{l}.k"].T).view(T, NKV, HD)
+                v = (xb @ t[f"l{l}.v"].T).view(T, NKV, HD)
+                pairing, rot = ("interleaved", ROT) if l == 0 else ("half", HD)
+                q, k = turn(q, tables[l], pairing, rot), turn(k, tables[l], pairing, rot)
+                x = x + P.attention(q, k, v, window=windows[l]).reshape(T, NH * HD) @ t[f"l{l}.o"].T
+                xb = P.rmsnorm(x, t[f"l{l}.n2"], 1e-6)
+                pick = (xb @ t[f"l{l}.router"].T).argmax(dim=-1)
+                ys = [t[f"l{l}.w2"][e] @ torch.relu(t[f"l{l}.w1"][e] @ xb[i]) for i, e in enumerate(pick.tolist())]
+                x = x + torch.stack(ys)
+            return P.rmsnorm(x, t["final"], 1e-6) @ t["embed"].T
+
+        prompts = [torch.randint(0, V, (n,), generator=g).tolist() for n in (12, 3, 17)]
+        refs = [plain(p) for p in prompts]
+        slots = eng.open(3)
+        lg = eng.step(slots, prompts, [list(range(len(p))) for p in prompts]).cpu().double()
+        assert (lg - torch.cat(refs)).abs().max() < 2e-4
+        eng.close(slots)
+        slots = eng.open(2)                    # prefix, then token by token, in slots that were used before
+        eng.step(slots, [prompts[0][:5], prompts[2][:9]], [[], []])
+        for i in range(7):
+            lg = eng.step(slots, [[prompts[0][5 + i]], [prompts[2][9 + i]]]).cpu().double()
+            assert (lg[0] - refs[0][5 + i]).abs().max() < 2e-4 and (lg[1] - refs[2][9 + i]).abs().max() < 2e-4
+        eng.close(slots)
+        assert eng.cache.n_live == 0
+    finally:
+        unregister_part("position", "toy_linear")
+        unregister_part("ffn", "toy_one_of_four")
+
+
 def test_the_kernels_refuse_to_run_without_their_library(monkeypatch):
     """No silent fallback: if the compiled library cannot be found or built, the first kernel call raises."""
     from turboquant_cpp_amd.csrc import build, ops
