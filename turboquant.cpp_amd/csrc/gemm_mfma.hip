@@ -201,21 +201,29 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g)
   bf16_t* Ws = As + BM * TBK;
   bf16_t* Vs = Ws + TBN * TBK;
   // Which tile this workgroup takes.  Workgroups are dealt to the chip's 8 dies in turn (id % 8), and each die
-  // has its own L2: so the tiles are numbered such that one die gets a contiguous run of them, and a run goes
-  // through bands of 8 row tiles, down a band's column of row tiles first.  Workgroups that run at the same
-  // time on a die then share their tiles of `a` and of `w` in that die's L2.
+  // has its own L2: so the tiles are numbered such that one die gets a contiguous run of them.  One matrix: a
+  // run goes through bands of 8 row tiles, down a band's column of row tiles first, so that workgroups that run
+  // at the same time on a die share their tiles of `a` and of `w` in that die's L2.  A matrix per expert: a run
+  // goes row tile by row tile through all columns, so that an expert's matrix is read by one die (by two where
+  // a run ends), and only the row tiles in use are dealt.
   int tile_m, tile_n;
   {
-    const int gx = gridDim.x, gy = gridDim.y, total = gx * gy;
-    const int id = blockIdx.y * gx + blockIdx.x;
+    const int gx = g.tile_group && g.n_tiles ? min(g.n_tiles[0], (int)gridDim.x) : (int)gridDim.x;
+    const int gy = gridDim.y, total = gx * gy;
+    const int id = blockIdx.y * gridDim.x + blockIdx.x;
     const int die = id % 8, q = total / 8, rem = total % 8;
+    if (id / 8 >= q + (die < rem ? 1 : 0)) return;
     const int logical = die * q + min(die, rem) + id / 8;
-    const int band = logical / (8 * gy), in_band = logical % (8 * gy);
-    const int bh = min(8, gx - band * 8);
-    tile_m = band * 8 + in_band % bh;
-    tile_n = in_band / bh;
+    if (g.tile_group) {
+      tile_m = logical / gy;
+      tile_n = logical % gy;
+    } else {
+      const int band = logical / (8 * gy), in_band = logical % (8 * gy);
+      const int bh = min(8, gx - band * 8);
+      tile_m = band * 8 + in_band % bh;
+      tile_n = in_band / bh;
+    }
   }
-  if (g.n_tiles && tile_m >= g.n_tiles[0]) return;
   const int group = g.tile_group ? g.tile_group[tile_m] : 0;
   const bf16_t* w = g.w + (size_t)group * g.group_stride;
   const bf16_t* w2 = DUAL ? g.w2 + (size_t)group * g.group_stride : nullptr;
