@@ -91,7 +91,9 @@ def attention(q, k_pages, v_pages, layer_offset, positions, slot_of_token, block
 
 
 def gemm(a, w, act, bias=None, w2=None, out_act=False, a_rows=None, tile_group=None, n_tiles=None, tile_rows=None,
-         gather=True):
+         gather=True, partial_sums=False):
+    if partial_sums:
+        return gemm(a, w, act, bias=bias).unsqueeze(0)
     af = a.float()
     if tile_group is None:
         src = af if a_rows is None else af[a_rows.long()]

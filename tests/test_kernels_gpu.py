@@ -102,6 +102,24 @@ def test_gemm_dense(ops, act, M, N, K, mode):
 
 
 @pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("M,N,K,bias", [(300, 200, 2200, True), (129, 130, 4104, False), (70, 64, 1000, False), (9, 40, 4096, True)])
+def test_gemm_partial_sums(ops, act, M, N, K, bias):
+    """A product may come back as partial sums over runs of k ([S, M, N], the bias in the first); however many the
+    kernel makes, their sum is the product."""
+    a = rnd((M, K), adt(act), 14)
+    w = rnd((N, K), adt(act), 15, 0.2)
+    b = rnd((N,), adt(act), 16) if bias else None
+    y = ops.gemm(a.to(DEV), w.to(DEV), act, bias=None if b is None else b.to(DEV), partial_sums=True).cpu()
+    assert y.dim() == 3 and tuple(y.shape[1:]) == (M, N)
+    if act == "bfloat16":
+        assert y.shape[0] == (1 if M <= 64 or K < 2048 else (2 if K < 4096 else 4))
+    ref = ref_gemm(a, w, b, None)
+    scale = ref.abs().max().item()
+    err = (y.double().sum(0) - ref).abs().max().item()
+    assert err < (1e-5 * scale * math.sqrt(K) if act == "float32" else 4e-3 * scale), (err, scale)
+
+
+@pytest.mark.parametrize("act", ACTS)
 def test_gemm_float32_weights_on_the_bfloat16_path(ops, act):
     """A matrix the checkpoint stores in 32 bits stays so and still multiplies."""
     a = rnd((9, 72), adt(act), 20)

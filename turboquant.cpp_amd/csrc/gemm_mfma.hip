@@ -39,6 +39,8 @@ struct MfmaGemmArgs {
   void* out;
   int64_t ldc;
   int M, N, K;
+  int k_per;                // many rows only: k is split into runs of k_per, run z going to out + z * split_stride
+  int64_t split_stride;
 };
 
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
@@ -230,6 +232,13 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g)
   const int m0 = tile_m * BM, n0 = tile_n * TBN;
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int wm = wave / WN, wn = wave % WN;
+  // this workgroup's run of k: k_lo .. k_lo + Kl (all of k unless the product is split), and where its sums go
+  const int k_lo = blockIdx.z * g.k_per;
+  const int Kl = min(g.K, k_lo + g.k_per) - k_lo;
+  if (blockIdx.z) {
+    g.out = (float*)g.out + blockIdx.z * g.split_stride;
+    g.bias = nullptr;
+  }
 
   // What this thread fetches of each tile: chunk `ch` of row `row`.  Rows past the end of `a` or `w`, and rows
   // of padding in an expert's tile, read some valid row instead: an output depends on its own row of `a` and
@@ -243,15 +252,15 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g)
     const int m = min(m0 + row, g.M - 1);
     int src = m;
     if (g.a_rows && g.a_gather) src = max(g.a_rows[m], 0);
-    a_src[i] = g.a + (size_t)src * g.lda + ch * 8;
+    a_src[i] = g.a + (size_t)src * g.lda + k_lo + ch * 8;
     a_dst[i] = swz(row, ch);
   }
 #pragma unroll
   for (int i = 0; i < W_CH; ++i) {
     const int idx = tid + i * NT, row = idx / 8, ch = idx % 8;
     const int n = min(n0 + row, g.N - 1);
-    w_src[i] = w + (size_t)n * g.K + ch * 8;
-    v_src[i] = DUAL ? w2 + (size_t)n * g.K + ch * 8 : nullptr;
+    w_src[i] = w + (size_t)n * g.K + k_lo + ch * 8;
+    v_src[i] = DUAL ? w2 + (size_t)n * g.K + k_lo + ch * 8 : nullptr;
     w_dst[i] = swz(row, ch);
   }
   const int ch_of_thread = tid % 8;     // (tid + i * NT) % 8
@@ -274,7 +283,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g)
   // above are only ever indexed by constants and stay in registers.)
 #define TQ_FETCH(k0)                                                                                          \
   do {                                                                                                        \
-    if ((k0) + TBK <= g.K) {                                                                                  \
+    if ((k0) + TBK <= Kl) {                                                                                   \
       _Pragma("unroll") for (int i = 0; i < A_CH; ++i)                                                        \
           pa[i] = *reinterpret_cast<const u32x4*>(a_src[i] + (k0));                                           \
       _Pragma("unroll") for (int i = 0; i < W_CH; ++i) {                                                      \
@@ -282,7 +291,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g)
         if (DUAL) pv[i] = *reinterpret_cast<const u32x4*>(v_src[i] + (k0));                                   \
       }                                                                                                       \
     } else {                                                                                                  \
-      const bool k_ok = (k0) + ch_of_thread * 8 < g.K;                                                        \
+      const bool k_ok = (k0) + ch_of_thread * 8 < Kl;                                                         \
       _Pragma("unroll") for (int i = 0; i < A_CH; ++i)                                                        \
           pa[i] = k_ok ? *reinterpret_cast<const u32x4*>(a_src[i] + (k0)) : z;                                \
       _Pragma("unroll") for (int i = 0; i < W_CH; ++i) {                                                      \
@@ -304,14 +313,14 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g)
   // t + 2 is on its way from memory into registers: one barrier per step of 64 of k.
   TQ_FETCH(0);
   TQ_STAGE(0);
-  if (TBK < g.K) TQ_FETCH(TBK);
+  if (TBK < Kl) TQ_FETCH(TBK);
   __syncthreads();
   const int lr = lane % 32, lc = lane / 32;
   int cur = 0;
-  for (int k0 = 0; k0 < g.K; k0 += TBK, cur ^= BUF) {
-    if (k0 + TBK < g.K) {
+  for (int k0 = 0; k0 < Kl; k0 += TBK, cur ^= BUF) {
+    if (k0 + TBK < Kl) {
       TQ_STAGE(cur ^ BUF);
-      if (k0 + 2 * TBK < g.K) TQ_FETCH(k0 + 2 * TBK);
+      if (k0 + 2 * TBK < Kl) TQ_FETCH(k0 + 2 * TBK);
     }
     const bf16_t* Ac = As + cur;
     const bf16_t* Wc = Ws + cur;
@@ -392,8 +401,8 @@ static int launch_stream(const MfmaGemmArgs& g, bool dual, bool out_act, int row
 }
 
 template <int BM, int WM, int WN>
-static int launch_tile(const MfmaGemmArgs& g, bool dual, bool out_act, hipStream_t st) {
-  const dim3 grid((g.M + BM - 1) / BM, (g.N + TBN - 1) / TBN);
+static int launch_tile(const MfmaGemmArgs& g, bool dual, bool out_act, int splits, hipStream_t st) {
+  const dim3 grid((g.M + BM - 1) / BM, (g.N + TBN - 1) / TBN, splits);
   const size_t shmem = (size_t)2 * (BM + TBN * (dual ? 2 : 1)) * TBK * sizeof(bf16_t);
 #define TQ_TILE(D, O)                                                                                  \
   do {                                                                                                 \
@@ -414,18 +423,34 @@ static int launch_tile(const MfmaGemmArgs& g, bool dual, bool out_act, hipStream
   return 0;
 }
 
+// Into how many runs of k a plain product of M rows may be split when its partial sums are wanted apart: a
+// product of many rows whose tiles do not fill the chip twice, and that has k enough, goes faster in 2 to 4 runs,
+// each at least 1024 long.  1 for few rows, which take the streaming kernel.
+TQ_API int tq_gemm_mfma_splits(int M, int N, int K) {
+  if (M <= 64) return 1;
+  const int64_t tiles = (int64_t)((M + 127) / 128) * ((N + TBN - 1) / TBN);
+  int s = 1;
+  while (s < 4 && tiles * s < 512 && K / (s * 2) >= 1024) s *= 2;
+  return s;
+}
+
 // a: bfloat16 [.., K] with row stride lda (a multiple of 8, as K must be); w, w2: bfloat16.
 // tile_rows: with tile_group set, the padding unit of the row order (16 or 64); else a hint that is ignored.
+// splits > 1 (as tq_gemm_mfma_splits says, for a plain product into float): run z of k goes to out + z * M * ldc,
+// the bias to run 0; the sum over the runs is the caller's.
 TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gather, const void* w, const void* w2,
                         int64_t group_stride, const int* tile_group, const int* n_tiles, const void* bias,
                         int bias_type, void* out, int64_t ldc, int out_is_act, int M, int N, int K, int tile_rows,
-                        hipStream_t st) {
+                        int splits, hipStream_t st) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || K % 8 != 0 || lda % 8 != 0) return TQ_ERR_BAD_ARG;
   if (((uintptr_t)a | (uintptr_t)w | (uintptr_t)w2) % 16 != 0 || (group_stride % 8) != 0) return TQ_ERR_BAD_ARG;
-  MfmaGemmArgs g{(const bf16_t*)a, lda, a_rows, a_gather, (const bf16_t*)w, (const bf16_t*)w2, group_stride,
-                 tile_group, n_tiles, bias, bias_type, out, ldc, M, N, K};
   const bool dual = w2 != nullptr, out_act = out_is_act != 0;
+  if (splits < 1 || splits > 64) return TQ_ERR_BAD_ARG;
+  if (splits > 1 && (dual || out_act || tile_group || a_rows || splits != tq_gemm_mfma_splits(M, N, K))) return TQ_ERR_BAD_ARG;
+  const int k_per = ((K + TBK - 1) / TBK + splits - 1) / splits * TBK;
+  MfmaGemmArgs g{(const bf16_t*)a, lda, a_rows, a_gather, (const bf16_t*)w, (const bf16_t*)w2, group_stride,
+                 tile_group, n_tiles, bias, bias_type, out, ldc, M, N, K, splits > 1 ? k_per : K, (int64_t)M * ldc};
   int rc = 0;
   if (tile_group) {
     if (tile_rows == 16) {
@@ -433,7 +458,7 @@ TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gat
       rc = launch_stream<1>(g, dual, out_act, M / 16, st);
     } else if (tile_rows == 64) {
       if ((N + TBN - 1) / TBN > 65535) return TQ_ERR_UNSUPPORTED;
-      rc = launch_tile<64, 2, 4>(g, dual, out_act, st);
+      rc = launch_tile<64, 2, 4>(g, dual, out_act, 1, st);
     } else {
       return TQ_ERR_BAD_ARG;
     }
@@ -445,7 +470,8 @@ TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gat
     rc = launch_stream<4>(g, dual, out_act, 1, st);
   } else {
     if ((N + TBN - 1) / TBN > 65535) return TQ_ERR_UNSUPPORTED;
-    rc = M <= 64 * 16 && !dual ? launch_tile<64, 2, 4>(g, dual, out_act, st) : launch_tile<128, 4, 2>(g, dual, out_act, st);
+    rc = M <= 64 * 16 && !dual ? launch_tile<64, 2, 4>(g, dual, out_act, splits, st)
+                               : launch_tile<128, 4, 2>(g, dual, out_act, splits, st);
   }
   if (rc) return rc;
   TQ_LAUNCH_CHECK();

@@ -47,7 +47,8 @@ _SIGNATURES = {
 # entry points that only the bfloat16 library has
 _OPTIONAL = {
     "tq_gemm_mfma": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int,
-                     _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+                     _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "tq_gemm_mfma_splits": [_c_int, _c_int, _c_int],
     "tq_attention_mfma": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int,
                           _c_int, _c_int, _c_int, _c_f32, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
 }
@@ -262,13 +263,16 @@ def _use_mfma(act, a: torch.Tensor, w: torch.Tensor, K: int) -> bool:
 
 def gemm(a: torch.Tensor, w: torch.Tensor, act, bias: torch.Tensor | None = None, w2: torch.Tensor | None = None,
          out_act: bool = False, a_rows: torch.Tensor | None = None, tile_group: torch.Tensor | None = None,
-         n_tiles: torch.Tensor | None = None, tile_rows: int | None = None, gather: bool = True) -> torch.Tensor:
+         n_tiles: torch.Tensor | None = None, tile_rows: int | None = None, gather: bool = True,
+         partial_sums: bool = False) -> torch.Tensor:
     """out[m, n] = sum_k a[row(m), k] * w[g, n, k]  (+ bias[n]);  with ``w2``: silu(a w^T) * (a w2^T).
 
     ``a`` [M, K] activations.  ``w`` [N, K], or [G, N, K] with ``tile_group`` naming the matrix of each tile of
     ``tile_rows`` output rows and ``a_rows`` [P] the row of ``a`` behind each output row (-1: none; with
     ``gather`` false a live output row m reads row m of ``a``).
     Output is float32 unless ``out_act``.  Sums run over k in ascending order whatever M is.
+    ``partial_sums`` (plain products into float32 only): the result is [S, M, N], S >= 1 partial sums over runs of
+    k that the caller adds up in order, as the next norm does with a part's output; the kernel chooses S.
     """
     k = "gemm"
     adt = ACT_DTYPES[dtype_name(act)]
@@ -301,14 +305,20 @@ def gemm(a: torch.Tensor, w: torch.Tensor, act, bias: torch.Tensor | None = None
         _check(w2, k, "w2", w.dtype, tuple(w.shape))
     if bias is not None:
         _check(bias, k, "bias", tuple(_WTYPE), (N,))
-    out = torch.empty((M, N), dtype=adt if out_act else torch.float32, device=a.device)
+    if partial_sums:
+        _need(w2 is None and not out_act and not grouped and a_rows is None, k,
+              "partial sums are for plain products into float32")
     lib = library(act)
     if _use_mfma(act, a, w, K) and (bias is None or bias.dtype in _WTYPE):
+        splits = lib.tq_gemm_mfma_splits(M, N, K) if partial_sums else 1
+        out = torch.empty((splits, M, N) if partial_sums else (M, N), dtype=adt if out_act else torch.float32,
+                          device=a.device)
         _run("gemm_mfma", lib.tq_gemm_mfma(_ptr(a), a.stride(0), _ptr(a_rows), int(gather), _ptr(w), _ptr(w2), gstride,
                                            _ptr(tile_group), _ptr(n_tiles), _ptr(bias),
                                            _WTYPE[bias.dtype] if bias is not None else 0, _ptr(out), N, int(out_act),
-                                           M, N, K, tile_rows, _stream()))
+                                           M, N, K, tile_rows, splits, _stream()))
         return out
+    out = torch.empty((1, M, N) if partial_sums else (M, N), dtype=adt if out_act else torch.float32, device=a.device)
     _run(k, lib.tq_gemm_generic(_ptr(a), a.stride(0), _ptr(a_rows), int(gather), _ptr(w), _ptr(w2), _WTYPE[w.dtype], gstride,
                                 _ptr(tile_group), _ptr(n_tiles), _ptr(bias),
                                 _WTYPE[bias.dtype] if bias is not None else 0, _ptr(out), N, int(out_act), M, N, K,

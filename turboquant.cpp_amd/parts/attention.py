@@ -73,4 +73,4 @@ class GroupedQueryAttention(Part):
         o = ops.attention(q, kv.k_pages, kv.v_pages, kv.layer_offset, b.positions, b.slot_of_token, kv.table,
                           kv.page_size, kv.page_stride, self.num_heads, self.num_kv_heads, self.head_dim,
                           self.window, self.scale, ctx.act, runs=b.runs())
-        return ops.gemm(o, self.out_weight, ctx.act).unsqueeze(0)
+        return ops.gemm(o, self.out_weight, ctx.act, partial_sums=True)

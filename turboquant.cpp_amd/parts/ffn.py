@@ -31,7 +31,7 @@ class DenseSwiGLU(Part):
 
     def forward(self, normed, normed32, ctx):
         h = ops.gemm(normed, self.gate, ctx.act, w2=self.up, out_act=True)
-        return ops.gemm(h, self.down, ctx.act).unsqueeze(0)
+        return ops.gemm(h, self.down, ctx.act, partial_sums=True)
 
 
 @register_part("ffn", "moe_swiglu")
@@ -87,4 +87,4 @@ class SparseMoE(Part):
 
     def _shared(self, normed, ctx):
         hs = ops.gemm(normed, self.shared_gate, ctx.act, w2=self.shared_up, out_act=True)
-        return ops.gemm(hs, self.shared_down, ctx.act).unsqueeze(0)
+        return ops.gemm(hs, self.shared_down, ctx.act, partial_sums=True)
