@@ -396,6 +396,57 @@ def test_attention_finds_a_far_key(ops, act):
     assert (out_w2.float().view(nh, hd) - v[far].to(adt(act)).float()).abs().max() < 1e-2
 
 
+@pytest.mark.parametrize("window", [None, 3000])
+def test_decoding_over_long_caches(ops, window):
+    """One token per sequence at positions on both sides of every length at which the split kernel changes the
+    length of its runs (2048, 4096, 6144) and well beyond, in one batch; in each sequence one far key stands out a
+    little, so that a run that is skipped or joined twice shows.  Against the plain formula for the last token."""
+    act = "bfloat16"
+    nh, nkv, hd, page = 6, 2, 64, 64
+    lens = [2047, 2048, 2049, 4095, 4097, 6143, 6145, 9001, 130]
+    table, slots, page_stride, kp, vp = paged_setup(lens, page, nkv, hd, 1, act, 95)
+    scale = 1.0 / math.sqrt(hd)
+    g = torch.Generator().manual_seed(96)
+    qs, want = [], []
+    kp3, vp3 = kp.view(-1, nkv, page, hd), vp.view(-1, nkv, hd, page)          # [page][kv head][row][hd], values transposed
+    for i, n in enumerate(lens):
+        q = torch.randn((nh, hd), generator=g).to(adt(act))
+        k = (0.5 * torch.randn((n, nkv, hd), generator=g)).to(adt(act))
+        v = torch.randn((n, nkv, hd), generator=g).to(adt(act))
+        far = (n * 37) // 100
+        k[far] = (q.float().view(nkv, nh // nkv, hd)[:, 0] * 0.6).to(adt(act))     # a score that stands out
+        pos = torch.arange(n)
+        pages = table[slots[i], (pos // page).long()].long()
+        kp3[pages, :, pos % page, :] = k
+        vp3[pages, :, :, pos % page] = v
+        lo = 0 if window is None or n <= window else n - window
+        kk, vv = k.double()[lo:], v.double()[lo:]
+        out = torch.empty((nh, hd), dtype=torch.float64)
+        for h in range(nh):
+            kvh = h // (nh // nkv)
+            pr = torch.softmax((kk[:, kvh] @ q[h].double()) * scale, dim=0)
+            out[h] = pr @ vv[:, kvh]
+        qs.append(q)
+        want.append(out.reshape(-1))
+    B = len(lens)
+    positions = torch.tensor([n - 1 for n in lens], dtype=torch.int32)
+    runs = {"cu_seqlens": torch.arange(B + 1, dtype=torch.int32).to(DEV), "slots": torch.tensor(slots, dtype=torch.int32).to(DEV),
+            "start": positions.to(DEV), "max_new": 1, "max_end": max(lens), "decode": True}
+    out = ops.attention(torch.stack(qs).reshape(B, nh * hd).to(DEV), kp.to(DEV), vp.to(DEV), 0, positions.to(DEV),
+                        torch.tensor(slots, dtype=torch.int32).to(DEV), table.to(DEV), page, page_stride, nh, nkv, hd,
+                        window, scale, act, runs=runs).cpu()
+    err = (out.double() - torch.stack(want)).abs().max(dim=1).values
+    assert err.max() < 2e-2, err
+    # each sequence alone gives the same bits: what a run is depends on the token's position only
+    for i in (1, 4, 7):
+        runs1 = {"cu_seqlens": torch.tensor([0, 1], dtype=torch.int32).to(DEV), "slots": torch.tensor([slots[i]], dtype=torch.int32).to(DEV),
+                 "start": positions[i:i + 1].to(DEV), "max_new": 1, "max_end": lens[i], "decode": True}
+        alone = ops.attention(qs[i].reshape(1, nh * hd).to(DEV), kp.to(DEV), vp.to(DEV), 0, positions[i:i + 1].to(DEV),
+                              torch.tensor([slots[i]], dtype=torch.int32).to(DEV), table.to(DEV), page, page_stride, nh, nkv,
+                              hd, window, scale, act, runs=runs1).cpu()
+        assert torch.equal(alone[0], out[i])
+
+
 # ------------------------------------------------------------------------------------------------ sampling
 @pytest.mark.parametrize("V", [10, 1000, 151937])
 def test_argmax_first_maximum(ops, V):

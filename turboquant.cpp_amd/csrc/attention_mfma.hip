@@ -17,8 +17,8 @@
 //
 // Two entry points share this: whole prompts (columns = 16 consecutive tokens of a sequence, one head; four
 // waves per workgroup) and decoding (columns = the query heads that share one kv head, one token; the cache is
-// split into runs of SPLIT tiles, one wave each, and a second kernel joins the runs in order).  Tiles start at
-// multiples of 64 positions and runs at multiples of SPLIT tiles, so the order of every sum depends only on
+// split into runs of 1 to 4 tiles, one wave each, and a second kernel joins the runs in order).  Tiles start at
+// multiples of 64 positions and runs at multiples of the run length, so the order of every sum depends only on
 // the token's own position.
 #include "common.h"
 
@@ -27,7 +27,16 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define TILE 64
 #define LOG2E 1.4426950408889634f
-#define SPLIT 4          // tiles per run when decoding: 256 positions
+// Tiles per run when decoding a token at position p: short sequences are cut finer, so that a small batch still
+// gives the chip hundreds of waves; a function of the token's own position only.
+__host__ __device__ __forceinline__ int tiles_per_run(int p) { return p >= 3 * 2048 ? 4 : p / 2048 + 1; }
+// Most runs that a token at a position below max_end can have.
+static int most_runs(int max_end) {
+  const int tiles = (max_end + 63) / 64;
+  const int short_runs = tiles < 32 ? tiles : 32;          // below position 6144 no token has more than 32
+  const int long_runs = (tiles + 3) / 4;
+  return short_runs > long_runs ? short_runs : long_runs;
+}
 
 struct AttnArgs {
   const bf16_t* q;              // [T][nh][hd]
@@ -339,7 +348,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 
 // ------------------------------------------------------------------------------------------ decoding
 // One new token per sequence at position start[b].  grid (max_runs, nkv * ceil(g / 16), B), block 64: the wave
-// takes run x (tiles SPLIT x .. SPLIT x + SPLIT - 1) for up to 16 of the g = nh / nkv heads of one kv head and
+// takes run x (tiles S x .. S x + S - 1, S = tiles_per_run(position)) for up to 16 of the g = nh / nkv heads of one kv head and
 // writes their unnormalised sums with maximum and denominator.
 template <int DT, bool EXACT>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DT > 8 ? 2 : 3))) void attn_decode_kernel(AttnArgs a) {
@@ -349,7 +358,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DT > 8 ? 2 :
   const int lane = threadIdx.x, r = lane % 16, c = lane / 16;
   const int p = a.start[b];
   const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
-  const int tile_beg = max(run * SPLIT, lo / TILE), tile_end = min((run + 1) * SPLIT, p / TILE + 1);
+  const int S = tiles_per_run(p);
+  const int tile_beg = max(run * S, lo / TILE), tile_end = min((run + 1) * S, p / TILE + 1);
   if (tile_beg >= tile_end) return;
   const int hg = cg * 16 + r;                 // head within the group
   const bool valid = hg < g;
@@ -390,7 +400,8 @@ __global__ __launch_bounds__(64) void attn_join_kernel(AttnArgs a) {
   const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
   const int p = a.start[b];
   const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
-  const int run_beg = lo / TILE / SPLIT, run_end = p / TILE / SPLIT + 1;
+  const int S = tiles_per_run(p);
+  const int run_beg = lo / TILE / S, run_end = p / TILE / S + 1;
   const int stride = a.hd + 2;
   const float* part = a.partial + ((size_t)b * a.nh + h) * a.max_runs * stride;
   float m = -INFINITY;
@@ -438,8 +449,7 @@ static void launch_decode(const AttnArgs& a, int B, hipStream_t st) {
 
 // Number of floats of `partial` that decoding B sequences up to position max_end needs.
 TQ_API int64_t tq_attention_decode_scratch(int B, int nh, int hd, int max_end) {
-  const int max_runs = (max_end + TILE * SPLIT - 1) / (TILE * SPLIT);
-  return (int64_t)B * nh * max_runs * (hd + 2);
+  return (int64_t)B * nh * most_runs(max_end) * (hd + 2);
 }
 
 // decode != 0: every sequence brings exactly one token.  max_new: longest run of new tokens of a sequence;
@@ -452,10 +462,10 @@ TQ_API int tq_attention_mfma(const void* q, const void* k_pool, const void* v_po
   if (hd % 16 != 0 || hd < 16 || hd > 256 || page_size % TILE != 0 || nkv <= 0 || nh % nkv != 0)
     return TQ_ERR_UNSUPPORTED;
   if (nh > 65535 || B > 65535 || page_stride % 8 != 0 || !(scale > 0.f)) return TQ_ERR_UNSUPPORTED;
-  if (decode && (max_end + TILE * SPLIT - 1) / (TILE * SPLIT) > MAX_RUNS_LDS) return TQ_ERR_UNSUPPORTED;
+  if (decode && most_runs(max_end) > MAX_RUNS_LDS) return TQ_ERR_UNSUPPORTED;
   AttnArgs a{(const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, bt_stride, cu_seqlens, slots,
              start, page_size, page_stride, nh, nkv, hd, window, scale, (bf16_t*)out, partial,
-             (max_end + TILE * SPLIT - 1) / (TILE * SPLIT)};
+             most_runs(max_end)};
   const int dt = hd / 16;
   // head sizes 64, 128 and 256 have kernels of their own in which nothing depends on hd at run time
   if (decode) {

@@ -49,6 +49,7 @@ _OPTIONAL = {
     "tq_gemm_mfma": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int,
                      _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "tq_gemm_mfma_splits": [_c_int, _c_int, _c_int],
+    "tq_attention_decode_scratch": [_c_int, _c_int, _c_int, _c_int],
     "tq_attention_mfma": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int,
                           _c_int, _c_int, _c_int, _c_f32, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
 }
@@ -87,6 +88,8 @@ def library(dtype) -> ctypes.CDLL:
         if hasattr(lib, fn):
             f = getattr(lib, fn)
             f.argtypes, f.restype = sig, _c_int
+    if hasattr(lib, "tq_attention_decode_scratch"):
+        lib.tq_attention_decode_scratch.restype = _c_i64
     _LIBS[name] = lib
     return lib
 
@@ -363,8 +366,8 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, lay
         partial = None
         if runs["decode"]:
             _need(T == B, k, "decoding brings one token per sequence")
-            n_runs = -(-runs["max_end"] // 256)
-            partial = torch.empty((B * num_heads * n_runs * (head_dim + 2),), dtype=torch.float32, device=q.device)
+            partial = torch.empty((lib.tq_attention_decode_scratch(B, num_heads, head_dim, int(runs["max_end"])),),
+                                  dtype=torch.float32, device=q.device)
         _run("attention_mfma", lib.tq_attention_mfma(
             _ptr(q), k_pages.data_ptr() + layer_offset * esz, v_pages.data_ptr() + layer_offset * esz,
             _ptr(block_table), block_table.shape[1], _ptr(runs["cu_seqlens"]), _ptr(runs["slots"]), _ptr(runs["start"]),

@@ -101,8 +101,10 @@ class Engine:
                     torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
         if logits is None:
             batch = pack_step(slots, starts, token_lists, wants, self.device)
+            # a second stream pays when kernels are short; a long prompt's products fill the chip one at a time
+            few = sum(len(t) for t in token_lists) <= 256
             ctx = StepContext(batch=batch, cache=self.cache, act=self.model.act, device=self.device,
-                              side_stream=self.side_stream)
+                              side_stream=self.side_stream if few else None)
             logits = self.model.forward(ctx)
         for slot in slots:
             self.cache.commit(slot)
