@@ -32,6 +32,25 @@ TQ_API int tq_embed(const int* tokens, const void* table, int wtype, float* x, i
 //   the experts' outputs that nobody has summed yet, as moe_combine below would:
 //   d = sum_j weights[row][j] * y[pair_slot[row][j]] (j ascending) + gate[row] * sum_s delta[s][row].
 // The sum of squares is taken in a fixed order that does not depend on the number of rows.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ f32x4 load4f(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
+__device__ __forceinline__ f32x4 load4f(const bf16_t* p) {
+  const uint2 u = *reinterpret_cast<const uint2*>(p);
+  return f32x4{__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+               __uint_as_float(u.y & 0xffff0000u)};
+}
+__device__ __forceinline__ void store4(float* p, f32x4 v) { *reinterpret_cast<f32x4*>(p) = v; }
+__device__ __forceinline__ void store4(bf16_t* p, f32x4 v) {
+  uint2 u;
+  u.x = (uint32_t)f32_to_bf16(v.x).bits | ((uint32_t)f32_to_bf16(v.y).bits << 16);
+  u.y = (uint32_t)f32_to_bf16(v.z).bits | ((uint32_t)f32_to_bf16(v.w).bits << 16);
+  *reinterpret_cast<uint2*>(p) = u;
+}
+
+// A thread takes four consecutive elements at a time when H is a multiple of four (every load is 16 bytes and
+// all of a thread's loads can be on their way at once), else one element at a time; what is computed per
+// element is the same.
 template <class W>
 __global__ void add_rmsnorm_kernel(float* __restrict__ x, const float* __restrict__ delta, int S,
                                    size_t delta_stride, const float* __restrict__ y,
@@ -39,13 +58,14 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const float* __restric
                                    const float* __restrict__ gate, const W* __restrict__ w, float eps,
                                    const int* __restrict__ rows, act_t* __restrict__ out,
                                    float* __restrict__ out32, int H) {
-  extern __shared__ float v[];       // H floats, then one float per wave
+  extern __shared__ __attribute__((aligned(16))) float v[];       // H floats, then one float per wave
   __shared__ int slot[64];
   __shared__ float wgt[64];
-  float* red = v + H;
+  float* red = v + (H + 3) / 4 * 4;
   const int r = blockIdx.x;
   const int row = rows ? rows[r] : r;
   float* xr = x + (size_t)row * H;
+  const float* dr = delta + (size_t)row * H;
   float g = 1.0f;
   if (y) {
     if (threadIdx.x < topk) {      // the token's rows and weights once, not once per element
@@ -55,32 +75,67 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const float* __restric
     if (gate) g = gate[row];
     __syncthreads();
   }
+  const bool vec = H % 4 == 0;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) {
-    float a = xr[i];
-    if (y) {
-      float acc = 0.f;
-      for (int j = 0; j < topk; ++j) acc += wgt[j] * y[(size_t)slot[j] * H + i];
-      if (S > 0) {
-        float sh = 0.f;
-        for (int s = 0; s < S; ++s) sh += delta[s * delta_stride + (size_t)row * H + i];
-        acc += g * sh;
+  if (vec) {
+#pragma unroll 2
+    for (int i = threadIdx.x * 4; i < H; i += blockDim.x * 4) {
+      f32x4 a = load4f(xr + i);
+      if (y) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < topk; ++j) acc += wgt[j] * load4f(y + (size_t)slot[j] * H + i);
+        if (S > 0) {
+          f32x4 sh = {0.f, 0.f, 0.f, 0.f};
+          for (int s = 0; s < S; ++s) sh += load4f(dr + s * delta_stride + i);
+          acc += g * sh;
+        }
+        a += acc;
+      } else {
+        for (int s = 0; s < S; ++s) a += load4f(dr + s * delta_stride + i);
       }
-      a += acc;
-    } else {
-      for (int s = 0; s < S; ++s) a += delta[s * delta_stride + (size_t)row * H + i];
+      store4(v + i, a);
+      if (!rows) store4(xr + i, a);
+      ss += a.x * a.x;
+      ss += a.y * a.y;
+      ss += a.z * a.z;
+      ss += a.w * a.w;
     }
-    v[i] = a;
-    if (!rows) xr[i] = a;
-    ss += a * a;
+  } else {
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+      float a = xr[i];
+      if (y) {
+        float acc = 0.f;
+        for (int j = 0; j < topk; ++j) acc += wgt[j] * y[(size_t)slot[j] * H + i];
+        if (S > 0) {
+          float sh = 0.f;
+          for (int s = 0; s < S; ++s) sh += dr[s * delta_stride + i];
+          acc += g * sh;
+        }
+        a += acc;
+      } else {
+        for (int s = 0; s < S; ++s) a += dr[s * delta_stride + i];
+      }
+      v[i] = a;
+      if (!rows) xr[i] = a;
+      ss += a * a;
+    }
   }
   ss = block_sum(ss, red);
   ss = ss / (float)H + eps;
   const float rs = 1.0f / sqrtf(ss);
-  for (int i = threadIdx.x; i < H; i += blockDim.x) {
-    const float o = v[i] * rs * to_f32(w[i]);
-    if (out) out[(size_t)r * H + i] = from_f32<act_t>(o);
-    if (out32) out32[(size_t)r * H + i] = o;
+  if (vec) {
+#pragma unroll 2
+    for (int i = threadIdx.x * 4; i < H; i += blockDim.x * 4) {
+      const f32x4 o = load4f(v + i) * rs * load4f(w + i);
+      if (out) store4(out + (size_t)r * H + i, o);
+      if (out32) store4(out32 + (size_t)r * H + i, o);
+    }
+  } else {
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+      const float o = v[i] * rs * to_f32(w[i]);
+      if (out) out[(size_t)r * H + i] = from_f32<act_t>(o);
+      if (out32) out32[(size_t)r * H + i] = o;
+    }
   }
 }
 
@@ -91,7 +146,7 @@ TQ_API int tq_add_rmsnorm(float* x, const float* delta, int S, int64_t delta_str
   if (R <= 0) return 0;
   if (y && (topk < 1 || topk > 64 || !pair_slot || !weights)) return TQ_ERR_BAD_ARG;
   const int threads = 256;
-  const size_t shmem = (size_t)(H + threads / TQ_WAVE) * sizeof(float);
+  const size_t shmem = (size_t)((H + 3) / 4 * 4 + threads / TQ_WAVE) * sizeof(float);
   if (shmem > 150 * 1024) return TQ_ERR_UNSUPPORTED;
   TQ_DISPATCH_W(wtype, {
     if (shmem > 48 * 1024)
