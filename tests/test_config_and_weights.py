@@ -66,6 +66,8 @@ def test_a_size_or_constant_that_is_missing_is_an_error_not_a_default(key):
     ({"head_dim": 15}, "even"),
     ({"architectures": ["LlamaForCausalLM"]}, "unknown architecture"),
     ({"architectures": []}, "architectures"),
+    ({"rope_scaling": {"type": "yarn", "factor": 4.0}}, "rope_scaling"),
+    ({"hidden_act": "gelu"}, "hidden_act"),
 ])
 def test_inconsistent_configurations_are_refused(change, word):
     d = copy.deepcopy(TINY_A)

@@ -75,6 +75,9 @@ def config_from_json(data: dict) -> Qwen2MoeConfig:
         head_dim = hidden // heads
     use_window = r.boolean("use_sliding_window", False)
     window = r.optional_integer("sliding_window")
+    # options that would change the formulas and that this architecture's plan does not carry out
+    require(data.get("rope_scaling") is None, f"rope_scaling {data.get('rope_scaling')!r} is not implemented")
+    require(data.get("hidden_act", "silu") == "silu", f"hidden_act {data.get('hidden_act')!r} is not implemented (silu is)")
     layers = r.integer("num_hidden_layers", minimum=1)
     stop: list[int] = []
     for key in ("eos_token_id",):
