@@ -185,7 +185,7 @@ def main() -> int:
             s, _, _ = run_decode(b, args.points_context, 32, 4)
             points[f"decode_b{b}"] = round(b / s, 1)
     out = {
-        "metric": "decode tok/s at batch 8, context 8192 (Qwen1.5-MoE-A2.7B layer sizes, random weights)",
+        "metric": f"decode tok/s at batch {args.batch}, context {args.context} (Qwen1.5-MoE-A2.7B layer sizes, random weights)",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": short, "data": "synthetic",
