@@ -11,8 +11,9 @@ blocks on demand with create / append / seq_len / free calls and status checks
   Slots are opened when a batch starts, closed when its sequence ends, and handed out again.
 * Keys and values live in *pages* of ``page_size`` positions.  Layers whose needs agree (kv heads,
   head size, window) form a *group* with storage of its own: one pool of pages, each page holding the
-  rows of all the group's layers for ``page_size`` positions of one sequence, laid out
-  ``[layer][kv head][row][head_dim]``.  A group that keeps a window gives back the pages that have
+  rows of all the group's layers for ``page_size`` positions of one sequence: keys laid out
+  ``[layer][kv head][row][head_dim]``, values transposed, ``[layer][kv head][head_dim][row]`` (both as the
+  attention kernels' operands want them).  A group that keeps a window gives back the pages that have
   fallen out of every later token's window, so its sequences hold pages for the window only.
 * The page table of a group, ``[slot][logical page] -> page`` (-1: none), lives on the device and is
   updated only when pages change hands; kernels find a token's rows through its slot.
