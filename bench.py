@@ -126,18 +126,18 @@ def main() -> int:
 
         # the first warm-up step (which runs eagerly) also counts the distinct experts that each layer's router picks
         picked = []
-        router_topk = ops.router_topk
+        route = ops.route
 
-        def counting_router(*a, **k):
-            out = router_topk(*a, **k)
+        def counting_route(*a, **k):
+            out = route(*a, **k)
             picked.append(int(torch.unique(out[0]).numel()))
             return out
 
-        ops.router_topk = counting_router
+        ops.route = counting_route
         try:
             tokens = one_step(tokens)
         finally:
-            ops.router_topk = router_topk
+            ops.route = route
         experts_used = sum(picked) / max(len(picked), 1)
         for _ in range(warmup - 1):
             tokens = one_step(tokens)

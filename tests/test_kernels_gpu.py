@@ -257,6 +257,27 @@ def test_router_random(ops, act, E, k, H, renorm):
     assert (gate.cpu().double() - torch.sigmoid(x.double() @ sg.double()[0])).abs().max() < 1e-5
 
 
+@pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("E,k,H,renorm,shared", [(5, 5, 72, True, True), (60, 4, 2048, False, True), (130, 8, 70, True, False)])
+def test_routing_in_one_call(ops, act, E, k, H, renorm, shared):
+    """``route`` is router_topk followed by moe_align; up to 16 tokens take a kernel that chooses and orders at
+    once: the same results either way, also for a token that sits in a larger batch."""
+    big = 21
+    x = rnd((big, H), torch.float32, 64).to(DEV)
+    wr = rnd((E, H), adt(act), 65).to(DEV)
+    sg = rnd((1, H), adt(act), 66, 0.1).to(DEV) if shared else None
+    ids_all, w_all, gate_all = ops.router_topk(x, wr, sg, k, renorm, act)
+    for T in (1, 3, 16, big):
+        for unit in (16, 64):
+            got = ops.route(x[:T].contiguous(), wr, sg, k, renorm, unit, act)
+            assert torch.equal(got[0], ids_all[:T]) and torch.equal(got[1], w_all[:T])
+            assert (got[2] is None) == (not shared) and (not shared or torch.equal(got[2], gate_all[:T]))
+            want = ops.moe_align(ids_all[:T].contiguous(), E, unit, act)
+            n = int(want[3])          # tiles in use; the entries of tile_expert beyond them are not written
+            assert torch.equal(got[3], want[0]) and torch.equal(got[4], want[1]) and torch.equal(got[6], want[3])
+            assert torch.equal(got[5][:n], want[2][:n])
+
+
 # ------------------------------------------------------------------------------------------------ rope + cache + attention
 def paged_setup(lens, page_size, nkv, hd, n_layers, act, seed):
     """Pages handed out in a scrambled order, so that a kernel that ignores the table fails."""

@@ -137,18 +137,14 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float* __restr
   }
 }
 
-__global__ __launch_bounds__(256) void router_select_kernel(const float* __restrict__ logits, int rows, int E,
-                                                            int topk, int renorm, int* __restrict__ ids,
-                                                            float* __restrict__ weights,
-                                                            float* __restrict__ shared_gate, int T) {
-  extern __shared__ float sm[];      // [4][E]
-  const int wave = threadIdx.x / TQ_WAVE, lane = threadIdx.x % TQ_WAVE;
-  const int t = blockIdx.x * 4 + wave;
-  if (t >= T) return;
-  float* lg = sm + wave * E;
-  const float* src = logits + (size_t)t * rows;
+// One wave chooses for one token.  src: the token's `rows` logits; lg: E floats of LDS for this wave; ids,
+// weights, shared_gate: where the token's results go; ids2: a second place for the ids (LDS), or null.
+__device__ __forceinline__ void select_token(const float* __restrict__ src, int rows, int E, int topk, int renorm,
+                                             float* lg, int* __restrict__ ids, int* ids2,
+                                             float* __restrict__ weights, float* __restrict__ shared_gate) {
+  const int lane = threadIdx.x % TQ_WAVE;
   for (int e = lane; e < E; e += TQ_WAVE) lg[e] = src[e];
-  if (rows > E && lane == 0) shared_gate[t] = 1.0f / (1.0f + expf(-src[E]));
+  if (rows > E && lane == 0) shared_gate[0] = 1.0f / (1.0f + expf(-src[E]));
   __builtin_amdgcn_wave_barrier();
   float mx = 0.f, denom = 1.f;
   if (!renorm) {      // softmax over all experts, before any logit is taken out
@@ -182,7 +178,8 @@ __global__ __launch_bounds__(256) void router_select_kernel(const float* __restr
     if (bi < 0) bi = 0;   // only if every logit is NaN
     if (lane == k) sel = bv;
     if (lane == 0) {
-      ids[t * topk + k] = bi;
+      ids[k] = bi;
+      if (ids2) ids2[k] = bi;
       lg[bi] = -INFINITY;   // taken out of the later rounds
     }
     __builtin_amdgcn_wave_barrier();
@@ -191,18 +188,26 @@ __global__ __launch_bounds__(256) void router_select_kernel(const float* __restr
     const float m = wave_max(lane < topk ? sel : -INFINITY);
     const float p = lane < topk ? expf(sel - m) : 0.f;
     const float s = wave_sum(p);
-    if (lane < topk) weights[t * topk + lane] = s > 0.f ? p * (1.0f / s) : 0.f;
+    if (lane < topk) weights[lane] = s > 0.f ? p * (1.0f / s) : 0.f;
   } else {
-    if (lane < topk) weights[t * topk + lane] = expf(sel - mx) * (1.0f / denom);
+    if (lane < topk) weights[lane] = expf(sel - mx) * (1.0f / denom);
   }
 }
 
-// logits: scratch of T * (E + 1) floats (T * E without a shared gate vector).
-TQ_API int tq_router_topk(const float* x, const void* wr, const void* shared_w, int wtype, int E, int topk,
-                          int renorm, int* ids, float* weights, float* shared_gate, float* logits, int T, int H,
-                          hipStream_t st) {
-  if (T <= 0) return 0;
-  if (topk < 1 || topk > 64 || topk > E || E > 8192) return TQ_ERR_UNSUPPORTED;
+__global__ __launch_bounds__(256) void router_select_kernel(const float* __restrict__ logits, int rows, int E,
+                                                            int topk, int renorm, int* __restrict__ ids,
+                                                            float* __restrict__ weights,
+                                                            float* __restrict__ shared_gate, int T) {
+  extern __shared__ float sm[];      // [4][E]
+  const int wave = threadIdx.x / TQ_WAVE;
+  const int t = blockIdx.x * 4 + wave;
+  if (t >= T) return;
+  select_token(logits + (size_t)t * rows, rows, E, topk, renorm, sm + wave * E, ids + (size_t)t * topk, nullptr,
+               weights + (size_t)t * topk, shared_gate + t);
+}
+
+static int launch_router_logits(const float* x, const void* wr, const void* shared_w, int wtype, int E,
+                                float* logits, int T, int H, hipStream_t st) {
   int tg = RT;
   const size_t hp = ((size_t)H + 511) / 512 * 512;      // a token's row in LDS
   while (tg > 1 && (size_t)tg * hp * sizeof(float) > 32 * 1024) tg /= 2;   // small enough for several workgroups per CU
@@ -239,6 +244,18 @@ TQ_API int tq_router_topk(const float* x, const void* wr, const void* shared_w, 
 #undef TQ_ROUTER_RW
 #undef TQ_ROUTER
   TQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// logits: scratch of T * (E + 1) floats (T * E without a shared gate vector).
+TQ_API int tq_router_topk(const float* x, const void* wr, const void* shared_w, int wtype, int E, int topk,
+                          int renorm, int* ids, float* weights, float* shared_gate, float* logits, int T, int H,
+                          hipStream_t st) {
+  if (T <= 0) return 0;
+  if (topk < 1 || topk > 64 || topk > E || E > 8192) return TQ_ERR_UNSUPPORTED;
+  const int rc = launch_router_logits(x, wr, shared_w, wtype, E, logits, T, H, st);
+  if (rc) return rc;
+  const int rows = E + (shared_w ? 1 : 0);
   hipLaunchKernelGGL(router_select_kernel, dim3((T + 3) / 4), dim3(256), (size_t)4 * E * sizeof(float), st, logits,
                      rows, E, topk, renorm, ids, weights, shared_gate, T);
   TQ_LAUNCH_CHECK();
@@ -260,13 +277,11 @@ TQ_API int tq_router_topk(const float* x, const void* wr, const void* shared_w, 
 // the expert, and each pair's row is that plus its rank.
 #define AW 16   // waves
 
-__global__ __launch_bounds__(64 * AW) void moe_align_kernel(const int* __restrict__ ids, int n_pairs, int E,
-                                                            int topk, int unit, int cap,
-                                                            int* __restrict__ sorted_token,
-                                                            int* __restrict__ pair_slot,
-                                                            int* __restrict__ tile_expert,
-                                                            int* __restrict__ n_tiles) {
-  extern __shared__ int cnt[];        // [AW][E] counts, then E starts
+// ids may lie in LDS or in memory; cnt: (AW + 1) * E ints of LDS ([AW][E] counts, then E starts).  All AW waves
+// of the workgroup call it together.
+__device__ __forceinline__ void align_pairs(const int* ids, int n_pairs, int E, int topk, int unit, int cap,
+                                            int* __restrict__ sorted_token, int* __restrict__ pair_slot,
+                                            int* __restrict__ tile_expert, int* __restrict__ n_tiles, int* cnt) {
   int* starts = cnt + AW * E;
   const int wave = threadIdx.x / TQ_WAVE, lane = threadIdx.x % TQ_WAVE;
   for (int i = threadIdx.x; i < cap; i += blockDim.x) sorted_token[i] = -1;
@@ -334,6 +349,38 @@ __global__ __launch_bounds__(64 * AW) void moe_align_kernel(const int* __restric
   }
 }
 
+__global__ __launch_bounds__(64 * AW) void moe_align_kernel(const int* __restrict__ ids, int n_pairs, int E,
+                                                            int topk, int unit, int cap,
+                                                            int* __restrict__ sorted_token,
+                                                            int* __restrict__ pair_slot,
+                                                            int* __restrict__ tile_expert,
+                                                            int* __restrict__ n_tiles) {
+  extern __shared__ int cnt[];
+  align_pairs(ids, n_pairs, E, topk, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles, cnt);
+}
+
+// The choice and the order of pairs in one workgroup, for up to AW tokens (decoding): wave w chooses for token w,
+// then all waves order the pairs; the same device functions and so the same results as the two kernels.
+__global__ __launch_bounds__(64 * AW) void select_align_kernel(const float* __restrict__ logits, int rows, int E,
+                                                               int topk, int renorm, int* __restrict__ ids,
+                                                               float* __restrict__ weights,
+                                                               float* __restrict__ shared_gate, int T, int unit,
+                                                               int cap, int* __restrict__ sorted_token,
+                                                               int* __restrict__ pair_slot,
+                                                               int* __restrict__ tile_expert,
+                                                               int* __restrict__ n_tiles) {
+  extern __shared__ int sm_i[];       // (AW + 1) * E ints for the order, AW * topk ids, AW * E floats for the choice
+  int* cnt = sm_i;
+  int* ids_l = cnt + (AW + 1) * E;
+  float* lg = (float*)(ids_l + AW * topk);
+  const int wave = threadIdx.x / TQ_WAVE;
+  if (wave < T)
+    select_token(logits + (size_t)wave * rows, rows, E, topk, renorm, lg + wave * E, ids + (size_t)wave * topk,
+                 ids_l + wave * topk, weights + (size_t)wave * topk, shared_gate + wave);
+  __syncthreads();
+  align_pairs(ids_l, T * topk, E, topk, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles, cnt);
+}
+
 // cap: rows that sorted_token holds, a multiple of unit and at least n_pairs + min(E, n_pairs) * (unit - 1);
 // tile_expert holds cap / unit entries.
 TQ_API int tq_moe_align(const int* ids, int n_pairs, int E, int topk, int unit, int cap, int* sorted_token,
@@ -346,6 +393,29 @@ TQ_API int tq_moe_align(const int* ids, int n_pairs, int E, int topk, int unit, 
     hipFuncSetAttribute((const void*)moe_align_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
   hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(64 * AW), shmem, st, ids, n_pairs, E, topk, unit, cap,
                      sorted_token, pair_slot, tile_expert, n_tiles);
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// tq_router_topk followed by tq_moe_align; up to 16 tokens take two kernels instead of three.
+TQ_API int tq_route(const float* x, const void* wr, const void* shared_w, int wtype, int E, int topk, int renorm,
+                    int* ids, float* weights, float* shared_gate, float* logits, int unit, int cap, int* sorted_token,
+                    int* pair_slot, int* tile_expert, int* n_tiles, int T, int H, hipStream_t st) {
+  if (T <= 0) return 0;
+  const size_t shmem = ((size_t)(AW + 1) * E + (size_t)AW * topk + (size_t)AW * E) * 4;
+  if (T > AW || shmem > 64 * 1024) {
+    const int rc = tq_router_topk(x, wr, shared_w, wtype, E, topk, renorm, ids, weights, shared_gate, logits, T, H, st);
+    return rc ? rc : tq_moe_align(ids, T * topk, E, topk, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles, st);
+  }
+  if (topk < 1 || topk > 64 || topk > E || E > 8192) return TQ_ERR_UNSUPPORTED;
+  const int n_pairs = T * topk;
+  if (unit < 1 || cap % unit != 0 || cap < n_pairs + (E < n_pairs ? E : n_pairs) * (unit - 1)) return TQ_ERR_BAD_ARG;
+  const int rc = launch_router_logits(x, wr, shared_w, wtype, E, logits, T, H, st);
+  if (rc) return rc;
+  if (shmem > 48 * 1024)
+    hipFuncSetAttribute((const void*)select_align_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+  hipLaunchKernelGGL(select_align_kernel, dim3(1), dim3(64 * AW), shmem, st, logits, E + (shared_w ? 1 : 0), E, topk,
+                     renorm, ids, weights, shared_gate, T, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles);
   TQ_LAUNCH_CHECK();
   return 0;
 }

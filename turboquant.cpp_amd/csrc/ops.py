@@ -40,6 +40,8 @@ _SIGNATURES = {
     "tq_router_topk": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
                        _c_ptr],
     "tq_moe_align": [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+    "tq_route": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
+                 _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
     "tq_argmax": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr],
     "tq_rep_penalty": [_c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_ptr, _c_f32, _c_ptr],
     "tq_sample_topp": [_c_ptr, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
@@ -387,7 +389,16 @@ def router_topk(x32: torch.Tensor, router: torch.Tensor, shared_scale: torch.Ten
                 renormalize: bool, act):
     """ids int32 [T, k], weights float32 [T, k], and sigmoid(x . shared_scale) float32 [T] (or None)."""
     k = "router_topk"
+    T, H, E, ids, weights, gate, logits = _router_outputs(k, x32, router, shared_scale, top_k)
+    _run(k, library(act).tq_router_topk(_ptr(x32), _ptr(router), _ptr(shared_scale), _WTYPE[router.dtype], E, top_k,
+                                        int(bool(renormalize)), _ptr(ids), _ptr(weights), _ptr(gate), _ptr(logits),
+                                        T, H, _stream()))
+    return ids, weights, gate
+
+
+def _router_outputs(k: str, x32: torch.Tensor, router: torch.Tensor, shared_scale: torch.Tensor | None, top_k: int):
     _check(x32, k, "x", torch.float32)
+    _need(x32.dim() == 2, k, "x must be [T, H]")
     T, H = x32.shape
     _check(router, k, "router", tuple(_WTYPE))
     _need(router.dim() == 2 and router.shape[1] == H, k, f"router must be [E, {H}]")
@@ -400,10 +411,33 @@ def router_topk(x32: torch.Tensor, router: torch.Tensor, shared_scale: torch.Ten
     weights = torch.empty((T, top_k), dtype=torch.float32, device=x32.device)
     gate = torch.empty((T,), dtype=torch.float32, device=x32.device) if shared_scale is not None else None
     logits = torch.empty((T, E + (1 if shared_scale is not None else 0)), dtype=torch.float32, device=x32.device)
-    _run(k, library(act).tq_router_topk(_ptr(x32), _ptr(router), _ptr(shared_scale), _WTYPE[router.dtype], E, top_k,
-                                        int(bool(renormalize)), _ptr(ids), _ptr(weights), _ptr(gate), _ptr(logits),
-                                        T, H, _stream()))
-    return ids, weights, gate
+    return T, H, E, ids, weights, gate, logits
+
+
+def _align_outputs(T: int, topk: int, num_experts: int, unit: int, dev):
+    n_pairs = T * topk
+    # every expert with at least one pair wastes at most unit-1 rows
+    cap = n_pairs + min(num_experts, n_pairs) * (unit - 1)
+    cap = (cap + unit - 1) // unit * unit
+    sorted_token = torch.empty((cap,), dtype=torch.int32, device=dev)
+    pair_slot = torch.empty((T, topk), dtype=torch.int32, device=dev)
+    tile_expert = torch.empty((cap // unit,), dtype=torch.int32, device=dev)
+    n_tiles = torch.empty((1,), dtype=torch.int32, device=dev)
+    return cap, sorted_token, pair_slot, tile_expert, n_tiles
+
+
+def route(x32: torch.Tensor, router: torch.Tensor, shared_scale: torch.Tensor | None, top_k: int, renormalize: bool,
+          unit: int, act):
+    """``router_topk`` followed by ``moe_align`` in one call: (ids, weights, gate, sorted_token, pair_slot,
+    tile_expert, n_tiles), with the same results; a handful of tokens takes one kernel less."""
+    k = "route"
+    T, H, E, ids, weights, gate, logits = _router_outputs(k, x32, router, shared_scale, top_k)
+    _need(unit in (16, 64), k, "unit must be 16 or 64")
+    cap, sorted_token, pair_slot, tile_expert, n_tiles = _align_outputs(T, top_k, E, unit, x32.device)
+    _run(k, library(act).tq_route(_ptr(x32), _ptr(router), _ptr(shared_scale), _WTYPE[router.dtype], E, top_k,
+                                  int(bool(renormalize)), _ptr(ids), _ptr(weights), _ptr(gate), _ptr(logits), unit, cap,
+                                  _ptr(sorted_token), _ptr(pair_slot), _ptr(tile_expert), _ptr(n_tiles), T, H, _stream()))
+    return ids, weights, gate, sorted_token, pair_slot, tile_expert, n_tiles
 
 
 def moe_align(ids: torch.Tensor, num_experts: int, unit: int, act):
@@ -413,14 +447,7 @@ def moe_align(ids: torch.Tensor, num_experts: int, unit: int, act):
     _check(ids, k, "ids", torch.int32)
     T, topk = ids.shape
     n_pairs = T * topk
-    # every expert with at least one pair wastes at most unit-1 rows
-    cap = n_pairs + min(num_experts, n_pairs) * (unit - 1)
-    cap = (cap + unit - 1) // unit * unit
-    dev = ids.device
-    sorted_token = torch.empty((cap,), dtype=torch.int32, device=dev)
-    pair_slot = torch.empty((T, topk), dtype=torch.int32, device=dev)
-    tile_expert = torch.empty((cap // unit,), dtype=torch.int32, device=dev)
-    n_tiles = torch.empty((1,), dtype=torch.int32, device=dev)
+    cap, sorted_token, pair_slot, tile_expert, n_tiles = _align_outputs(T, topk, num_experts, unit, ids.device)
     _run(k, library(act).tq_moe_align(_ptr(ids), n_pairs, num_experts, topk, unit, cap, _ptr(sorted_token),
                                       _ptr(pair_slot), _ptr(tile_expert), _ptr(n_tiles), _stream()))
     return sorted_token, pair_slot, tile_expert, n_tiles

@@ -72,10 +72,10 @@ class SparseMoE(Part):
                     shared = self._shared(normed, ctx)
             else:
                 shared = self._shared(normed, ctx)
-        ids, weights, gate = ops.router_topk(normed32, self.router, self.shared_scale if self.shared_gated else None,
-                                             self.top_k, self.renormalize, ctx.act)
         unit = 16 if T * self.top_k <= 16 * self.num_experts else 64
-        sorted_token, pair_slot, tile_expert, n_tiles = ops.moe_align(ids, self.num_experts, unit, ctx.act)
+        _, weights, gate, sorted_token, pair_slot, tile_expert, n_tiles = ops.route(
+            normed32, self.router, self.shared_scale if self.shared_gated else None, self.top_k, self.renormalize,
+            unit, ctx.act)
         h = ops.gemm(normed, self.expert_gate, ctx.act, w2=self.expert_up, out_act=True, a_rows=sorted_token,
                      tile_group=tile_expert, n_tiles=n_tiles, tile_rows=unit)
         y = ops.gemm(h, self.expert_down, ctx.act, a_rows=sorted_token, tile_group=tile_expert, n_tiles=n_tiles,
