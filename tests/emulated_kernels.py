@@ -39,7 +39,7 @@ def _rows_of(table, slot, positions, page_size):
 
 
 def rope_kv_write(qkv, positions, slot_of_token, block_table, inv_freq, pairing, rotary_dim, k_pages, v_pages,
-                  layer_offset, page_size, page_stride, num_heads, num_kv_heads, head_dim, act):
+                  layer_offset, page_size, page_stride, num_heads, num_kv_heads, head_dim, act, runs=None):
     T = positions.numel()
     x = qkv.view(T, num_heads + 2 * num_kv_heads, head_dim)
     ang = positions.float()[:, None] * inv_freq[None, :]

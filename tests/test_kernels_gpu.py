@@ -328,6 +328,36 @@ def test_rope_kv_write(ops, act, pairing, rot):
     assert int((kc != 0).sum()) <= T * nkv * hd and int((vc != 0).sum()) <= T * nkv * hd
 
 
+@pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("nh,nkv,hd,page", [(3, 1, 48, 64), (4, 2, 128, 128), (2, 2, 16, 64)])
+def test_values_of_whole_runs_are_written_by_tiles(ops, act, nh, nkv, hd, page):
+    """Told that the tokens are runs of consecutive positions, the kernel writes the values of whole prompts by
+    tiles of 64 positions; the pages must hold the same bits as after the token-by-token write, for runs that
+    start in the middle of a page, end in the middle of one, span several pages or are a single token."""
+    from plain_qwen2moe import rope_frequencies
+    starts, news = [0, 37, 64, 130, 5], [150, 100, 64, 1, 9]
+    lens = [a + b for a, b in zip(starts, news)]
+    table, slots, page_stride, kp, vp = paged_setup(lens, page, nkv, hd, 2, act, 110)
+    off = nkv * page * hd
+    T = sum(news)
+    qkv = rnd((T, (nh + 2 * nkv) * hd), torch.float32, 111)
+    positions = torch.cat([torch.arange(a, a + b) for a, b in zip(starts, news)]).to(torch.int32)
+    slot_of = torch.cat([torch.full((b,), s) for s, b in zip(slots, news)]).to(torch.int32)
+    freqs = torch.from_numpy(rope_frequencies(hd, 1e4))
+    cu = torch.tensor([0] + list(torch.tensor(news).cumsum(0)), dtype=torch.int32)
+    runs = {"cu_seqlens": cu.to(DEV), "slots": torch.tensor(slots, dtype=torch.int32).to(DEV),
+            "start": torch.tensor(starts, dtype=torch.int32).to(DEV), "max_new": max(news), "max_end": max(lens), "decode": False}
+    pages = []
+    for r in (None, runs):
+        kd, vd = kp.to(DEV).clone(), vp.to(DEV).clone()
+        q = ops.rope_kv_write(qkv.to(DEV), positions.to(DEV), slot_of.to(DEV), table.to(DEV), freqs.to(DEV), 0, hd, kd, vd,
+                              off, page, page_stride, nh, nkv, hd, act, runs=r)
+        pages.append((q.cpu(), kd.cpu(), vd.cpu()))
+    for a, b in zip(*pages):
+        assert torch.equal(a, b)
+    assert int((pages[0][2] != 0).sum()) > T * nkv * hd // 2
+
+
 def test_rope_pairings_are_one_rotation(ops):
     """interleaved(P x) = P half(x) for the permutation P that interleaves the two halves."""
     from plain_qwen2moe import rope as plain_rope

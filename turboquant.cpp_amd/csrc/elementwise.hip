@@ -169,7 +169,8 @@ TQ_API int tq_add_rmsnorm(float* x, const float* delta, int S, int64_t delta_str
 // layer's own offset (already added to k_pool / v_pool) keys lie [page][kv head][row][hd] and values
 // transposed, [page][kv head][hd][row].
 // A workgroup of four waves takes `spb` heads of one token (grid (T, ceil(heads / spb))); a wave takes every
-// fourth of them and turns pair i of all its heads with one sine and cosine.
+// fourth of them and turns pair i of all its heads with one sine and cosine.  write_kv: 0 queries only, 1 keys
+// and values, 2 keys only (the values of whole runs of tokens go through v_write_tile_kernel below).
 __global__ __launch_bounds__(256) void rope_kv_write_kernel(const float* __restrict__ qkv, const int* __restrict__ positions,
                                      const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
                                      int bt_stride, const float* __restrict__ inv_freq, int pairing, int rot,
@@ -213,7 +214,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(const float* __restr
     act_t* dst = s < nh ? q_t + (size_t)s * hd : k_t + (size_t)(s - nh) * kv_head_stride;
     for (int i = rot + lane; i < hd; i += TQ_WAVE) dst[i] = from_f32<act_t>(src[i]);
   }
-  if (!write_kv) return;
+  if (write_kv != 1) return;
   for (int s = s0; s < s1; s += 4) {           // values lie transposed, [hd][row]
     if (s < nh + nkv) continue;
     const float* src = src_t + (size_t)s * hd;
@@ -222,12 +223,78 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(const float* __restr
   }
 }
 
+// The values of runs of tokens, one run per sequence (tokens cu_seqlens[b] .. of sequence b lie at positions
+// start[b] ..): a workgroup takes 64 positions that share a page (grid (chunks, nkv, B)), turns their rows
+// [position][hd] into [hd][position] in LDS and writes every dimension's positions 16 bytes at a time, where the
+// token-by-token write above would touch a cache line per dimension for two bytes.
+#define VT_POS 64
+template <int VEC>      // positions per 16-byte store
+__global__ __launch_bounds__(256) void v_write_tile_kernel(const float* __restrict__ qkv,
+                                                           const int* __restrict__ cu_seqlens,
+                                                           const int* __restrict__ slots,
+                                                           const int* __restrict__ start,
+                                                           const int* __restrict__ block_table, int bt_stride,
+                                                           act_t* __restrict__ v_pool, int page_size,
+                                                           int64_t page_stride, int nh, int nkv, int hd) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char vt_raw[];
+  act_t* ts = (act_t*)vt_raw;                        // [hd][VT_POS + VEC]
+  constexpr int TS = VT_POS + VEC;
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int t0 = cu_seqlens[b], n = cu_seqlens[b + 1] - t0, st = start[b];
+  const int P0 = (st / VT_POS + blockIdx.x) * VT_POS;
+  const int lo = max(P0, st), hi = min(P0 + VT_POS, st + n);
+  if (lo >= hi) return;
+  const int wave = threadIdx.x / TQ_WAVE, lane = threadIdx.x % TQ_WAVE;
+  const int heads = nh + 2 * nkv;
+  const float* src0 = qkv + ((size_t)(t0 + lo - st) * heads + nh + nkv + h) * hd;      // value row of position lo
+  const size_t row_stride = (size_t)heads * hd;
+  if (hd % 4 == 0) {        // 16 bytes of a row per thread and turn, all of a thread's loads on their way at once
+    const int q4 = hd / 4, total = (hi - lo) * q4;
+#pragma unroll 8
+    for (int idx = threadIdx.x; idx < total; idx += 256) {
+      const int r = idx / q4, d = (idx % q4) * 4;
+      const f32x4 v = load4f(src0 + r * row_stride + d);
+      act_t* to = ts + d * TS + (lo + r - P0);
+      to[0] = from_f32<act_t>(v.x);
+      to[TS] = from_f32<act_t>(v.y);
+      to[2 * TS] = from_f32<act_t>(v.z);
+      to[3 * TS] = from_f32<act_t>(v.w);
+    }
+  } else {
+    for (int r = wave; r < hi - lo; r += 4)
+      for (int d = lane; d < hd; d += TQ_WAVE) ts[d * TS + (lo + r - P0)] = from_f32<act_t>(src0[r * row_stride + d]);
+  }
+  __syncthreads();
+  const int page = block_table[(size_t)slots[b] * bt_stride + P0 / page_size];
+  act_t* base = v_pool + (size_t)page * page_stride + (size_t)h * page_size * hd + P0 % page_size;
+  constexpr int GROUPS = VT_POS / VEC;
+  for (int idx = threadIdx.x; idx < hd * GROUPS; idx += blockDim.x) {
+    const int d = idx / GROUPS, g = idx % GROUPS;
+    const int p0 = P0 + g * VEC;
+    act_t* dst = base + (size_t)d * page_size + g * VEC;
+    const act_t* from = ts + d * TS + g * VEC;
+    if (p0 >= lo && p0 + VEC <= hi) {
+      *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(from);
+    } else {
+      for (int j = max(p0, lo) - p0; j < min(p0 + VEC, hi) - p0; ++j) dst[j] = from[j];
+    }
+  }
+}
+
+// cu_seqlens, slots, start (null, or [B + 1], [B], [B] with max_new the longest run): the tokens as runs of
+// consecutive positions, one per sequence; given for whole prompts, they let the values go by tiles.
 TQ_API int tq_rope_kv_write(const float* qkv, const int* positions, const int* seq_of_token,
                             const int* block_table, int bt_stride, const float* inv_freq, int pairing, int rot,
                             void* q_out, void* k_pool, void* v_pool, int page_size, int64_t page_stride, int T,
-                            int nh, int nkv, int hd, int write_kv, hipStream_t st) {
+                            int nh, int nkv, int hd, int write_kv, const int* cu_seqlens, const int* slots,
+                            const int* start, int B, int max_new, hipStream_t st) {
   if (T <= 0) return 0;
   if (rot < 0 || rot > hd || (rot & 1) || (pairing != 0 && pairing != 1)) return TQ_ERR_BAD_ARG;
+  constexpr int VEC = 16 / (int)sizeof(act_t);
+  const size_t vt_shmem = (size_t)hd * (VT_POS + VEC) * sizeof(act_t);
+  const bool tiles = write_kv && cu_seqlens && slots && start && B > 0 && B <= 65535 && nkv <= 65535 && max_new > 8 &&
+                     page_size % VT_POS == 0 && vt_shmem <= 64 * 1024;
+  if (tiles) write_kv = 2;
   const int heads = nh + 2 * nkv;
   // few tokens: a head per wave, so that the chip sees many small workgroups; many: all heads of a token in one
   int spb = 4;
@@ -237,6 +304,14 @@ TQ_API int tq_rope_kv_write(const float* qkv, const int* positions, const int* s
                      seq_of_token, block_table, bt_stride, inv_freq, pairing, rot, (act_t*)q_out, (act_t*)k_pool,
                      (act_t*)v_pool, page_size, page_stride, nh, nkv, hd, write_kv, spb);
   TQ_LAUNCH_CHECK();
+  if (tiles) {
+    if (vt_shmem > 48 * 1024)
+      hipFuncSetAttribute((const void*)v_write_tile_kernel<VEC>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)vt_shmem);
+    hipLaunchKernelGGL(v_write_tile_kernel<VEC>, dim3((max_new + VT_POS - 1) / VT_POS + 1, nkv, B), dim3(256), vt_shmem,
+                       st, qkv, cu_seqlens, slots, start, block_table, bt_stride, (act_t*)v_pool, page_size,
+                       page_stride, nh, nkv, hd);
+    TQ_LAUNCH_CHECK();
+  }
   return 0;
 }
 

@@ -31,7 +31,8 @@ _SIGNATURES = {
     "tq_add_rmsnorm": [_c_ptr, _c_ptr, _c_int, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_f32,
                        _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr],
     "tq_rope_kv_write": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
-                         _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+                         _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
+                         _c_ptr],
     "tq_moe_combine": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
     "tq_gemm_generic": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int,
                         _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
@@ -207,10 +208,12 @@ def add_rmsnorm(x: torch.Tensor, delta, weight: torch.Tensor, eps: float, act,
 def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor,
                   inv_freq: torch.Tensor, pairing: int, rotary_dim: int, k_pages: torch.Tensor | None,
                   v_pages: torch.Tensor | None, layer_offset: int, page_size: int, page_stride: int,
-                  num_heads: int, num_kv_heads: int, head_dim: int, act) -> torch.Tensor:
+                  num_heads: int, num_kv_heads: int, head_dim: int, act, runs: dict | None = None) -> torch.Tensor:
     """Rotates queries and keys, returns the queries [T, nh*hd] and writes keys and values into the pages.
     ``k_pages``/``v_pages`` are the flat page pools of the cache group (None: nothing is written, for a
-    layer that reads another layer's cache); ``layer_offset`` is the layer's offset inside a page."""
+    layer that reads another layer's cache); ``layer_offset`` is the layer's offset inside a page.  ``runs``
+    (as for ``attention``) describes the tokens as one run of consecutive positions per sequence; with it the
+    values of whole prompts are written by tiles."""
     k = "rope_kv_write"
     T = positions.numel()
     width = (num_heads + 2 * num_kv_heads) * head_dim
@@ -231,10 +234,19 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torc
         _need(layer_offset + num_kv_heads * page_size * head_dim <= page_stride, k, "layer does not fit in a page")
         esz = k_pages.element_size()
         kp, vp = k_pages.data_ptr() + layer_offset * esz, v_pages.data_ptr() + layer_offset * esz
+    cu = slots = start = None
+    B = max_new = 0
+    if runs is not None and write and not runs["decode"]:
+        B = runs["slots"].numel()
+        cu, slots, start, max_new = runs["cu_seqlens"], runs["slots"], runs["start"], int(runs["max_new"])
+        _check(cu, k, "cu_seqlens", torch.int32, (B + 1,))
+        _check(slots, k, "slots", torch.int32, (B,))
+        _check(start, k, "start", torch.int32, (B,))
+        _need(int(runs["max_end"]) <= block_table.shape[1] * page_size, k, "positions reach beyond the page table")
     _run(k, library(act).tq_rope_kv_write(_ptr(qkv), _ptr(positions), _ptr(seq_of_token), _ptr(block_table),
                                           block_table.shape[1], _ptr(inv_freq), pairing, rotary_dim, _ptr(q), kp, vp,
                                           page_size, page_stride, T, num_heads, num_kv_heads, head_dim, int(write),
-                                          _stream()))
+                                          _ptr(cu), _ptr(slots), _ptr(start), B, max_new, _stream()))
     return q
 
 

@@ -69,7 +69,7 @@ class GroupedQueryAttention(Part):
                               self.position.pairing_code, self.position.rotary_dim,
                               kv.k_pages if kv.owns else None, kv.v_pages if kv.owns else None,
                               kv.layer_offset, kv.page_size, kv.page_stride,
-                              self.num_heads, self.num_kv_heads, self.head_dim, ctx.act)
+                              self.num_heads, self.num_kv_heads, self.head_dim, ctx.act, runs=b.runs())
         o = ops.attention(q, kv.k_pages, kv.v_pages, kv.layer_offset, b.positions, b.slot_of_token, kv.table,
                           kv.page_size, kv.page_stride, self.num_heads, self.num_kv_heads, self.head_dim,
                           self.window, self.scale, ctx.act, runs=b.runs())
