@@ -204,6 +204,10 @@ def sample_topp(logits, temperature, top_p, uniforms, act):
     return torch.tensor(out, dtype=torch.int32)
 
 
+def gemm_pair(first, second, act):
+    return gemm(first.pop("a"), first.pop("w"), act, **first), gemm(second.pop("a"), second.pop("w"), act, **second)
+
+
 def route(x32, router, shared_scale, top_k, renormalize, unit, act):
     ids, weights, gate = router_topk(x32, router, shared_scale, top_k, renormalize, act)
     return (ids, weights, gate) + tuple(moe_align(ids, router.shape[0], unit, act))
@@ -212,6 +216,6 @@ def route(x32, router, shared_scale, top_k, renormalize, unit, act):
 def install(monkeypatch):
     """Puts the stand-ins in place of the kernels for one test."""
     from turboquant_cpp_amd.csrc import ops
-    for name in ("embed", "add_rmsnorm", "rope_kv_write", "attention", "gemm", "router_topk", "moe_align", "route",
+    for name in ("embed", "add_rmsnorm", "rope_kv_write", "attention", "gemm", "router_topk", "moe_align", "route", "gemm_pair",
                  "moe_combine", "argmax", "rep_penalty", "sample_topp"):
         monkeypatch.setattr(ops, name, globals()[name])

@@ -177,6 +177,41 @@ def test_expert_products(ops, act, unit, T, E, k, H, I):
 
 
 @pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("gated", [True, False])
+def test_two_products_in_one_launch(ops, act, gated):
+    """A product over experts and a plain product of the same few rows, asked for as a pair: the first gives the
+    bits it gives alone (its split of k is its own), the second agrees with the plain formula; more rows, or
+    products of different kinds, fall back to two calls with the same results."""
+    E, I, H, k, S = 7, 48, 264, 3, 104
+    for T in (1, 5, 16, 40):
+        x = rnd((T, H), adt(act), 45)
+        g = torch.Generator().manual_seed(46)
+        ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32)
+        unit = 16 if T <= 16 else 64
+        st, slot, te, nt = ops.moe_align(ids.to(DEV), E, unit, act)
+        wg, wu = rnd((E, I, H), adt(act), 47, 0.2), rnd((E, I, H), adt(act), 48, 0.2)
+        sg, su = rnd((S, H), adt(act), 49, 0.2), rnd((S, H), adt(act), 50, 0.2)
+        first = dict(a=x.to(DEV), w=wg.to(DEV), a_rows=st, tile_group=te, n_tiles=nt, tile_rows=unit)
+        second = dict(a=x.to(DEV), w=sg.to(DEV))
+        if gated:
+            first.update(w2=wu.to(DEV), out_act=True)
+            second.update(w2=su.to(DEV), out_act=True)
+        y1, y2 = ops.gemm_pair(dict(first), dict(second), act)
+        a1 = ops.gemm(first.pop("a"), first.pop("w"), act, **first)
+        a2 = ops.gemm(second.pop("a"), second.pop("w"), act, **second)
+        live = (st >= 0)
+        assert torch.equal(y1[live], a1[live])
+        ref2 = ref_gemm(x, sg, None, su if gated else None)
+        scale = ref2.abs().max().item()
+        lim = 1e-5 * scale * math.sqrt(H) if act == "float32" else (2e-2 if gated else 4e-3) * scale
+        assert (y2.cpu().double() - ref2).abs().max().item() < lim
+        assert (a2.cpu().double() - ref2).abs().max().item() < lim
+    # products of different kinds are two calls
+    y1, y2 = ops.gemm_pair(dict(a=x.to(DEV), w=sg.to(DEV), w2=su.to(DEV), out_act=True), dict(a=x.to(DEV), w=sg.to(DEV)), act)
+    assert y1.dtype == adt(act) and y2.dtype == torch.float32
+
+
+@pytest.mark.parametrize("act", ACTS)
 def test_moe_combine(ops, act):
     T, k, H, P, S = 6, 3, 100, 40, 2
     g = torch.Generator().manual_seed(50)

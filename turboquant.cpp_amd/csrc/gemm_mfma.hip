@@ -68,16 +68,15 @@ __device__ __forceinline__ void store_out(const MfmaGemmArgs& g, int m, int n, f
 }
 
 // ------------------------------------------------------------------------------------------ few rows
-// grid (ceil(N / 16), row tiles of 16 * MT rows); block 64 * (waves that split k).
+// A workgroup of 64 * (waves that split k) threads takes column tile `tile_n` (16 columns) of row tile `tile_m`
+// (16 * MT rows); red: LDS of [waves][MT * (DUAL ? 2 : 1)][4][64] floats.
 template <int MT, bool DUAL, bool OUT_ACT>
-__global__ __launch_bounds__(1024) void gemm_stream_kernel(MfmaGemmArgs g) {
-  extern __shared__ float red[];   // [waves][MT * (DUAL ? 2 : 1)][4][64]
-  const int tile_m = blockIdx.y;
+__device__ __forceinline__ void stream_body(const MfmaGemmArgs& g, int tile_n, int tile_m, float* red) {
   if (g.n_tiles && tile_m >= g.n_tiles[0]) return;
   const int group = g.tile_group ? g.tile_group[tile_m] : 0;
   const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, nw = blockDim.x / 64;
   const int r = lane % 16, c = lane / 16;
-  const int n0 = blockIdx.x * 16, m0 = tile_m * 16 * MT;
+  const int n0 = tile_n * 16, m0 = tile_m * 16 * MT;
   const int n = n0 + r;
   const bool n_ok = n < g.N;
   const bf16_t* wp = g.w + (size_t)group * g.group_stride + (size_t)(n_ok ? n : 0) * g.K + c * 8;
@@ -174,6 +173,28 @@ __global__ __launch_bounds__(1024) void gemm_stream_kernel(MfmaGemmArgs g) {
       if (DUAL) o = silu_f(o) * acc2[mt][v];
       store_out<OUT_ACT>(g, m, n, o);
     }
+}
+
+// grid (ceil(N / 16), row tiles of 16 * MT rows).
+template <int MT, bool DUAL, bool OUT_ACT>
+__global__ __launch_bounds__(1024) void gemm_stream_kernel(MfmaGemmArgs g) {
+  extern __shared__ float red[];
+  stream_body<MT, DUAL, OUT_ACT>(g, blockIdx.x, blockIdx.y, red);
+}
+
+// Two products that do not depend on each other in one launch (decoding: the routed experts' product beside
+// the shared expert's): workgroups 0 .. n2 - 1 take the second, smaller one (column tile id % nx2 of row tile
+// id / nx2), so that it is under way at once, the others the first.  Both are split over k by the waves of this
+// launch.
+template <bool DUAL, bool OUT_ACT>
+__global__ __launch_bounds__(1024) void gemm_stream_pair_kernel(MfmaGemmArgs g1, int nx1, MfmaGemmArgs g2, int nx2,
+                                                                 int n2) {
+  extern __shared__ float red[];
+  const int id = blockIdx.x;
+  if (id < n2)
+    stream_body<1, DUAL, OUT_ACT>(g2, id % nx2, id / nx2, red);
+  else
+    stream_body<1, DUAL, OUT_ACT>(g1, (id - n2) % nx1, (id - n2) / nx1, red);
 }
 
 // ------------------------------------------------------------------------------------------ many rows
@@ -474,6 +495,51 @@ TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gat
                                : launch_tile<128, 4, 2>(g, dual, out_act, splits, st);
   }
   if (rc) return rc;
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// Two products of few rows in one launch.  d1, d2: 18 numbers each, in the order of tq_gemm_mfma's arguments from
+// `a` to `tile_rows`.  Both must be products that the streaming kernel takes 16 rows at a time (a matrix per
+// expert with tile_rows 16, or one matrix with M <= 16), both gated or both not, both into the same type.  The
+// waves that split k are those of the first product (the larger one by convention).
+TQ_API int tq_gemm_mfma_pair(const int64_t* d1, const int64_t* d2, hipStream_t st) {
+  MfmaGemmArgs g[2];
+  int row_tiles[2];
+  bool dual[2], out_act[2];
+  const int64_t* d[2] = {d1, d2};
+  for (int i = 0; i < 2; ++i) {
+    const int64_t* p = d[i];
+    const int M = (int)p[14], N = (int)p[15], K = (int)p[16], tile_rows = (int)p[17];
+    if (M <= 0 || N <= 0 || K <= 0 || K % 8 != 0 || p[1] % 8 != 0 || p[6] % 8 != 0) return TQ_ERR_BAD_ARG;
+    if (((uintptr_t)p[0] | (uintptr_t)p[4] | (uintptr_t)p[5]) % 16 != 0) return TQ_ERR_BAD_ARG;
+    g[i] = MfmaGemmArgs{(const bf16_t*)p[0], p[1], (const int*)p[2], (int)p[3], (const bf16_t*)p[4], (const bf16_t*)p[5],
+                        p[6], (const int*)p[7], (const int*)p[8], (const void*)p[9], (int)p[10], (void*)p[11], p[12],
+                        M, N, K, K, 0};
+    dual[i] = p[5] != 0;
+    out_act[i] = p[13] != 0;
+    if (g[i].tile_group) {
+      if (tile_rows != 16 || M % 16) return TQ_ERR_BAD_ARG;
+      row_tiles[i] = M / 16;
+    } else {
+      if (M > 16) return TQ_ERR_BAD_ARG;
+      row_tiles[i] = 1;
+    }
+  }
+  if (dual[0] != dual[1] || out_act[0] != out_act[1]) return TQ_ERR_BAD_ARG;
+  const int nw = split_k_waves(g[0].N, g[0].K, g[0].tile_group != nullptr);
+  const size_t shmem = nw > 1 ? (size_t)nw * (dual[0] ? 2 : 1) * 4 * 64 * sizeof(float) : 0;
+  const int nx1 = (g[0].N + 15) / 16, nx2 = (g[1].N + 15) / 16;
+  const int64_t n1 = (int64_t)nx1 * row_tiles[0], n2 = (int64_t)nx2 * row_tiles[1];
+  if (n1 + n2 > 0x7fffffff) return TQ_ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)(n1 + n2));
+#define TQ_PAIR(D, O) \
+  hipLaunchKernelGGL((gemm_stream_pair_kernel<D, O>), grid, dim3(64 * nw), shmem, st, g[0], nx1, g[1], nx2, (int)n2)
+  if (dual[0] && out_act[0]) TQ_PAIR(true, true);
+  else if (dual[0]) TQ_PAIR(true, false);
+  else if (out_act[0]) TQ_PAIR(false, true);
+  else TQ_PAIR(false, false);
+#undef TQ_PAIR
   TQ_LAUNCH_CHECK();
   return 0;
 }

@@ -52,6 +52,7 @@ _OPTIONAL = {
     "tq_gemm_mfma": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int,
                      _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "tq_gemm_mfma_splits": [_c_int, _c_int, _c_int],
+    "tq_gemm_mfma_pair": [_c_ptr, _c_ptr, _c_ptr],
     "tq_attention_decode_scratch": [_c_int, _c_int, _c_int, _c_int],
     "tq_attention_mfma": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int,
                           _c_int, _c_int, _c_int, _c_f32, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
@@ -278,20 +279,8 @@ def _use_mfma(act, a: torch.Tensor, w: torch.Tensor, K: int) -> bool:
             and has_kernel(act, "tq_gemm_mfma"))
 
 
-def gemm(a: torch.Tensor, w: torch.Tensor, act, bias: torch.Tensor | None = None, w2: torch.Tensor | None = None,
-         out_act: bool = False, a_rows: torch.Tensor | None = None, tile_group: torch.Tensor | None = None,
-         n_tiles: torch.Tensor | None = None, tile_rows: int | None = None, gather: bool = True,
-         partial_sums: bool = False) -> torch.Tensor:
-    """out[m, n] = sum_k a[row(m), k] * w[g, n, k]  (+ bias[n]);  with ``w2``: silu(a w^T) * (a w2^T).
-
-    ``a`` [M, K] activations.  ``w`` [N, K], or [G, N, K] with ``tile_group`` naming the matrix of each tile of
-    ``tile_rows`` output rows and ``a_rows`` [P] the row of ``a`` behind each output row (-1: none; with
-    ``gather`` false a live output row m reads row m of ``a``).
-    Output is float32 unless ``out_act``.  Sums run over k in ascending order whatever M is.
-    ``partial_sums`` (plain products into float32 only): the result is [S, M, N], S >= 1 partial sums over runs of
-    k that the caller adds up in order, as the next norm does with a part's output; the kernel chooses S.
-    """
-    k = "gemm"
+def _gemm_problem(k: str, a, w, act, bias, w2, out_act, a_rows, tile_group, n_tiles, tile_rows, gather):
+    """Checks one product's operands; returns (M, N, K, tile_rows, group stride)."""
     adt = ACT_DTYPES[dtype_name(act)]
     _check(a, k, "a", adt)
     _need(a.dim() == 2, k, "a must be [M, K]")
@@ -322,6 +311,27 @@ def gemm(a: torch.Tensor, w: torch.Tensor, act, bias: torch.Tensor | None = None
         _check(w2, k, "w2", w.dtype, tuple(w.shape))
     if bias is not None:
         _check(bias, k, "bias", tuple(_WTYPE), (N,))
+    return M, N, K, tile_rows, gstride
+
+
+def gemm(a: torch.Tensor, w: torch.Tensor, act, bias: torch.Tensor | None = None, w2: torch.Tensor | None = None,
+         out_act: bool = False, a_rows: torch.Tensor | None = None, tile_group: torch.Tensor | None = None,
+         n_tiles: torch.Tensor | None = None, tile_rows: int | None = None, gather: bool = True,
+         partial_sums: bool = False) -> torch.Tensor:
+    """out[m, n] = sum_k a[row(m), k] * w[g, n, k]  (+ bias[n]);  with ``w2``: silu(a w^T) * (a w2^T).
+
+    ``a`` [M, K] activations.  ``w`` [N, K], or [G, N, K] with ``tile_group`` naming the matrix of each tile of
+    ``tile_rows`` output rows and ``a_rows`` [P] the row of ``a`` behind each output row (-1: none; with
+    ``gather`` false a live output row m reads row m of ``a``).
+    Output is float32 unless ``out_act``.  Sums run over k in ascending order whatever M is.
+    ``partial_sums`` (plain products into float32 only): the result is [S, M, N], S >= 1 partial sums over runs of
+    k that the caller adds up in order, as the next norm does with a part's output; the kernel chooses S.
+    """
+    k = "gemm"
+    adt = ACT_DTYPES[dtype_name(act)]
+    grouped = tile_group is not None
+    M, N, K, tile_rows, gstride = _gemm_problem(k, a, w, act, bias, w2, out_act, a_rows, tile_group, n_tiles, tile_rows,
+                                                gather)
     if partial_sums:
         _need(w2 is None and not out_act and not grouped and a_rows is None, k,
               "partial sums are for plain products into float32")
@@ -341,6 +351,44 @@ def gemm(a: torch.Tensor, w: torch.Tensor, act, bias: torch.Tensor | None = None
                                 _WTYPE[bias.dtype] if bias is not None else 0, _ptr(out), N, int(out_act), M, N, K,
                                 tile_rows, _stream()))
     return out
+
+
+def gemm_pair(first: dict, second: dict, act) -> tuple[torch.Tensor, torch.Tensor]:
+    """Two products that do not depend on each other; ``first`` and ``second`` hold the arguments of ``gemm``
+    (without ``partial_sums``).  Products of few rows of the same kind (both gated or both plain, into the same
+    type) go out in one launch, so that the smaller one costs no launch of its own; anything else is two calls."""
+    k = "gemm_pair"
+    keys = ("bias", "w2", "out_act", "a_rows", "tile_group", "n_tiles", "tile_rows", "gather")
+    probs = []
+    for p in (first, second):
+        full = {"bias": None, "w2": None, "out_act": False, "a_rows": None, "tile_group": None, "n_tiles": None,
+                "tile_rows": None, "gather": True}
+        _need(set(p) <= set(full) | {"a", "w"}, k, f"unknown arguments {sorted(set(p) - set(full) - {'a', 'w'})}")
+        full.update(p)
+        probs.append(full)
+    lib = library(act) if dtype_name(act) == "bfloat16" else None
+    fused = lib is not None and hasattr(lib, "tq_gemm_mfma_pair")
+    dims = []
+    for p in probs:
+        M, N, K, tile_rows, gstride = _gemm_problem(k, p["a"], p["w"], act, p["bias"], p["w2"], p["out_act"], p["a_rows"],
+                                                    p["tile_group"], p["n_tiles"], p["tile_rows"], p["gather"])
+        dims.append((M, N, K, tile_rows, gstride))
+        few = (p["tile_group"] is not None and tile_rows == 16) or (p["tile_group"] is None and M <= 16)
+        fused = fused and few and _use_mfma(act, p["a"], p["w"], K) and (p["bias"] is None or p["bias"].dtype in _WTYPE)
+    fused = fused and (probs[0]["w2"] is None) == (probs[1]["w2"] is None) and probs[0]["out_act"] == probs[1]["out_act"]
+    if not fused:
+        return tuple(gemm(p["a"], p["w"], act, **{n: p[n] for n in keys}) for p in probs)
+    adt = ACT_DTYPES[dtype_name(act)]
+    outs, descs = [], []
+    for p, (M, N, K, tile_rows, gstride) in zip(probs, dims):
+        out = torch.empty((M, N), dtype=adt if p["out_act"] else torch.float32, device=p["a"].device)
+        outs.append(out)
+        vals = [_ptr(p["a"]), p["a"].stride(0), _ptr(p["a_rows"]), int(p["gather"]), _ptr(p["w"]), _ptr(p["w2"]), gstride,
+                _ptr(p["tile_group"]), _ptr(p["n_tiles"]), _ptr(p["bias"]),
+                _WTYPE[p["bias"].dtype] if p["bias"] is not None else 0, _ptr(out), N, int(p["out_act"]), M, N, K, tile_rows]
+        descs.append((ctypes.c_int64 * 18)(*[0 if v is None else int(v) for v in vals]))
+    _run(k, lib.tq_gemm_mfma_pair(descs[0], descs[1], _stream()))
+    return outs[0], outs[1]
 
 
 # ------------------------------------------------------------------ attention

@@ -63,7 +63,19 @@ class SparseMoE(Part):
 
     def forward(self, normed, normed32, ctx):
         T = normed.shape[0]
-        # the shared expert needs nothing from the router: it runs on a second stream beside the routed experts
+        unit = 16 if T * self.top_k <= 16 * self.num_experts else 64
+        route = lambda: ops.route(normed32, self.router, self.shared_scale if self.shared_gated else None,
+                                  self.top_k, self.renormalize, unit, ctx.act)
+        if self.shared_size > 0 and T <= 16 and unit == 16:
+            # a handful of tokens: the shared expert's two products ride in the launches of the routed experts'
+            _, weights, gate, sorted_token, pair_slot, tile_expert, n_tiles = route()
+            experts = dict(a_rows=sorted_token, tile_group=tile_expert, n_tiles=n_tiles, tile_rows=unit)
+            h, hs = ops.gemm_pair(dict(a=normed, w=self.expert_gate, w2=self.expert_up, out_act=True, **experts),
+                                  dict(a=normed, w=self.shared_gate, w2=self.shared_up, out_act=True), ctx.act)
+            y, shared = ops.gemm_pair(dict(a=h, w=self.expert_down, gather=False, **experts),
+                                      dict(a=hs, w=self.shared_down), ctx.act)
+            return ops.GatheredSum(y, pair_slot, weights, shared.unsqueeze(0), gate)
+        # the shared expert needs nothing from the router: it may run on a second stream beside the routed experts
         shared, side = None, None
         if self.shared_size > 0:
             side = ctx.fork() if hasattr(ctx, "fork") else None
@@ -72,10 +84,7 @@ class SparseMoE(Part):
                     shared = self._shared(normed, ctx)
             else:
                 shared = self._shared(normed, ctx)
-        unit = 16 if T * self.top_k <= 16 * self.num_experts else 64
-        _, weights, gate, sorted_token, pair_slot, tile_expert, n_tiles = ops.route(
-            normed32, self.router, self.shared_scale if self.shared_gated else None, self.top_k, self.renormalize,
-            unit, ctx.act)
+        _, weights, gate, sorted_token, pair_slot, tile_expert, n_tiles = route()
         h = ops.gemm(normed, self.expert_gate, ctx.act, w2=self.expert_up, out_act=True, a_rows=sorted_token,
                      tile_group=tile_expert, n_tiles=n_tiles, tile_rows=unit)
         y = ops.gemm(h, self.expert_down, ctx.act, a_rows=sorted_token, tile_group=tile_expert, n_tiles=n_tiles,
