@@ -612,6 +612,40 @@ def test_a_feed_forward_with_routing_and_another_position_encoding_defined_here(
         unregister_part("ffn", "toy_one_of_four")
 
 
+def test_a_capture_is_not_disturbed_by_garbage_of_earlier_engines(engines, sharp_dirs):
+    """Engines that are dropped leave graphs behind for the garbage collector; if it found them in the middle of
+    another engine's capture, destroying them there would end the process.  Here the collector is made eager and
+    garbage is left lying about before a capture; the capture must go through and give the bits of an eager step."""
+    import gc
+    from turboquant_cpp_amd.engine.model import load_model
+    from turboquant_cpp_amd.engine.step import Engine
+    d, _ = sharp_dirs("A", "bfloat16")
+    model = load_model(d, act="bfloat16", device=DEV)
+    prompts = prompts_for("A", [5, 9], 200)
+
+    def decode(engine, steps):
+        slots = engine.open(2)
+        engine.step(slots, prompts)
+        out = [engine.step(slots, [[3 + i], [4 + i]]).clone() for i in range(steps)]
+        engine.close(slots)
+        return out
+
+    want = decode(Engine(model, max_tokens=256, use_graphs=False), 4)
+    gc.collect()
+    gc.disable()
+    for _ in range(3):                       # engines with captured graphs, dropped but not yet collected
+        decode(Engine(model, max_tokens=256), 3)
+    old = gc.get_threshold()
+    gc.set_threshold(1, 1, 1)                # the collector runs at the next allocations
+    gc.enable()
+    try:
+        got = decode(Engine(model, max_tokens=256), 4)      # eager, capture, replay, replay
+    finally:
+        gc.set_threshold(*old)
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+
+
 def test_the_kernels_refuse_to_run_without_their_library(monkeypatch):
     """No silent fallback: if the compiled library cannot be found or built, the first kernel call raises."""
     from turboquant_cpp_amd.csrc import build, ops

@@ -8,6 +8,8 @@ key of the graph.  No memset is recorded (only kernels), and results are the bit
 """
 from __future__ import annotations
 
+import gc
+
 import numpy as np
 import torch
 
@@ -67,8 +69,18 @@ class DecodeGraph:
         ctx = StepContext(batch=self.batch(slots, starts), cache=e.cache, act=e.model.act, device=e.device,
                           side_stream=e.side_stream)
         torch.cuda.synchronize()
-        with torch.cuda.graph(self.graph, pool=self.pool):
-            self.logits = e.model.forward(ctx)
+        # Nothing may be destroyed on the device while the stream is capturing: an older graph that the garbage
+        # collector happens to find in the middle of the capture would end the process.  So what is garbage goes
+        # now, and the collector rests until the capture is over.
+        gc.collect()
+        collecting = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(self.graph, pool=self.pool):
+                self.logits = e.model.forward(ctx)
+        finally:
+            if collecting:
+                gc.enable()
         self.graph.replay()
         return self.logits
 
