@@ -212,6 +212,36 @@ def test_two_products_in_one_launch(ops, act, gated):
 
 
 @pytest.mark.parametrize("act", ACTS)
+def test_second_product_of_a_pair_in_runs_of_k(ops, act):
+    """The experts' down products (short k) beside a plain product with a long k whose partial sums are wanted
+    apart: the second one comes in several runs of k (bfloat16: 8 here, and as many whatever the number of rows),
+    their sum is the product, the bias is counted once, and the first product keeps the bits it has alone."""
+    E, I, H, k, S = 5, 512, 264, 2, 4104
+    shapes = set()
+    for T in (1, 7, 16):
+        g = torch.Generator().manual_seed(146)
+        ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32)
+        st, slot, te, nt = ops.moe_align(ids.to(DEV), E, 16, act)
+        h = rnd((st.numel(), I), adt(act), 147)
+        hs = rnd((T, S), adt(act), 148)
+        wd, sd = rnd((E, H, I), adt(act), 149, 0.2), rnd((H, S), adt(act), 150, 0.2)
+        bias = rnd((H,), adt(act), 151)
+        first = dict(a=h.to(DEV), w=wd.to(DEV), a_rows=st, tile_group=te, n_tiles=nt, tile_rows=16, gather=False)
+        second = dict(a=hs.to(DEV), w=sd.to(DEV), bias=bias.to(DEV), partial_sums=True)
+        y1, y2 = ops.gemm_pair(dict(first), dict(second), act)
+        a1 = ops.gemm(first.pop("a"), first.pop("w"), act, **first)
+        live = (st >= 0)
+        assert torch.equal(y1[live], a1[live])
+        assert y2.dim() == 3 and y2.shape[1:] == (T, H) and y2.dtype == torch.float32
+        shapes.add(y2.shape[0])
+        ref2 = ref_gemm(hs, sd, bias, None)
+        scale = ref2.abs().max().item()
+        lim = 1e-5 * scale * math.sqrt(S) if act == "float32" else 4e-3 * scale
+        assert (y2.cpu().double().sum(0) - ref2).abs().max().item() < lim
+    assert shapes == ({8} if act == "bfloat16" else {1})
+
+
+@pytest.mark.parametrize("act", ACTS)
 def test_moe_combine(ops, act):
     T, k, H, P, S = 6, 3, 100, 40, 2
     g = torch.Generator().manual_seed(50)

@@ -39,7 +39,7 @@ struct MfmaGemmArgs {
   void* out;
   int64_t ldc;
   int M, N, K;
-  int k_per;                // many rows only: k is split into runs of k_per, run z going to out + z * split_stride
+  int k_per;                // k is split into runs of k_per, run z going to out + z * split_stride (float)
   int64_t split_stride;
 };
 
@@ -69,10 +69,16 @@ __device__ __forceinline__ void store_out(const MfmaGemmArgs& g, int m, int n, f
 
 // ------------------------------------------------------------------------------------------ few rows
 // A workgroup of 64 * (waves that split k) threads takes column tile `tile_n` (16 columns) of row tile `tile_m`
-// (16 * MT rows); red: LDS of [waves][MT * (DUAL ? 2 : 1)][4][64] floats.
+// (16 * MT rows) over run `z` of k (k_per long; run 0 is all of k unless the product is split into partial
+// sums); red: LDS of [waves][MT * (DUAL ? 2 : 1)][4][64] floats.
 template <int MT, bool DUAL, bool OUT_ACT>
-__device__ __forceinline__ void stream_body(const MfmaGemmArgs& g, int tile_n, int tile_m, float* red) {
+__device__ __forceinline__ void stream_body(MfmaGemmArgs g, int tile_n, int tile_m, int z, float* red) {
   if (g.n_tiles && tile_m >= g.n_tiles[0]) return;
+  const int k_lo = z * g.k_per, k_hi = min(g.K, k_lo + g.k_per);
+  if (z) {
+    g.out = (float*)g.out + z * g.split_stride;
+    g.bias = nullptr;
+  }
   const int group = g.tile_group ? g.tile_group[tile_m] : 0;
   const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, nw = blockDim.x / 64;
   const int r = lane % 16, c = lane / 16;
@@ -93,9 +99,9 @@ __device__ __forceinline__ void stream_body(const MfmaGemmArgs& g, int tile_n, i
     ap[mt] = src >= 0 ? g.a + (size_t)src * g.lda + c * 8 : nullptr;
   }
   // this wave's share of k, in steps of 32
-  const int steps = (g.K + 31) / 32;
+  const int steps = (k_hi - k_lo + 31) / 32;
   const int per = (steps + nw - 1) / nw;
-  const int k_beg = wave * per * 32, k_end = min(g.K, (wave + 1) * per * 32);
+  const int k_beg = k_lo + wave * per * 32, k_end = min(k_hi, k_lo + (wave + 1) * per * 32);
 
   f32x4 acc[MT], acc2[DUAL ? MT : 1];
 #pragma unroll
@@ -179,22 +185,23 @@ __device__ __forceinline__ void stream_body(const MfmaGemmArgs& g, int tile_n, i
 template <int MT, bool DUAL, bool OUT_ACT>
 __global__ __launch_bounds__(1024) void gemm_stream_kernel(MfmaGemmArgs g) {
   extern __shared__ float red[];
-  stream_body<MT, DUAL, OUT_ACT>(g, blockIdx.x, blockIdx.y, red);
+  stream_body<MT, DUAL, OUT_ACT>(g, blockIdx.x, blockIdx.y, 0, red);
 }
 
 // Two products that do not depend on each other in one launch (decoding: the routed experts' product beside
 // the shared expert's): workgroups 0 .. n2 - 1 take the second, smaller one (column tile id % nx2 of row tile
-// id / nx2), so that it is under way at once, the others the first.  Both are split over k by the waves of this
-// launch.
+// id / nx2 % rows2, run id / nx2 / rows2 of k), so that it is under way at once, the others the first.  Both are
+// split over k by the waves of this launch; the second one, when its k is much longer than the first one's, also
+// into runs whose partial sums go out apart.
 template <bool DUAL, bool OUT_ACT>
 __global__ __launch_bounds__(1024) void gemm_stream_pair_kernel(MfmaGemmArgs g1, int nx1, MfmaGemmArgs g2, int nx2,
-                                                                 int n2) {
+                                                                 int rows2, int n2) {
   extern __shared__ float red[];
   const int id = blockIdx.x;
   if (id < n2)
-    stream_body<1, DUAL, OUT_ACT>(g2, id % nx2, id / nx2, red);
+    stream_body<1, DUAL, OUT_ACT>(g2, id % nx2, id / nx2 % rows2, id / nx2 / rows2, red);
   else
-    stream_body<1, DUAL, OUT_ACT>(g1, (id - n2) % nx1, (id - n2) / nx1, red);
+    stream_body<1, DUAL, OUT_ACT>(g1, (id - n2) % nx1, (id - n2) / nx1, 0, red);
 }
 
 // ------------------------------------------------------------------------------------------ many rows
@@ -499,11 +506,27 @@ TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gat
   return 0;
 }
 
+// Into how many runs of k the second product of a pair is split when its partial sums are wanted apart: the
+// workgroups of a pair have the waves that suit the first product, so a second product that alone would have s
+// times as many waves over its k gets s runs instead.  A function of the two products' N and K and of whether each
+// has a matrix per expert.
+static int pair_run_of_k(int N1, int K1, bool grouped1, int N2, int K2, bool grouped2) {
+  const int nw = split_k_waves(N1, K1, grouped1), nw2 = split_k_waves(N2, K2, grouped2);
+  if (nw2 <= nw) return K2;
+  return ((K2 + 31) / 32 + nw2 / nw - 1) / (nw2 / nw) * 32;      // a multiple of 32
+}
+TQ_API int tq_gemm_mfma_pair_splits(int N1, int K1, int grouped1, int N2, int K2, int grouped2) {
+  const int k_per = pair_run_of_k(N1, K1, grouped1 != 0, N2, K2, grouped2 != 0);
+  return (K2 + k_per - 1) / k_per;
+}
+
 // Two products of few rows in one launch.  d1, d2: 18 numbers each, in the order of tq_gemm_mfma's arguments from
 // `a` to `tile_rows`.  Both must be products that the streaming kernel takes 16 rows at a time (a matrix per
 // expert with tile_rows 16, or one matrix with M <= 16), both gated or both not, both into the same type.  The
-// waves that split k are those of the first product (the larger one by convention).
-TQ_API int tq_gemm_mfma_pair(const int64_t* d1, const int64_t* d2, hipStream_t st) {
+// waves that split k are those of the first product (the larger one by convention).  splits2 > 1 (as
+// tq_gemm_mfma_pair_splits says, for a plain second product into float): run z of its k goes to
+// out + z * M * ldc, the bias to run 0.
+TQ_API int tq_gemm_mfma_pair(const int64_t* d1, const int64_t* d2, int splits2, hipStream_t st) {
   MfmaGemmArgs g[2];
   int row_tiles[2];
   bool dual[2], out_act[2];
@@ -527,14 +550,21 @@ TQ_API int tq_gemm_mfma_pair(const int64_t* d1, const int64_t* d2, hipStream_t s
     }
   }
   if (dual[0] != dual[1] || out_act[0] != out_act[1]) return TQ_ERR_BAD_ARG;
+  if (splits2 < 1) return TQ_ERR_BAD_ARG;
+  if (splits2 > 1) {
+    if (dual[1] || out_act[1] || g[1].a_rows || g[1].tile_group) return TQ_ERR_BAD_ARG;
+    g[1].k_per = pair_run_of_k(g[0].N, g[0].K, g[0].tile_group != nullptr, g[1].N, g[1].K, false);
+    if (splits2 != (g[1].K + g[1].k_per - 1) / g[1].k_per) return TQ_ERR_BAD_ARG;
+    g[1].split_stride = (int64_t)g[1].M * g[1].ldc;
+  }
   const int nw = split_k_waves(g[0].N, g[0].K, g[0].tile_group != nullptr);
   const size_t shmem = nw > 1 ? (size_t)nw * (dual[0] ? 2 : 1) * 4 * 64 * sizeof(float) : 0;
   const int nx1 = (g[0].N + 15) / 16, nx2 = (g[1].N + 15) / 16;
-  const int64_t n1 = (int64_t)nx1 * row_tiles[0], n2 = (int64_t)nx2 * row_tiles[1];
+  const int64_t n1 = (int64_t)nx1 * row_tiles[0], n2 = (int64_t)nx2 * row_tiles[1] * splits2;
   if (n1 + n2 > 0x7fffffff) return TQ_ERR_UNSUPPORTED;
   const dim3 grid((unsigned)(n1 + n2));
 #define TQ_PAIR(D, O) \
-  hipLaunchKernelGGL((gemm_stream_pair_kernel<D, O>), grid, dim3(64 * nw), shmem, st, g[0], nx1, g[1], nx2, (int)n2)
+  hipLaunchKernelGGL((gemm_stream_pair_kernel<D, O>), grid, dim3(64 * nw), shmem, st, g[0], nx1, g[1], nx2, row_tiles[1], (int)n2)
   if (dual[0] && out_act[0]) TQ_PAIR(true, true);
   else if (dual[0]) TQ_PAIR(true, false);
   else if (out_act[0]) TQ_PAIR(false, true);

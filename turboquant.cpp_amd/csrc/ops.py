@@ -52,7 +52,8 @@ _OPTIONAL = {
     "tq_gemm_mfma": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int,
                      _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "tq_gemm_mfma_splits": [_c_int, _c_int, _c_int],
-    "tq_gemm_mfma_pair": [_c_ptr, _c_ptr, _c_ptr],
+    "tq_gemm_mfma_pair_splits": [_c_int, _c_int, _c_int, _c_int, _c_int, _c_int],
+    "tq_gemm_mfma_pair": [_c_ptr, _c_ptr, _c_int, _c_ptr],
     "tq_attention_decode_scratch": [_c_int, _c_int, _c_int, _c_int],
     "tq_attention_mfma": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int,
                           _c_int, _c_int, _c_int, _c_f32, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
@@ -355,14 +356,16 @@ def gemm(a: torch.Tensor, w: torch.Tensor, act, bias: torch.Tensor | None = None
 
 def gemm_pair(first: dict, second: dict, act) -> tuple[torch.Tensor, torch.Tensor]:
     """Two products that do not depend on each other; ``first`` and ``second`` hold the arguments of ``gemm``
-    (without ``partial_sums``).  Products of few rows of the same kind (both gated or both plain, into the same
-    type) go out in one launch, so that the smaller one costs no launch of its own; anything else is two calls."""
+    (``partial_sums`` only in the second).  Products of few rows of the same kind (both gated or both plain, into
+    the same type) go out in one launch, so that the smaller one costs no launch of its own; anything else is two
+    calls."""
     k = "gemm_pair"
-    keys = ("bias", "w2", "out_act", "a_rows", "tile_group", "n_tiles", "tile_rows", "gather")
+    keys = ("bias", "w2", "out_act", "a_rows", "tile_group", "n_tiles", "tile_rows", "gather", "partial_sums")
     probs = []
+    _need(not first.get("partial_sums", False), k, "only the second product may leave partial sums")
     for p in (first, second):
         full = {"bias": None, "w2": None, "out_act": False, "a_rows": None, "tile_group": None, "n_tiles": None,
-                "tile_rows": None, "gather": True}
+                "tile_rows": None, "gather": True, "partial_sums": False}
         _need(set(p) <= set(full) | {"a", "w"}, k, f"unknown arguments {sorted(set(p) - set(full) - {'a', 'w'})}")
         full.update(p)
         probs.append(full)
@@ -380,14 +383,22 @@ def gemm_pair(first: dict, second: dict, act) -> tuple[torch.Tensor, torch.Tenso
         return tuple(gemm(p["a"], p["w"], act, **{n: p[n] for n in keys}) for p in probs)
     adt = ACT_DTYPES[dtype_name(act)]
     outs, descs = [], []
+    splits = 1
+    if probs[1]["partial_sums"]:
+        p2 = probs[1]
+        _need(p2["w2"] is None and not p2["out_act"] and p2["tile_group"] is None and p2["a_rows"] is None, k,
+              "partial sums are for plain products into float32")
+        splits = lib.tq_gemm_mfma_pair_splits(dims[0][1], dims[0][2], int(probs[0]["tile_group"] is not None),
+                                              dims[1][1], dims[1][2], 0)
     for p, (M, N, K, tile_rows, gstride) in zip(probs, dims):
-        out = torch.empty((M, N), dtype=adt if p["out_act"] else torch.float32, device=p["a"].device)
+        shape = (splits, M, N) if p["partial_sums"] else (M, N)
+        out = torch.empty(shape, dtype=adt if p["out_act"] else torch.float32, device=p["a"].device)
         outs.append(out)
         vals = [_ptr(p["a"]), p["a"].stride(0), _ptr(p["a_rows"]), int(p["gather"]), _ptr(p["w"]), _ptr(p["w2"]), gstride,
                 _ptr(p["tile_group"]), _ptr(p["n_tiles"]), _ptr(p["bias"]),
                 _WTYPE[p["bias"].dtype] if p["bias"] is not None else 0, _ptr(out), N, int(p["out_act"]), M, N, K, tile_rows]
         descs.append((ctypes.c_int64 * 18)(*[0 if v is None else int(v) for v in vals]))
-    _run(k, lib.tq_gemm_mfma_pair(descs[0], descs[1], _stream()))
+    _run(k, lib.tq_gemm_mfma_pair(descs[0], descs[1], splits, _stream()))
     return outs[0], outs[1]
 
 

@@ -73,8 +73,8 @@ class SparseMoE(Part):
             h, hs = ops.gemm_pair(dict(a=normed, w=self.expert_gate, w2=self.expert_up, out_act=True, **experts),
                                   dict(a=normed, w=self.shared_gate, w2=self.shared_up, out_act=True), ctx.act)
             y, shared = ops.gemm_pair(dict(a=h, w=self.expert_down, gather=False, **experts),
-                                      dict(a=hs, w=self.shared_down), ctx.act)
-            return ops.GatheredSum(y, pair_slot, weights, shared.unsqueeze(0), gate)
+                                      dict(a=hs, w=self.shared_down, partial_sums=True), ctx.act)
+            return ops.GatheredSum(y, pair_slot, weights, shared, gate)
         # the shared expert needs nothing from the router: it may run on a second stream beside the routed experts
         shared, side = None, None
         if self.shared_size > 0:
