@@ -5,8 +5,10 @@
 //
 //  * gemm_stream_kernel, for few rows (decoding): the work is reading w once.  A wave owns 16 rows of w
 //    and streams them straight from memory into the operand registers of v_mfma_f32_16x16x32_bf16 (lane
-//    l holds 8 consecutive k of row l % 16: four lanes read 64 contiguous bytes of a row); the few rows of
-//    `a` are read the same way and stay in cache.  The waves of a workgroup split k among them and
+//    l holds 8 consecutive k of row l % 16).  The loads take whole lines of 128 bytes, eight lanes to a row, with
+//    the hint that the bytes are read once, and pairs of lanes then exchange registers: half lines per
+//    instruction, which the operand layout would give by itself, read a quarter slower.  The few rows of `a`
+//    are read the same way, without the hint, and stay in cache.  The waves of a workgroup split k among them and
 //    add their partial sums in wave order through LDS, so that even a narrow matrix gives the chip enough
 //    waves and bytes in flight.  How k is split depends on N and K only, never on the number of rows.
 //  * gemm_tile_kernel, for many rows (prompts): tiles of BM x 128 outputs by eight waves, 64 of k at a time staged
@@ -45,13 +47,25 @@ struct MfmaGemmArgs {
 
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
 
-__device__ __forceinline__ bf16x8 load8(const bf16_t* p) {
-  const uint4 v = *reinterpret_cast<const uint4*>(p);
-  return __builtin_bit_cast(bf16x8, v);
+// For bytes that are read once (a matrix streamed past a few rows): a load that tells the caches so.  Measured on
+// a plain read of 1 GiB whose instructions take whole lines of 128 bytes: 6.8 TB/s with this hint, 4.7 without; with
+// half lines per instruction (16 rows x 64 bytes, the operand layout of the 16x16x32 product) 5.7.
+__device__ __forceinline__ u32x4 load16_once(const bf16_t* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
 }
-__device__ __forceinline__ bf16x8 zero8() {
-  const uint4 v = make_uint4(0, 0, 0, 0);
-  return __builtin_bit_cast(bf16x8, v);
+// Lanes l and l ^ 8 (the same quarter c = l / 16, rows r and r ^ 8 of a tile of 16 rows) fetched whole lines: lane
+// (r, c) chunk c + 4 (r / 8) of row r % 8 into t0 and of row 8 + r % 8 into t1.  Afterwards t0 is chunk c and t1
+// chunk c + 4 of the lane's own row r: the operands of two consecutive 16x16x32 products.
+__device__ __forceinline__ void to_own_row(u32x4& t0, u32x4& t1) {
+  u32x4 s0, s1;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    // row_ror:8 reads lane l ^ 8 of each row of 16 lanes; the bank mask says which lanes take it (0xc: 8..15, 0x3: 0..7)
+    s0[i] = __builtin_amdgcn_update_dpp(t0[i], t1[i], 0x128, 0xf, 0xc, false);
+    s1[i] = __builtin_amdgcn_update_dpp(t1[i], t0[i], 0x128, 0xf, 0x3, false);
+  }
+  t0 = s0;
+  t1 = s1;
 }
 
 __device__ __forceinline__ float bias_at(const MfmaGemmArgs& g, int n) {
@@ -85,22 +99,24 @@ __device__ __forceinline__ void stream_body(MfmaGemmArgs g, int tile_n, int tile
   const int n0 = tile_n * 16, m0 = tile_m * 16 * MT;
   const int n = n0 + r;
   const bool n_ok = n < g.N;
-  const bf16_t* wp = g.w + (size_t)group * g.group_stride + (size_t)(n_ok ? n : 0) * g.K + c * 8;
-  const bf16_t* vp = DUAL ? g.w2 + (size_t)group * g.group_stride + (size_t)(n_ok ? n : 0) * g.K + c * 8 : nullptr;
-  const bf16_t* ap[MT];
+  // the rows of `a` that this lane fetches: r % 8 and 8 + r % 8 of each tile of 16 (as with w below)
+  const int q = c + 4 * (r / 8);            // and the chunk of 8 within each 64 of k
+  const bf16_t* ap[MT][2];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const int m = m0 + mt * 16 + r;
-    int src = -1;
-    if (m < g.M) {
-      src = g.a_rows ? g.a_rows[m] : m;
-      if (src >= 0 && !g.a_gather) src = m;
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      const int m = m0 + mt * 16 + 8 * hf + r % 8;
+      int src = -1;
+      if (m < g.M) {
+        src = g.a_rows ? g.a_rows[m] : m;
+        if (src >= 0 && !g.a_gather) src = m;
+      }
+      ap[mt][hf] = src >= 0 ? g.a + (size_t)src * g.lda + q * 8 : nullptr;
     }
-    ap[mt] = src >= 0 ? g.a + (size_t)src * g.lda + c * 8 : nullptr;
-  }
-  // this wave's share of k, in steps of 32
+  // this wave's share of k, in steps of 32; an even number of them, so that every pair of steps is a line of w
   const int steps = (k_hi - k_lo + 31) / 32;
-  const int per = (steps + nw - 1) / nw;
+  const int per = ((steps + nw - 1) / nw + 1) & ~1;
   const int k_beg = k_lo + wave * per * 32, k_end = min(k_hi, k_lo + (wave + 1) * per * 32);
 
   f32x4 acc[MT], acc2[DUAL ? MT : 1];
@@ -110,32 +126,50 @@ __device__ __forceinline__ void stream_body(MfmaGemmArgs g, int tile_n, int tile
     if (DUAL) acc2[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
   // U steps of 32 at a time, every load issued before the first product, so that a wave keeps U (2U with the
-  // gated pair) kilobytes of w in flight.  Rows that do not exist read row 0 instead (what they produce is never
-  // stored); steps beyond the wave's share or beyond K load nothing and multiply zeros.
+  // gated pair) kilobytes of w in flight.  w and a are fetched by whole lines: for each pair of steps (64 of k,
+  // 128 bytes of a row) eight lanes take a row, one instruction the tile's rows 0..7 and the next rows 8..15,
+  // and lanes l and l ^ 8 then exchange what belongs to the other's row.  Rows of w that do not exist read row 0
+  // instead (what they produce is never stored); rows of a that do not exist, and chunks beyond the wave's
+  // share or beyond K, load nothing and multiply zeros.
   constexpr int U = (DUAL ? 4 : 8) / (MT == 4 ? 2 : 1);
   {
-    const bf16_t* wq = n_ok ? wp : g.w + (size_t)group * g.group_stride + c * 8;
-    const bf16_t* vq = DUAL ? (n_ok ? vp : g.w2 + (size_t)group * g.group_stride + c * 8) : nullptr;
-    const bf16_t* aq[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) aq[mt] = ap[mt] ? ap[mt] : g.a + c * 8;
+    const int n_a = n0 + r % 8, n_b = n_a + 8;
+    const size_t row_a = (size_t)group * g.group_stride + (size_t)(n_a < g.N ? n_a : 0) * g.K + q * 8;
+    const size_t row_b = (size_t)group * g.group_stride + (size_t)(n_b < g.N ? n_b : 0) * g.K + q * 8;
+    const u32x4 zero = {0u, 0u, 0u, 0u};
     for (int k = k_beg; k < k_end; k += 32 * U) {
-      bf16x8 wf[U], vf[DUAL ? U : 1], af[MT][U];
+      u32x4 wf[U], vf[DUAL ? U : 1];
+      u32x4 af[MT][U];
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int ku = k + 32 * u;
-        const bool ok = ku < k_end && ku + c * 8 < g.K;   // K is a multiple of 8: a chunk of 8 is in or out as a whole
-        wf[u] = ok ? load8(wq + ku) : zero8();
-        if (DUAL) vf[u] = ok ? load8(vq + ku) : zero8();
+      for (int j = 0; j < U / 2; ++j) {
+        const int kp = k + 64 * j;
+        const bool okw = kp + q * 8 < k_end;      // k_end <= K, both multiples of 8: a chunk is in or out as a whole
+        wf[2 * j] = okw ? load16_once(g.w + row_a + kp) : zero;
+        wf[2 * j + 1] = okw ? load16_once(g.w + row_b + kp) : zero;
+        if (DUAL) {
+          vf[2 * j] = okw ? load16_once(g.w2 + row_a + kp) : zero;
+          vf[2 * j + 1] = okw ? load16_once(g.w2 + row_b + kp) : zero;
+        }
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) af[mt][u] = ok ? load8(aq[mt] + ku) : zero8();
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int hf = 0; hf < 2; ++hf)
+            af[mt][2 * j + hf] = okw && ap[mt][hf] ? *reinterpret_cast<const u32x4*>(ap[mt][hf] + kp) : zero;
+      }
+#pragma unroll
+      for (int j = 0; j < U / 2; ++j) {
+        to_own_row(wf[2 * j], wf[2 * j + 1]);
+        if (DUAL) to_own_row(vf[2 * j], vf[2 * j + 1]);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) to_own_row(af[mt][2 * j], af[mt][2 * j + 1]);
       }
 #pragma unroll
       for (int u = 0; u < U; ++u)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mt][u], wf[u], acc[mt], 0, 0, 0);
-          if (DUAL) acc2[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mt][u], vf[u], acc2[mt], 0, 0, 0);
+          const bf16x8 ax = __builtin_bit_cast(bf16x8, af[mt][u]);
+          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax, __builtin_bit_cast(bf16x8, wf[u]), acc[mt], 0, 0, 0);
+          if (DUAL) acc2[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax, __builtin_bit_cast(bf16x8, vf[u]), acc2[mt], 0, 0, 0);
         }
     }
   }
@@ -513,7 +547,7 @@ TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gat
 static int pair_run_of_k(int N1, int K1, bool grouped1, int N2, int K2, bool grouped2) {
   const int nw = split_k_waves(N1, K1, grouped1), nw2 = split_k_waves(N2, K2, grouped2);
   if (nw2 <= nw) return K2;
-  return ((K2 + 31) / 32 + nw2 / nw - 1) / (nw2 / nw) * 32;      // a multiple of 32
+  return ((K2 + 63) / 64 + nw2 / nw - 1) / (nw2 / nw) * 64;      // a multiple of 64: runs start at whole lines
 }
 TQ_API int tq_gemm_mfma_pair_splits(int N1, int K1, int grouped1, int N2, int K2, int grouped2) {
   const int k_per = pair_run_of_k(N1, K1, grouped1 != 0, N2, K2, grouped2 != 0);
