@@ -17,7 +17,7 @@
 //
 // Two entry points share this: whole prompts (columns = 16 consecutive tokens of a sequence, one head; four
 // waves per workgroup) and decoding (columns = the query heads that share one kv head, one token; the cache is
-// split into runs of 1 to 4 tiles, one wave each, and a second kernel joins the runs in order).  Tiles start at
+// split into runs of 1 to 3 tiles, one wave each, and a second kernel joins the runs in order).  Tiles start at
 // multiples of 64 positions and runs at multiples of the run length, so the order of every sum depends only on
 // the token's own position.
 #include "common.h"
@@ -30,13 +30,14 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 #define TILE 64
 #define LOG2E 1.4426950408889634f
 // Tiles per run when decoding a token at position p: short sequences are cut finer, so that a small batch still
-// gives the chip hundreds of waves; a function of the token's own position only.
-__host__ __device__ __forceinline__ int tiles_per_run(int p) { return p >= 3 * 2048 ? 4 : p / 2048 + 1; }
+// gives the chip hundreds of waves; a function of the token's own position only.  Measured at position 8191 with
+// 16 kv heads: 3 tiles per run beat 4 by 15 % at 8 sequences and lose 2 to 4 % from 16 on.
+__host__ __device__ __forceinline__ int tiles_per_run(int p) { return p >= 2 * 2048 ? 3 : p / 2048 + 1; }
 // Most runs that a token at a position below max_end can have.
 static int most_runs(int max_end) {
   const int tiles = (max_end + 63) / 64;
-  const int short_runs = tiles < 32 ? tiles : 32;          // below position 6144 no token has more than 32
-  const int long_runs = (tiles + 3) / 4;
+  const int short_runs = tiles < 32 ? tiles : 32;          // below position 4096 no token has more than 32
+  const int long_runs = (tiles + 2) / 3;
   return short_runs > long_runs ? short_runs : long_runs;
 }
 
@@ -451,7 +452,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DT > 8 ? 2 :
 // Joins the runs of one (sequence, head) in order of position: grid (nh, B), block 64.  The weights
 // 2^(m_s - m) of the runs are worked out once, a lane per run, and kept in LDS; then every lane sums its
 // dimensions over the runs in order.
-#define MAX_RUNS_LDS 1024
+#define MAX_RUNS_LDS 2048
 __global__ __launch_bounds__(64) void attn_join_kernel(AttnArgs a) {
   __shared__ float wgt[MAX_RUNS_LDS];
   const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
