@@ -80,18 +80,44 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const float* __restric
   if (vec) {
 #pragma unroll 2
     for (int i = threadIdx.x * 4; i < H; i += blockDim.x * 4) {
+      // the terms are fetched four at a time and added in their order: the loads of a group are on their way
+      // together instead of one after the other
       f32x4 a = load4f(xr + i);
       if (y) {
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-        for (int j = 0; j < topk; ++j) acc += wgt[j] * load4f(y + (size_t)slot[j] * H + i);
+        for (int j = 0; j < topk; j += 4) {
+          f32x4 t[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            if (j + u < topk) t[u] = load4f(y + (size_t)slot[j + u] * H + i);
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            if (j + u < topk) acc += wgt[j + u] * t[u];
+        }
         if (S > 0) {
           f32x4 sh = {0.f, 0.f, 0.f, 0.f};
-          for (int s = 0; s < S; ++s) sh += load4f(dr + s * delta_stride + i);
+          for (int s = 0; s < S; s += 4) {
+            f32x4 t[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+              if (s + u < S) t[u] = load4f(dr + (s + u) * delta_stride + i);
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+              if (s + u < S) sh += t[u];
+          }
           acc += g * sh;
         }
         a += acc;
       } else {
-        for (int s = 0; s < S; ++s) a += load4f(dr + s * delta_stride + i);
+        for (int s = 0; s < S; s += 4) {
+          f32x4 t[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            if (s + u < S) t[u] = load4f(dr + (s + u) * delta_stride + i);
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            if (s + u < S) a += t[u];
+        }
       }
       store4(v + i, a);
       if (!rows) store4(xr + i, a);
