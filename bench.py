@@ -85,6 +85,7 @@ def main() -> int:
     from turboquant_cpp_amd.csrc import ops
     from turboquant_cpp_amd.engine.model import random_model
     from turboquant_cpp_amd.engine.step import Engine
+    from turboquant_cpp_amd.sampling.sampler import TokenFetch
 
     cfg = dict(A27B)
     cfg["num_hidden_layers"] = args.layers
@@ -118,11 +119,16 @@ def main() -> int:
             logits = lg if logits is None else torch.cat([logits, lg])
         torch.cuda.synchronize()
         print(f"[bench] prefilled {batch} x {prompt_len} tokens in {time.time() - tp:.1f}s", file=sys.stderr, flush=True)
-        tokens = ops.argmax(logits, act).tolist()
+        tokens = ops.argmax(logits, act)
+        fetch = TokenFetch(dev, batch)
 
-        def one_step(tokens):
-            lg = engine.step(slots, [[t] for t in tokens])
-            return ops.argmax(lg, act).tolist()
+        def one_step(ids):
+            """As the generation loop does it: the step is issued from the tokens on the device, and the host
+            reads those tokens (to look for end tokens) while the step runs."""
+            fetch.start(ids)
+            lg = engine.step_from_device(slots, ids)
+            fetch.wait()
+            return ops.argmax(lg, act)
 
         # the first warm-up step (which runs eagerly) also counts the distinct experts that each layer's router picks
         picked = []

@@ -189,6 +189,39 @@ def test_first_tokens_and_long_decoding(name, act, engines):
 
 
 @pytest.mark.parametrize("act", ACTS)
+def test_a_step_fed_from_the_device_is_the_step_fed_from_the_host(act, sharp_dirs):
+    """Decode steps whose tokens come from a tensor on the device (eager, captured, replayed) give the bits of the
+    same steps fed from lists, and the tokens come back to the host through the fetch."""
+    from turboquant_cpp_amd.engine.model import load_model
+    from turboquant_cpp_amd.engine.step import Engine
+    from turboquant_cpp_amd.sampling.sampler import TokenFetch
+    d, _ = sharp_dirs("B", act)
+    model = load_model(d, act=act, device=DEV)
+    prompts = prompts_for("B", [9, 30, 17], seed=31)
+    feed = prompts_for("B", [6, 6, 6], seed=32)
+    out = {}
+    for how in ("host", "device"):
+        eng = Engine(model, max_tokens=64 * 6)
+        slots = eng.open(3)
+        eng.step(slots, prompts)
+        fetch = TokenFetch(eng.device, 3)
+        rows = []
+        for t in range(6):
+            toks = [f[t] for f in feed]
+            if how == "host":
+                rows.append(eng.step(slots, [[x] for x in toks]).clone())
+            else:
+                ids = torch.tensor(toks, dtype=torch.int32, device=DEV)
+                fetch.start(ids)
+                lg = eng.step_from_device(slots, ids)
+                assert fetch.wait() == toks
+                rows.append(lg.clone())
+        eng.close(slots)
+        out[how] = torch.stack(rows)
+    assert torch.equal(out["host"], out["device"])
+
+
+@pytest.mark.parametrize("act", ACTS)
 def test_a_request_does_not_feel_its_batch_or_its_place_in_the_cache(act, engines):
     """Alone in a fresh cache, then among others after the cache has been used and its pages handed round:
     the same logits, far inside what bfloat16 rounding allows."""

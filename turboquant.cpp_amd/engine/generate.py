@@ -14,7 +14,9 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Callable, Sequence
 
-from ..sampling.sampler import Sampler, SamplingOptions
+import torch
+
+from ..sampling.sampler import Sampler, SamplingOptions, TokenFetch
 
 
 @dataclass
@@ -76,6 +78,11 @@ class SequenceTrack:
     detector: LoopDetector = field(default_factory=LoopDetector)
     finish_reason: str | None = None
 
+    def room_after_next(self) -> bool:
+        """Whether the sequence can go on after its next token, as far as that does not depend on the token:
+        neither the number of tokens asked for nor the positions are used up by it."""
+        return len(self.out) + 1 < self.options.max_tokens and self.prompt_len + len(self.out) + 1 < self.max_positions
+
     def accept(self, token: int) -> bool:
         """Takes the sampled token.  Returns True if the token is to be run through the model next,
         False if the sequence has ended (``finish_reason`` says why)."""
@@ -130,21 +137,36 @@ def generate(engine, prompts: Sequence[Sequence[int]], options: GenerationOption
         samp = {r: sampler.new_sequence(r, list(prompts[r])) for r in batch}
         slot_of = dict(zip(batch, slots))
         live = list(batch)
+        fetch = TokenFetch(engine.device, len(batch))
         try:
             logits = engine.step([slot_of[r] for r in live], [list(prompts[r]) for r in live])
             while True:
-                tokens = sampler.sample(logits, [samp[r] for r in live])
+                states = [samp[r] for r in live]
+                ids = sampler.launch(logits, states)
+                fetch.start(ids)
+                # The next step is issued before the host has seen these tokens, for every sequence that can
+                # go on whatever its token is; the host then reads the tokens while that step runs.  A sequence
+                # that ends on this token (an end token, a loop) has run one step in vain.
+                ahead = [i for i, r in enumerate(live) if tracks[r].room_after_next()]
+                next_logits = None
+                if ahead:
+                    feed = ids if len(ahead) == len(live) else ids[torch.tensor(ahead, dtype=torch.int64, device=ids.device)]
+                    next_logits = engine.step_from_device([slot_of[live[i]] for i in ahead], feed)
+                tokens = fetch.wait()
+                sampler.finish(tokens, states)
                 going = []
-                for r, t in zip(live, tokens):
+                for i, (r, t) in enumerate(zip(live, tokens)):
                     if tracks[r].accept(t):
-                        going.append((r, t))
+                        going.append(i)
                     else:
                         engine.close([slot_of.pop(r)])
                         results[r] = GenerationResult(tracks[r].out, tracks[r].finish_reason)
                 if not going:
                     break
-                live = [r for r, _ in going]
-                logits = engine.step([slot_of[r] for r in live], [[t] for _, t in going])
+                rows = [ahead.index(i) for i in going]       # a sequence that goes on was run ahead
+                logits = next_logits if rows == list(range(len(ahead))) else \
+                    next_logits[torch.tensor(rows, dtype=torch.int64, device=next_logits.device)]
+                live = [live[i] for i in going]
         finally:
             engine.close(list(slot_of.values()))
     return results

@@ -45,15 +45,20 @@ class DecodeGraph:
         self.pool = pool
 
     def fill(self, slots, starts, tokens) -> None:
+        """``tokens``: a list, or an int32 tensor on the device that is copied in behind the other arrays."""
         self.copied.synchronize()          # the last copy out of the pinned array has been done
         h, off = self.host_np, self.offsets
-        h[off["tokens"][0]:off["tokens"][1]] = tokens
+        on_device = isinstance(tokens, torch.Tensor)
+        if not on_device:
+            h[off["tokens"][0]:off["tokens"][1]] = tokens
         h[off["positions"][0]:off["positions"][1]] = starts
         h[off["slot_of_token"][0]:off["slot_of_token"][1]] = slots
         h[off["slots"][0]:off["slots"][1]] = slots
         h[off["start"][0]:off["start"][1]] = starts
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
+        if on_device:
+            self.views["tokens"].copy_(tokens)
 
     def batch(self, slots, starts) -> StepBatch:
         v = self.views

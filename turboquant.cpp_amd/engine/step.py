@@ -77,17 +77,7 @@ class Engine:
             bad = [t for t in toks if not 0 <= t < V]
             if bad:
                 raise StepError(f"sequence {i} brings token {bad[0]}, outside the vocabulary of {V}")
-        starts, reserved = [], []
-        try:
-            for slot, toks in zip(slots, token_lists):
-                starts.append(self.cache.reserve(slot, len(toks)))
-                reserved.append(slot)
-        except CacheError:
-            for slot in reserved:
-                s = self.cache.slots[slot]
-                s.reserved = 0
-            raise
-        self.cache.sync()
+        starts = self._reserve(slots, [len(t) for t in token_lists])
         logits = None
         if self.graphs is not None and all(len(t) == 1 for t in token_lists):
             for i, w in enumerate(wants):
@@ -100,12 +90,48 @@ class Engine:
                     all_rows[torch.tensor(rows, dtype=torch.int64, device=self.device)] if rows else \
                     torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
         if logits is None:
-            batch = pack_step(slots, starts, token_lists, wants, self.device)
-            # a second stream pays when kernels are short; a long prompt's products fill the chip one at a time
-            few = sum(len(t) for t in token_lists) <= 256
-            ctx = StepContext(batch=batch, cache=self.cache, act=self.model.act, device=self.device,
-                              side_stream=self.side_stream if few else None)
-            logits = self.model.forward(ctx)
+            logits = self._eager(pack_step(slots, starts, token_lists, wants, self.device))
         for slot in slots:
             self.cache.commit(slot)
         return logits
+
+    def step_from_device(self, slots: list[int], tokens: torch.Tensor) -> torch.Tensor:
+        """A decode step whose tokens are already on the device: ``tokens`` int32 [len(slots)], one for each
+        sequence, each inside the vocabulary (as a sampler's output is; nothing checks it here).  The host
+        need not have seen the tokens, so the step can be issued while the choice of these tokens is still
+        running.  Returns the logits of every sequence, [len(slots), vocab]; they may live in memory that the
+        next step of the same shape overwrites, so use them (or copy them) before that step is issued."""
+        if not slots or len(set(slots)) != len(slots):
+            raise StepError("a step needs at least one slot, and each only once")
+        if tokens.dtype != torch.int32 or tuple(tokens.shape) != (len(slots),) or \
+                (self.device is not None and tokens.device != torch.device(self.device)):
+            raise StepError(f"tokens must be int32 [{len(slots)}] on the model's device")
+        starts = self._reserve(slots, [1] * len(slots))
+        logits = self.graphs.run(slots, starts, tokens) if self.graphs is not None else None
+        if logits is None:
+            batch = pack_step(slots, starts, [[0]] * len(slots), [[0]] * len(slots), self.device)
+            batch.tokens.copy_(tokens)
+            logits = self._eager(batch)
+        for slot in slots:
+            self.cache.commit(slot)
+        return logits
+
+    def _reserve(self, slots, counts) -> list[int]:
+        """Room for ``counts[i]`` more positions in each slot, or none at all; returns where each sequence goes on."""
+        starts, reserved = [], []
+        try:
+            for slot, n in zip(slots, counts):
+                starts.append(self.cache.reserve(slot, n))
+                reserved.append(slot)
+        except CacheError:
+            for slot in reserved:
+                self.cache.slots[slot].reserved = 0
+            raise
+        self.cache.sync()
+        return starts
+
+    def _eager(self, batch) -> torch.Tensor:
+        # a second stream pays when kernels are short; a long prompt's products fill the chip one at a time
+        ctx = StepContext(batch=batch, cache=self.cache, act=self.model.act, device=self.device,
+                          side_stream=self.side_stream if batch.n_tokens <= 256 else None)
+        return self.model.forward(ctx)

@@ -53,6 +53,13 @@ class Sampler:
     def sample(self, logits: torch.Tensor, states: list[SequenceSampling]) -> list[int]:
         """One token per row of ``logits`` [R, V]; row i belongs to ``states[i]``.  Changes ``logits``
         when a repetition penalty applies."""
+        out = self.launch(logits, states).tolist()
+        self.finish(out, states)
+        return out
+
+    def launch(self, logits: torch.Tensor, states: list[SequenceSampling]) -> torch.Tensor:
+        """Issues the choice and returns the tokens as int32 [R] on the device; ``finish`` must be told the
+        tokens before the next ``launch`` for the same sequences."""
         o, R = self.options, logits.shape[0]
         if o.rep_penalty > 1.0 and self.window > 0:
             recent = np.full((R, self.window), -1, dtype=np.int32)
@@ -64,11 +71,36 @@ class Sampler:
             ops.rep_penalty(logits, torch.from_numpy(recent).to(self.device), torch.from_numpy(counts).to(self.device),
                             o.rep_penalty, self.act)
         if o.greedy:
-            ids = ops.argmax(logits, self.act)
-        else:
-            u = np.array([st.rng.next_float() for st in states], dtype=np.float32)
-            ids = ops.sample_topp(logits, o.temperature, o.top_p, torch.from_numpy(u).to(self.device), self.act)
-        out = ids.tolist()
-        for st, t in zip(states, out):
+            return ops.argmax(logits, self.act)
+        u = np.array([st.rng.next_float() for st in states], dtype=np.float32)
+        return ops.sample_topp(logits, o.temperature, o.top_p, torch.from_numpy(u).to(self.device), self.act)
+
+    def finish(self, tokens: list[int], states: list[SequenceSampling]) -> None:
+        for st, t in zip(states, tokens):
             st.push(t, self.window)
-        return out
+
+
+class TokenFetch:
+    """Brings a step's chosen tokens to the host without waiting for what is issued after them: on a GPU the copy
+    into pinned memory is issued right behind the choice, with an event behind it, and ``wait`` waits for that
+    event only; a step issued between ``start`` and ``wait`` runs while the host looks at the tokens."""
+
+    def __init__(self, device, capacity: int):
+        self.on_gpu = device is not None and torch.device(device).type == "cuda"
+        if self.on_gpu:
+            self.host = torch.empty(capacity, dtype=torch.int32).pin_memory()
+            self.done = torch.cuda.Event()
+        self.pending = None
+
+    def start(self, ids: torch.Tensor) -> None:
+        if self.on_gpu:
+            self.host[:ids.numel()].copy_(ids, non_blocking=True)
+            self.done.record()
+        self.pending = ids
+
+    def wait(self) -> list[int]:
+        ids, self.pending = self.pending, None
+        if not self.on_gpu:
+            return ids.tolist()
+        self.done.synchronize()
+        return self.host[:ids.numel()].tolist()
