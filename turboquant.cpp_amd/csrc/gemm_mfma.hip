@@ -82,10 +82,12 @@ __device__ __forceinline__ void store_out(const MfmaGemmArgs& g, int m, int n, f
 }
 
 // ------------------------------------------------------------------------------------------ few rows
-// A workgroup of 64 * (waves that split k) threads takes column tile `tile_n` (16 columns) of row tile `tile_m`
-// (16 * MT rows) over run `z` of k (k_per long; run 0 is all of k unless the product is split into partial
-// sums); red: LDS of [waves][MT * (DUAL ? 2 : 1)][4][64] floats.
-template <int MT, bool DUAL, bool OUT_ACT>
+// A workgroup of 64 * (waves that split k) threads takes column tile `tile_n` (16 * NTL columns) of row tile
+// `tile_m` (16 * MT rows) over run `z` of k (k_per long; run 0 is all of k unless the product is split into
+// partial sums); red: LDS of [waves][NTL * MT * (DUAL ? 2 : 1)][4][64] floats.  What a wave reads of `a` serves
+// its NTL tiles of 16 columns: with many rows the way of `a` from L2 into the compute unit is what binds, and two
+// column tiles per wave halve it.
+template <int MT, bool DUAL, bool OUT_ACT, int NTL = 1>
 __device__ __forceinline__ void stream_body(MfmaGemmArgs g, int tile_n, int tile_m, int z, float* red) {
   if (g.n_tiles && tile_m >= g.n_tiles[0]) return;
   const int k_lo = z * g.k_per, k_hi = min(g.K, k_lo + g.k_per);
@@ -96,9 +98,7 @@ __device__ __forceinline__ void stream_body(MfmaGemmArgs g, int tile_n, int tile
   const int group = g.tile_group ? g.tile_group[tile_m] : 0;
   const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, nw = blockDim.x / 64;
   const int r = lane % 16, c = lane / 16;
-  const int n0 = tile_n * 16, m0 = tile_m * 16 * MT;
-  const int n = n0 + r;
-  const bool n_ok = n < g.N;
+  const int n0 = tile_n * 16 * NTL, m0 = tile_m * 16 * MT;
   // the rows of `a` that this lane fetches: r % 8 and 8 + r % 8 of each tile of 16 (as with w below)
   const int q = c + 4 * (r / 8);            // and the chunk of 8 within each 64 of k
   const bf16_t* ap[MT][2];
@@ -119,36 +119,46 @@ __device__ __forceinline__ void stream_body(MfmaGemmArgs g, int tile_n, int tile
   const int per = ((steps + nw - 1) / nw + 1) & ~1;
   const int k_beg = k_lo + wave * per * 32, k_end = min(k_hi, k_lo + (wave + 1) * per * 32);
 
-  f32x4 acc[MT], acc2[DUAL ? MT : 1];
+  f32x4 acc[NTL][MT], acc2[DUAL ? NTL : 1][DUAL ? MT : 1];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-    if (DUAL) acc2[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  }
+  for (int t = 0; t < NTL; ++t)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      acc[t][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (DUAL) acc2[t][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
   // U steps of 32 at a time, every load issued before the first product, so that a wave keeps U (2U with the
-  // gated pair) kilobytes of w in flight.  w and a are fetched by whole lines: for each pair of steps (64 of k,
-  // 128 bytes of a row) eight lanes take a row, one instruction the tile's rows 0..7 and the next rows 8..15,
-  // and lanes l and l ^ 8 then exchange what belongs to the other's row.  Rows of w that do not exist read row 0
-  // instead (what they produce is never stored); rows of a that do not exist, and chunks beyond the wave's
-  // share or beyond K, load nothing and multiply zeros.
-  constexpr int U = (DUAL ? 4 : 8) / (MT == 4 ? 2 : 1);
+  // gated pair) kilobytes of w in flight per column tile.  w and a are fetched by whole lines: for each pair of
+  // steps (64 of k, 128 bytes of a row) eight lanes take a row, one instruction the tile's rows 0..7 and the next
+  // rows 8..15, and lanes l and l ^ 8 then exchange what belongs to the other's row.  Rows of w that do not exist
+  // read row 0 instead (what they produce is never stored); rows of a that do not exist, and chunks beyond the
+  // wave's share or beyond K, load nothing and multiply zeros.
+  constexpr int U_ONE = (DUAL ? 4 : 8) / (MT == 4 ? 2 : 1);
+  constexpr int U = U_ONE / NTL >= 2 ? U_ONE / NTL : 2;
   {
-    const int n_a = n0 + r % 8, n_b = n_a + 8;
-    const size_t row_a = (size_t)group * g.group_stride + (size_t)(n_a < g.N ? n_a : 0) * g.K + q * 8;
-    const size_t row_b = (size_t)group * g.group_stride + (size_t)(n_b < g.N ? n_b : 0) * g.K + q * 8;
+    size_t row_a[NTL], row_b[NTL];
+#pragma unroll
+    for (int t = 0; t < NTL; ++t) {
+      const int n_a = n0 + 16 * t + r % 8, n_b = n_a + 8;
+      row_a[t] = (size_t)group * g.group_stride + (size_t)(n_a < g.N ? n_a : 0) * g.K + q * 8;
+      row_b[t] = (size_t)group * g.group_stride + (size_t)(n_b < g.N ? n_b : 0) * g.K + q * 8;
+    }
     const u32x4 zero = {0u, 0u, 0u, 0u};
     for (int k = k_beg; k < k_end; k += 32 * U) {
-      u32x4 wf[U], vf[DUAL ? U : 1];
+      u32x4 wf[NTL][U], vf[DUAL ? NTL : 1][DUAL ? U : 1];
       u32x4 af[MT][U];
 #pragma unroll
       for (int j = 0; j < U / 2; ++j) {
         const int kp = k + 64 * j;
         const bool okw = kp + q * 8 < k_end;      // k_end <= K, both multiples of 8: a chunk is in or out as a whole
-        wf[2 * j] = okw ? load16_once(g.w + row_a + kp) : zero;
-        wf[2 * j + 1] = okw ? load16_once(g.w + row_b + kp) : zero;
-        if (DUAL) {
-          vf[2 * j] = okw ? load16_once(g.w2 + row_a + kp) : zero;
-          vf[2 * j + 1] = okw ? load16_once(g.w2 + row_b + kp) : zero;
+#pragma unroll
+        for (int t = 0; t < NTL; ++t) {
+          wf[t][2 * j] = okw ? load16_once(g.w + row_a[t] + kp) : zero;
+          wf[t][2 * j + 1] = okw ? load16_once(g.w + row_b[t] + kp) : zero;
+          if (DUAL) {
+            vf[t][2 * j] = okw ? load16_once(g.w2 + row_a[t] + kp) : zero;
+            vf[t][2 * j + 1] = okw ? load16_once(g.w2 + row_b[t] + kp) : zero;
+          }
         }
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
@@ -158,8 +168,11 @@ __device__ __forceinline__ void stream_body(MfmaGemmArgs g, int tile_n, int tile
       }
 #pragma unroll
       for (int j = 0; j < U / 2; ++j) {
-        to_own_row(wf[2 * j], wf[2 * j + 1]);
-        if (DUAL) to_own_row(vf[2 * j], vf[2 * j + 1]);
+#pragma unroll
+        for (int t = 0; t < NTL; ++t) {
+          to_own_row(wf[t][2 * j], wf[t][2 * j + 1]);
+          if (DUAL) to_own_row(vf[t][2 * j], vf[t][2 * j + 1]);
+        }
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) to_own_row(af[mt][2 * j], af[mt][2 * j + 1]);
       }
@@ -168,30 +181,37 @@ __device__ __forceinline__ void stream_body(MfmaGemmArgs g, int tile_n, int tile
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           const bf16x8 ax = __builtin_bit_cast(bf16x8, af[mt][u]);
-          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax, __builtin_bit_cast(bf16x8, wf[u]), acc[mt], 0, 0, 0);
-          if (DUAL) acc2[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax, __builtin_bit_cast(bf16x8, vf[u]), acc2[mt], 0, 0, 0);
+#pragma unroll
+          for (int t = 0; t < NTL; ++t) {
+            acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax, __builtin_bit_cast(bf16x8, wf[t][u]), acc[t][mt], 0, 0, 0);
+            if (DUAL)
+              acc2[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax, __builtin_bit_cast(bf16x8, vf[t][u]), acc2[t][mt], 0, 0, 0);
+          }
         }
     }
   }
   // The waves' partial sums are added in wave order, every thread of the workgroup taking some of the outputs.
-  constexpr int SETS = MT * (DUAL ? 2 : 1);
+  constexpr int PAIRS = NTL * MT;               // (column tile, row tile) pairs: set t * MT + mt, the gate's partner PAIRS on
+  constexpr int SETS = PAIRS * (DUAL ? 2 : 1);
   if (nw > 1) {
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+    for (int t = 0; t < NTL; ++t)
 #pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        red[((wave * SETS + mt) * 4 + v) * 64 + lane] = acc[mt][v];
-        if (DUAL) red[((wave * SETS + MT + mt) * 4 + v) * 64 + lane] = acc2[mt][v];
-      }
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          red[((wave * SETS + t * MT + mt) * 4 + v) * 64 + lane] = acc[t][mt][v];
+          if (DUAL) red[((wave * SETS + PAIRS + t * MT + mt) * 4 + v) * 64 + lane] = acc2[t][mt][v];
+        }
     __syncthreads();
-    for (int i = threadIdx.x; i < MT * 256; i += blockDim.x) {
-      const int ol = i % 64, v = (i / 64) % 4, mt = i / 256;
+    for (int i = threadIdx.x; i < PAIRS * 256; i += blockDim.x) {
+      const int ol = i % 64, v = (i / 64) % 4, pair = i / 256, mt = pair % MT, t = pair / MT;
       float s = 0.f, s2 = 0.f;
       for (int w = 0; w < nw; ++w) {
-        s += red[((w * SETS + mt) * 4 + v) * 64 + ol];
-        if (DUAL) s2 += red[((w * SETS + MT + mt) * 4 + v) * 64 + ol];
+        s += red[((w * SETS + pair) * 4 + v) * 64 + ol];
+        if (DUAL) s2 += red[((w * SETS + PAIRS + pair) * 4 + v) * 64 + ol];
       }
-      const int on = n0 + ol % 16, om = m0 + mt * 16 + 4 * (ol / 16) + v;
+      const int on = n0 + 16 * t + ol % 16, om = m0 + mt * 16 + 4 * (ol / 16) + v;
       if (on >= g.N || om >= g.M) continue;
       if (g.a_rows && g.a_rows[om] < 0) continue;
       float o = s + bias_at(g, on);
@@ -200,26 +220,31 @@ __device__ __forceinline__ void stream_body(MfmaGemmArgs g, int tile_n, int tile
     }
     return;
   }
-  if (!n_ok) return;
-  const float b = bias_at(g, n);
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
+  for (int t = 0; t < NTL; ++t) {
+    const int n = n0 + 16 * t + r;
+    if (n >= g.N) continue;
+    const float b = bias_at(g, n);
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      const int m = m0 + mt * 16 + 4 * c + v;
-      if (m >= g.M) continue;
-      if (g.a_rows && g.a_rows[m] < 0) continue;
-      float o = acc[mt][v] + b;
-      if (DUAL) o = silu_f(o) * acc2[mt][v];
-      store_out<OUT_ACT>(g, m, n, o);
-    }
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int m = m0 + mt * 16 + 4 * c + v;
+        if (m >= g.M) continue;
+        if (g.a_rows && g.a_rows[m] < 0) continue;
+        float o = acc[t][mt][v] + b;
+        if (DUAL) o = silu_f(o) * acc2[t][mt][v];
+        store_out<OUT_ACT>(g, m, n, o);
+      }
+  }
 }
 
-// grid (ceil(N / 16), row tiles of 16 * MT rows).
-template <int MT, bool DUAL, bool OUT_ACT>
-__global__ __launch_bounds__(1024) void gemm_stream_kernel(MfmaGemmArgs g) {
+// grid (ceil(N / (16 NTL)), row tiles of 16 * MT rows).  Two column tiles per wave need the registers of a
+// workgroup of at most 8 waves.
+template <int MT, bool DUAL, bool OUT_ACT, int NTL>
+__global__ __launch_bounds__(NTL > 1 ? 512 : 1024) void gemm_stream_kernel(MfmaGemmArgs g) {
   extern __shared__ float red[];
-  stream_body<MT, DUAL, OUT_ACT>(g, blockIdx.x, blockIdx.y, 0, red);
+  stream_body<MT, DUAL, OUT_ACT, NTL>(g, blockIdx.x, blockIdx.y, 0, red);
 }
 
 // Two products that do not depend on each other in one launch (decoding: the routed experts' product beside
@@ -445,20 +470,24 @@ static int split_k_waves(int N, int K, bool grouped) {
   return s;
 }
 
+// MT row tiles of 16; more than one (17 to 64 rows of one matrix) go with two column tiles per wave.
 template <int MT>
 static int launch_stream(const MfmaGemmArgs& g, bool dual, bool out_act, int row_tiles, hipStream_t st) {
-  const int nw = split_k_waves(g.N, g.K, g.tile_group != nullptr);
-  const dim3 grid((g.N + 15) / 16, row_tiles);
-  const size_t shmem = nw > 1 ? (size_t)nw * MT * (dual ? 2 : 1) * 4 * 64 * sizeof(float) : 0;
+  constexpr int NTL = MT > 1 ? 2 : 1;
+  int nw = split_k_waves((g.N + NTL - 1) / NTL, g.K, g.tile_group != nullptr);
+  const size_t per_wave = (size_t)NTL * MT * (dual ? 2 : 1) * 4 * 64 * sizeof(float);
+  while (nw > 1 && (nw * per_wave > 64 * 1024 || (NTL > 1 && nw > 8))) nw /= 2;
+  const dim3 grid((g.N + 16 * NTL - 1) / (16 * NTL), row_tiles);
+  const size_t shmem = nw > 1 ? nw * per_wave : 0;
   if (shmem > 64 * 1024) return TQ_ERR_UNSUPPORTED;
   if (dual && out_act)
-    hipLaunchKernelGGL((gemm_stream_kernel<MT, true, true>), grid, dim3(64 * nw), shmem, st, g);
+    hipLaunchKernelGGL((gemm_stream_kernel<MT, true, true, NTL>), grid, dim3(64 * nw), shmem, st, g);
   else if (dual)
-    hipLaunchKernelGGL((gemm_stream_kernel<MT, true, false>), grid, dim3(64 * nw), shmem, st, g);
+    hipLaunchKernelGGL((gemm_stream_kernel<MT, true, false, NTL>), grid, dim3(64 * nw), shmem, st, g);
   else if (out_act)
-    hipLaunchKernelGGL((gemm_stream_kernel<MT, false, true>), grid, dim3(64 * nw), shmem, st, g);
+    hipLaunchKernelGGL((gemm_stream_kernel<MT, false, true, NTL>), grid, dim3(64 * nw), shmem, st, g);
   else
-    hipLaunchKernelGGL((gemm_stream_kernel<MT, false, false>), grid, dim3(64 * nw), shmem, st, g);
+    hipLaunchKernelGGL((gemm_stream_kernel<MT, false, false, NTL>), grid, dim3(64 * nw), shmem, st, g);
   return 0;
 }
 
