@@ -297,6 +297,23 @@ def test_generate_matches_the_plain_loop_for_unequal_prompts_in_several_batches(
         assert eng.cache.n_live == 0
 
 
+def test_generate_runs_ahead_only_where_a_page_is_free(cpu_engine):
+    """Two pages, two sequences: after the prompts one sequence fills its page and the next step of both is
+    issued before their tokens are known, which finds no page free.  The loop then waits for the tokens; the
+    full sequence ends on its first token (an end token), gives its page back, and the other goes on into it."""
+    eng = cpu_engine("A", max_tokens=128, max_slots=2)
+    a, b = [3] * 60, [5] * 64
+    greedy = dict(temperature=0.0, rep_penalty=1.0, loop_detection=False)
+    first_of_b = generate(eng, [b], GenerationOptions(max_tokens=1, **greedy))[0].tokens[0]
+    alone = generate(eng, [a], GenerationOptions(max_tokens=12, **greedy))[0]
+    if first_of_b in alone.tokens:
+        pytest.skip("the end token chosen for this test also ends the other sequence")
+    both = generate(eng, [a, b], GenerationOptions(max_tokens=12, stop_tokens=(first_of_b,), **greedy))
+    assert both[1].tokens == [] and both[1].finish_reason == "stop"
+    assert both[0].tokens == alone.tokens and len(alone.tokens) == 12       # positions 60..71: into the second page
+    assert eng.cache.n_live == 0 and all(g.pool.n_free == g.pool.n_pages for g in eng.cache.groups)
+
+
 def test_generate_ends_a_sequence_when_the_cache_is_full(cpu_engine):
     eng = cpu_engine("A", max_tokens=64, max_slots=1)
     r = generate(eng, [[1] * 60], GenerationOptions(max_tokens=50, temperature=0.0, rep_penalty=1.0, loop_detection=False))[0]

@@ -16,6 +16,7 @@ from typing import Callable, Sequence
 
 import torch
 
+from ..cache.paged import CacheFull
 from ..sampling.sampler import Sampler, SamplingOptions, TokenFetch
 
 
@@ -121,7 +122,6 @@ def generate(engine, prompts: Sequence[Sequence[int]], options: GenerationOption
         raise ValueError("every prompt needs at least one token")
     if o.max_tokens < 1:
         return [GenerationResult([], "length") for _ in prompts]
-    stop = tuple(o.stop_tokens)
     sampler = Sampler(o.sampling(), engine.model.act, engine.device)
     results: list[GenerationResult | None] = [None] * len(prompts)
     max_pos = engine.cache.max_positions
@@ -151,7 +151,12 @@ def generate(engine, prompts: Sequence[Sequence[int]], options: GenerationOption
                 next_logits = None
                 if ahead:
                     feed = ids if len(ahead) == len(live) else ids[torch.tensor(ahead, dtype=torch.int64, device=ids.device)]
-                    next_logits = engine.step_from_device([slot_of[live[i]] for i in ahead], feed)
+                    try:
+                        next_logits = engine.step_from_device([slot_of[live[i]] for i in ahead], feed)
+                    except CacheFull:
+                        # no page to run ahead with: a sequence that ends on this token may give one back, so the
+                        # step waits for the tokens this once
+                        ahead = []
                 tokens = fetch.wait()
                 sampler.finish(tokens, states)
                 going = []
@@ -163,9 +168,12 @@ def generate(engine, prompts: Sequence[Sequence[int]], options: GenerationOption
                         results[r] = GenerationResult(tracks[r].out, tracks[r].finish_reason)
                 if not going:
                     break
-                rows = [ahead.index(i) for i in going]       # a sequence that goes on was run ahead
-                logits = next_logits if rows == list(range(len(ahead))) else \
-                    next_logits[torch.tensor(rows, dtype=torch.int64, device=next_logits.device)]
+                if not ahead:
+                    logits = engine.step([slot_of[live[i]] for i in going], [[tokens[i]] for i in going])
+                else:
+                    rows = [ahead.index(i) for i in going]       # a sequence that goes on was run ahead
+                    logits = next_logits if rows == list(range(len(ahead))) else \
+                        next_logits[torch.tensor(rows, dtype=torch.int64, device=next_logits.device)]
                 live = [live[i] for i in going]
         finally:
             engine.close(list(slot_of.values()))
