@@ -102,7 +102,8 @@ def test_gemm_dense(ops, act, M, N, K, mode):
 
 
 @pytest.mark.parametrize("act", ACTS)
-@pytest.mark.parametrize("M,N,K,bias", [(300, 200, 2200, True), (129, 130, 4104, False), (70, 64, 1000, False), (9, 40, 4096, True)])
+@pytest.mark.parametrize("M,N,K,bias", [(300, 200, 2200, True), (129, 130, 4104, False), (70, 64, 1000, False), (9, 40, 4096, True),
+                                        (40, 264, 8200, True), (64, 2048, 5632, False), (17, 72, 4096, False)])
 def test_gemm_partial_sums(ops, act, M, N, K, bias):
     """A product may come back as partial sums over runs of k ([S, M, N], the bias in the first); however many the
     kernel makes, their sum is the product."""
@@ -112,7 +113,15 @@ def test_gemm_partial_sums(ops, act, M, N, K, bias):
     y = ops.gemm(a.to(DEV), w.to(DEV), act, bias=None if b is None else b.to(DEV), partial_sums=True).cpu()
     assert y.dim() == 3 and tuple(y.shape[1:]) == (M, N)
     if act == "bfloat16":
-        assert y.shape[0] == (1 if M <= 64 or K < 2048 else (2 if K < 4096 else 4))
+        if M <= 16:
+            runs = 1
+        elif M <= 64:       # few rows of a narrow matrix: runs of at least 256 of k for each of 8 waves, up to 2048 waves
+            runs, waves = 1, -(-N // 32) * 8
+            while runs < 8 and waves * runs < 2048 and K // (16 * runs) >= 256:
+                runs *= 2
+        else:
+            runs = 1 if K < 2048 else (2 if K < 4096 else 4)
+        assert y.shape[0] == runs
     ref = ref_gemm(a, w, b, None)
     scale = ref.abs().max().item()
     err = (y.double().sum(0) - ref).abs().max().item()

@@ -239,12 +239,12 @@ __device__ __forceinline__ void stream_body(MfmaGemmArgs g, int tile_n, int tile
   }
 }
 
-// grid (ceil(N / (16 NTL)), row tiles of 16 * MT rows).  Two column tiles per wave need the registers of a
+// grid (ceil(N / (16 NTL)), row tiles of 16 * MT rows, runs of k).  Two column tiles per wave need the registers of a
 // workgroup of at most 8 waves.
 template <int MT, bool DUAL, bool OUT_ACT, int NTL>
 __global__ __launch_bounds__(NTL > 1 ? 512 : 1024) void gemm_stream_kernel(MfmaGemmArgs g) {
   extern __shared__ float red[];
-  stream_body<MT, DUAL, OUT_ACT, NTL>(g, blockIdx.x, blockIdx.y, 0, red);
+  stream_body<MT, DUAL, OUT_ACT, NTL>(g, blockIdx.x, blockIdx.y, blockIdx.z, red);
 }
 
 // Two products that do not depend on each other in one launch (decoding: the routed experts' product beside
@@ -472,12 +472,16 @@ static int split_k_waves(int N, int K, bool grouped) {
 
 // MT row tiles of 16; more than one (17 to 64 rows of one matrix) go with two column tiles per wave.
 template <int MT>
-static int launch_stream(const MfmaGemmArgs& g, bool dual, bool out_act, int row_tiles, hipStream_t st) {
+static int launch_stream(MfmaGemmArgs g, bool dual, bool out_act, int row_tiles, hipStream_t st, int splits = 1) {
   constexpr int NTL = MT > 1 ? 2 : 1;
-  int nw = split_k_waves((g.N + NTL - 1) / NTL, g.K, g.tile_group != nullptr);
+  if (splits > 1) {        // runs of k, each a multiple of 64 so that it starts at a whole line
+    g.k_per = ((g.K + 63) / 64 + splits - 1) / splits * 64;
+    if ((int64_t)(splits - 1) * g.k_per >= g.K) return TQ_ERR_BAD_ARG;
+  }
+  int nw = split_k_waves((g.N + NTL - 1) / NTL, splits > 1 ? g.k_per : g.K, g.tile_group != nullptr);
   const size_t per_wave = (size_t)NTL * MT * (dual ? 2 : 1) * 4 * 64 * sizeof(float);
   while (nw > 1 && (nw * per_wave > 64 * 1024 || (NTL > 1 && nw > 8))) nw /= 2;
-  const dim3 grid((g.N + 16 * NTL - 1) / (16 * NTL), row_tiles);
+  const dim3 grid((g.N + 16 * NTL - 1) / (16 * NTL), row_tiles, splits);
   const size_t shmem = nw > 1 ? nw * per_wave : 0;
   if (shmem > 64 * 1024) return TQ_ERR_UNSUPPORTED;
   if (dual && out_act)
@@ -514,11 +518,24 @@ static int launch_tile(const MfmaGemmArgs& g, bool dual, bool out_act, int split
   return 0;
 }
 
-// Into how many runs of k a plain product of M rows may be split when its partial sums are wanted apart: a
-// product of many rows whose tiles do not fill the chip twice, and that has k enough, goes faster in 2 to 4 runs,
-// each at least 1024 long.  1 for few rows, which take the streaming kernel.
+// Whether a product of 17 to 64 rows takes the tiled kernel: a matrix wide enough to give every compute unit two
+// tiles of 128 columns (a vocabulary).  The tiles read `a` through LDS once per 128 columns, the streaming kernel
+// once per 32 (measured at 151,936 x 2,048 and 64 rows: 159 us against 466 with 16 columns a wave).
+static bool wide_enough_for_tiles(int N) { return (N + TBN - 1) / TBN >= 512 && (N + TBN - 1) / TBN <= 65535; }
+
+// Into how many runs of k a plain product of M rows may be split when its partial sums are wanted apart.  Many
+// rows: a product whose tiles do not fill the chip twice, and that has k enough, goes faster in 2 to 4 runs, each
+// at least 1024 long.  17 to 64 rows of a narrow matrix with a long k (the streaming kernel with at most 8 waves
+// over k): as many runs as bring about 2048 waves, each wave keeping 256 of k.  1 for up to 16 rows.
 TQ_API int tq_gemm_mfma_splits(int M, int N, int K) {
-  if (M <= 64) return 1;
+  if (M <= 16) return 1;
+  if (M <= 64) {
+    if (wide_enough_for_tiles(N)) return 1;
+    const int64_t waves = (int64_t)((N + 31) / 32) * 8;
+    int s = 1;
+    while (s < 8 && waves * s < 2048 && K / (16 * s) >= 256) s *= 2;
+    return s;
+  }
   const int64_t tiles = (int64_t)((M + 127) / 128) * ((N + TBN - 1) / TBN);
   int s = 1;
   while (s < 4 && tiles * s < 512 && K / (s * 2) >= 1024) s *= 2;
@@ -555,15 +572,12 @@ TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gat
     }
   } else if (M <= 16) {
     rc = launch_stream<1>(g, dual, out_act, 1, st);
-  } else if (M <= 64 && (N + TBN - 1) / TBN >= 512 && (N + TBN - 1) / TBN <= 65535) {
-    // a matrix wide enough to give every compute unit two tiles of 128 columns (a vocabulary): the tiles read
-    // `a` through LDS once per 128 columns, the streaming kernel once per 16 (measured at 151,936 x 2,048 and 64
-    // rows: 159 us against 466)
+  } else if (M <= 64 && wide_enough_for_tiles(N)) {
     rc = launch_tile<64, 2, 4>(g, dual, out_act, splits, st);
   } else if (M <= 32) {
-    rc = launch_stream<2>(g, dual, out_act, 1, st);
+    rc = launch_stream<2>(g, dual, out_act, 1, st, splits);
   } else if (M <= 64) {
-    rc = launch_stream<4>(g, dual, out_act, 1, st);
+    rc = launch_stream<4>(g, dual, out_act, 1, st, splits);
   } else {
     if ((N + TBN - 1) / TBN > 65535) return TQ_ERR_UNSUPPORTED;
     rc = M <= 64 * 16 && !dual ? launch_tile<64, 2, 4>(g, dual, out_act, splits, st)
