@@ -213,9 +213,16 @@ def route(x32, router, shared_scale, top_k, renormalize, unit, act):
     return (ids, weights, gate) + tuple(moe_align(ids, router.shape[0], unit, act))
 
 
+def qkv_rope_write(a, qkv_weight, qkv_bias, positions, seq_of_token, block_table, inv_freq, pairing, rotary_dim, k_pages,
+                   v_pages, layer_offset, page_size, page_stride, num_heads, num_kv_heads, head_dim, act, runs=None):
+    qkv = gemm(a, qkv_weight, act, bias=qkv_bias)
+    return rope_kv_write(qkv, positions, seq_of_token, block_table, inv_freq, pairing, rotary_dim, k_pages, v_pages,
+                         layer_offset, page_size, page_stride, num_heads, num_kv_heads, head_dim, act, runs=runs)
+
+
 def install(monkeypatch):
     """Puts the stand-ins in place of the kernels for one test."""
     from turboquant_cpp_amd.csrc import ops
-    for name in ("embed", "add_rmsnorm", "rope_kv_write", "attention", "gemm", "router_topk", "moe_align", "route", "gemm_pair",
+    for name in ("embed", "add_rmsnorm", "rope_kv_write", "qkv_rope_write", "attention", "gemm", "router_topk", "moe_align", "route", "gemm_pair",
                  "moe_combine", "argmax", "rep_penalty", "sample_topp"):
         monkeypatch.setattr(ops, name, globals()[name])

@@ -432,6 +432,48 @@ def test_values_of_whole_runs_are_written_by_tiles(ops, act, nh, nkv, hd, page):
     assert int((pages[0][2] != 0).sum()) > T * nkv * hd // 2
 
 
+@pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("nh,nkv,hd,H,bias,write", [(3, 1, 64, 264, True, True), (16, 16, 128, 2048, True, True), (5, 5, 32, 72, False, True),
+                                                    (6, 2, 96, 136, True, False), (4, 2, 48, 136, True, True)])
+def test_queries_keys_values_in_one_launch(ops, act, nh, nkv, hd, H, bias, write):
+    """The product of q, k, v with rotation and cache write behind it, asked for as one operation: up to 16 tokens
+    in bfloat16 go out in one launch (head sizes that are multiples of 32), and queries and pages hold what the
+    product followed by the rotation kernel gives; other sizes are those two calls."""
+    from plain_qwen2moe import rope_frequencies
+    page, layers, layer = 64, 2, 1
+    starts, T_each = [3, 70, 0, 129], [1, 1, 1, 1]
+    lens = [a + b for a, b in zip(starts, T_each)]
+    table, slots, page_stride, kp, vp = paged_setup(lens, page, nkv, hd, layers, act, 170)
+    off = layer * nkv * page * hd
+    for T in (1, 4):
+        positions = torch.tensor(starts[:T], dtype=torch.int32)
+        slot_of = torch.tensor(slots[:T], dtype=torch.int32)
+        a = rnd((T, H), adt(act), 171)
+        w = rnd(((nh + 2 * nkv) * hd, H), adt(act), 172, 0.2)
+        b = rnd(((nh + 2 * nkv) * hd,), adt(act), 173) if bias else None
+        freqs = torch.from_numpy(rope_frequencies(hd, 1e6))
+        out = []
+        for fused in (True, False):
+            kd, vd = kp.to(DEV).clone(), vp.to(DEV).clone()
+            args = (positions.to(DEV), slot_of.to(DEV), table.to(DEV), freqs.to(DEV), 0, hd, kd if write else None,
+                    vd if write else None, off, page, page_stride, nh, nkv, hd, act)
+            if fused:
+                q = ops.qkv_rope_write(a.to(DEV), w.to(DEV), None if b is None else b.to(DEV), *args)
+            else:
+                q = ops.rope_kv_write(ops.gemm(a.to(DEV), w.to(DEV), act, bias=None if b is None else b.to(DEV)), *args)
+            out.append((q.cpu().float(), kd.cpu().float(), vd.cpu().float()))
+        scale = out[1][0].abs().max().item()
+        lim = 1e-5 * scale if act == "float32" else 1.6e-2 * scale        # two roundings to bfloat16 of sums in another order
+        for x, y in zip(*out):
+            assert (x - y).abs().max().item() <= lim
+        if write:
+            assert int((out[0][1] != 0).sum()) > T * nkv * hd // 2 and int((out[0][2] != 0).sum()) > T * nkv * hd // 2
+            assert torch.equal(out[0][1] != 0, out[1][1] != 0) or act == "bfloat16"      # the same rows and nothing else
+            assert int((out[0][1] != 0).sum()) <= T * nkv * hd and int((out[0][2] != 0).sum()) <= T * nkv * hd
+        else:
+            assert int((out[0][1] != 0).sum()) == 0 and int((out[0][2] != 0).sum()) == 0
+
+
 def test_rope_pairings_are_one_rotation(ops):
     """interleaved(P x) = P half(x) for the permutation P that interleaves the two halves."""
     from plain_qwen2moe import rope as plain_rope

@@ -82,44 +82,13 @@ __device__ __forceinline__ void store_out(const MfmaGemmArgs& g, int m, int n, f
 }
 
 // ------------------------------------------------------------------------------------------ few rows
-// A workgroup of 64 * (waves that split k) threads takes column tile `tile_n` (16 * NTL columns) of row tile
-// `tile_m` (16 * MT rows) over run `z` of k (k_per long; run 0 is all of k unless the product is split into
-// partial sums); red: LDS of [waves][NTL * MT * (DUAL ? 2 : 1)][4][64] floats.  What a wave reads of `a` serves
-// its NTL tiles of 16 columns: with many rows the way of `a` from L2 into the compute unit is what binds, and two
-// column tiles per wave halve it.
-template <int MT, bool DUAL, bool OUT_ACT, int NTL = 1>
-__device__ __forceinline__ void stream_body(MfmaGemmArgs g, int tile_n, int tile_m, int z, float* red) {
-  if (g.n_tiles && tile_m >= g.n_tiles[0]) return;
-  const int k_lo = z * g.k_per, k_hi = min(g.K, k_lo + g.k_per);
-  if (z) {
-    g.out = (float*)g.out + z * g.split_stride;
-    g.bias = nullptr;
-  }
-  const int group = g.tile_group ? g.tile_group[tile_m] : 0;
-  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, nw = blockDim.x / 64;
-  const int r = lane % 16, c = lane / 16;
-  const int n0 = tile_n * 16 * NTL, m0 = tile_m * 16 * MT;
-  // the rows of `a` that this lane fetches: r % 8 and 8 + r % 8 of each tile of 16 (as with w below)
-  const int q = c + 4 * (r / 8);            // and the chunk of 8 within each 64 of k
-  const bf16_t* ap[MT][2];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-    for (int hf = 0; hf < 2; ++hf) {
-      const int m = m0 + mt * 16 + 8 * hf + r % 8;
-      int src = -1;
-      if (m < g.M) {
-        src = g.a_rows ? g.a_rows[m] : m;
-        if (src >= 0 && !g.a_gather) src = m;
-      }
-      ap[mt][hf] = src >= 0 ? g.a + (size_t)src * g.lda + q * 8 : nullptr;
-    }
-  // this wave's share of k, in steps of 32; an even number of them, so that every pair of steps is a line of w
-  const int steps = (k_hi - k_lo + 31) / 32;
-  const int per = ((steps + nw - 1) / nw + 1) & ~1;
-  const int k_beg = k_lo + wave * per * 32, k_end = min(k_hi, k_lo + (wave + 1) * per * 32);
-
-  f32x4 acc[NTL][MT], acc2[DUAL ? NTL : 1][DUAL ? MT : 1];
+// The sums of one wave: its share k_beg .. k_end of k for NTL tiles of 16 columns (tile t starts at column col0[t])
+// and MT tiles of 16 rows (ap: the rows of `a` that this lane fetches, q: its chunk of 8 within each 64 of k).
+template <int MT, bool DUAL, int NTL>
+__device__ __forceinline__ void stream_accumulate(const MfmaGemmArgs& g, const int (&col0)[NTL], int group,
+                                                  const bf16_t* const (&ap)[MT][2], int q, int k_beg, int k_end,
+                                                  f32x4 (&acc)[NTL][MT], f32x4 (&acc2)[DUAL ? NTL : 1][DUAL ? MT : 1]) {
+  const int r = (threadIdx.x % 64) % 16;
 #pragma unroll
   for (int t = 0; t < NTL; ++t)
 #pragma unroll
@@ -139,7 +108,7 @@ __device__ __forceinline__ void stream_body(MfmaGemmArgs g, int tile_n, int tile
     size_t row_a[NTL], row_b[NTL];
 #pragma unroll
     for (int t = 0; t < NTL; ++t) {
-      const int n_a = n0 + 16 * t + r % 8, n_b = n_a + 8;
+      const int n_a = col0[t] + r % 8, n_b = n_a + 8;
       row_a[t] = (size_t)group * g.group_stride + (size_t)(n_a < g.N ? n_a : 0) * g.K + q * 8;
       row_b[t] = (size_t)group * g.group_stride + (size_t)(n_b < g.N ? n_b : 0) * g.K + q * 8;
     }
@@ -190,6 +159,50 @@ __device__ __forceinline__ void stream_body(MfmaGemmArgs g, int tile_n, int tile
         }
     }
   }
+}
+
+// A workgroup of 64 * (waves that split k) threads takes column tile `tile_n` (16 * NTL columns) of row tile
+// `tile_m` (16 * MT rows) over run `z` of k (k_per long; run 0 is all of k unless the product is split into
+// partial sums); red: LDS of [waves][NTL * MT * (DUAL ? 2 : 1)][4][64] floats.  What a wave reads of `a` serves
+// its NTL tiles of 16 columns: with many rows the way of `a` from L2 into the compute unit is what binds, and two
+// column tiles per wave halve it.
+template <int MT, bool DUAL, bool OUT_ACT, int NTL = 1>
+__device__ __forceinline__ void stream_body(MfmaGemmArgs g, int tile_n, int tile_m, int z, float* red) {
+  if (g.n_tiles && tile_m >= g.n_tiles[0]) return;
+  const int k_lo = z * g.k_per, k_hi = min(g.K, k_lo + g.k_per);
+  if (z) {
+    g.out = (float*)g.out + z * g.split_stride;
+    g.bias = nullptr;
+  }
+  const int group = g.tile_group ? g.tile_group[tile_m] : 0;
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, nw = blockDim.x / 64;
+  const int r = lane % 16, c = lane / 16;
+  const int n0 = tile_n * 16 * NTL, m0 = tile_m * 16 * MT;
+  // the rows of `a` that this lane fetches: r % 8 and 8 + r % 8 of each tile of 16 (as with w below)
+  const int q = c + 4 * (r / 8);            // and the chunk of 8 within each 64 of k
+  const bf16_t* ap[MT][2];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      const int m = m0 + mt * 16 + 8 * hf + r % 8;
+      int src = -1;
+      if (m < g.M) {
+        src = g.a_rows ? g.a_rows[m] : m;
+        if (src >= 0 && !g.a_gather) src = m;
+      }
+      ap[mt][hf] = src >= 0 ? g.a + (size_t)src * g.lda + q * 8 : nullptr;
+    }
+  // this wave's share of k, in steps of 32; an even number of them, so that every pair of steps is a line of w
+  const int steps = (k_hi - k_lo + 31) / 32;
+  const int per = ((steps + nw - 1) / nw + 1) & ~1;
+  const int k_beg = k_lo + wave * per * 32, k_end = min(k_hi, k_lo + (wave + 1) * per * 32);
+
+  f32x4 acc[NTL][MT], acc2[DUAL ? NTL : 1][DUAL ? MT : 1];
+  int col0[NTL];
+#pragma unroll
+  for (int t = 0; t < NTL; ++t) col0[t] = n0 + 16 * t;
+  stream_accumulate<MT, DUAL, NTL>(g, col0, group, ap, q, k_beg, k_end, acc, acc2);
   // The waves' partial sums are added in wave order, every thread of the workgroup taking some of the outputs.
   constexpr int PAIRS = NTL * MT;               // (column tile, row tile) pairs: set t * MT + mt, the gate's partner PAIRS on
   constexpr int SETS = PAIRS * (DUAL ? 2 : 1);
@@ -261,6 +274,93 @@ __global__ __launch_bounds__(1024) void gemm_stream_pair_kernel(MfmaGemmArgs g1,
     stream_body<1, DUAL, OUT_ACT>(g2, id % nx2, id / nx2 % rows2, id / nx2 / rows2, red);
   else
     stream_body<1, DUAL, OUT_ACT>(g1, (id - n2) % nx1, (id - n2) / nx1, 0, red);
+}
+
+// ------------------------------------------------------------------------------------------ q, k, v of a few tokens
+// The product that makes queries, keys and values of up to 16 tokens, with what follows it in the same launch:
+// bias, rotation of queries and keys (pairs (d, d + hd / 2), the whole head rotated), queries out in bfloat16,
+// keys and values into their cache pages (as rope_kv_write_kernel of elementwise.hip does it from the float
+// product; same formulas, same float arithmetic).  A workgroup takes the two tiles of 16 columns that hold the
+// partners of 16 pairs of one head: columns head * hd + 16 j .. and the same + hd / 2; grid (heads * hd / 32), the
+// waves split k.
+struct RopeWriteArgs {
+  const int* positions;        // [T]
+  const int* seq_of_token;     // [T]
+  const int* block_table;
+  int bt_stride;
+  const float* inv_freq;       // [hd / 2]
+  bf16_t* q_out;               // [T][nh * hd]
+  bf16_t* k_pool;              // the layer's offset already added; null: keys and values are not written
+  bf16_t* v_pool;
+  int page_size;
+  int64_t page_stride;
+  int nh, nkv, hd;
+};
+
+__global__ __launch_bounds__(512) void qkv_rope_write_kernel(MfmaGemmArgs g, RopeWriteArgs p) {
+  extern __shared__ float red[];       // [waves][2][4][64]
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, nw = blockDim.x / 64;
+  const int r = lane % 16, c = lane / 16;
+  const int per_head = p.hd / 32;
+  const int head = blockIdx.x / per_head, j = blockIdx.x % per_head;
+  const int col0[2] = {head * p.hd + 16 * j, head * p.hd + p.hd / 2 + 16 * j};
+  const int q = c + 4 * (r / 8);
+  const bf16_t* ap[1][2];
+#pragma unroll
+  for (int hf = 0; hf < 2; ++hf) {
+    const int m = 8 * hf + r % 8;
+    ap[0][hf] = m < g.M ? g.a + (size_t)m * g.lda + q * 8 : nullptr;
+  }
+  const int steps = (g.K + 31) / 32;
+  const int per = ((steps + nw - 1) / nw + 1) & ~1;
+  const int k_beg = wave * per * 32, k_end = min(g.K, (wave + 1) * per * 32);
+  f32x4 acc[2][1], acc2[1][1];
+  stream_accumulate<1, false, 2>(g, col0, 0, ap, q, k_beg, k_end, acc, acc2);
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) red[((wave * 2 + t) * 4 + v) * 64 + lane] = acc[t][0][v];
+  __syncthreads();
+  for (int i = threadIdx.x; i < 256; i += blockDim.x) {
+    const int ol = i % 64, v = i / 64;
+    const int m = 4 * (ol / 16) + v, d = 16 * j + ol % 16;      // token and dimension (of the pair's first half)
+    if (m >= g.M) continue;
+    float a = 0.f, b = 0.f;
+    for (int w = 0; w < nw; ++w) {      // in wave order, as the product alone adds them
+      a += red[((w * 2 + 0) * 4 + v) * 64 + ol];
+      b += red[((w * 2 + 1) * 4 + v) * 64 + ol];
+    }
+    a += bias_at(g, col0[0] + ol % 16);
+    b += bias_at(g, col0[1] + ol % 16);
+    const int pos = p.positions[m];
+    if (head < p.nh + p.nkv) {
+      const float theta = (float)pos * p.inv_freq[d];
+      float sn, cs;
+      sincosf(theta, &sn, &cs);
+      const float ra = a * cs - b * sn, rb = a * sn + b * cs;
+      a = ra;
+      b = rb;
+    }
+    if (head < p.nh) {
+      bf16_t* dst = p.q_out + ((size_t)m * p.nh + head) * p.hd;
+      dst[d] = f32_to_bf16(a);
+      dst[d + p.hd / 2] = f32_to_bf16(b);
+      continue;
+    }
+    if (!p.k_pool) continue;
+    const int page = p.block_table[(size_t)p.seq_of_token[m] * p.bt_stride + pos / p.page_size];
+    const int row = pos % p.page_size;
+    const size_t kv_head_stride = (size_t)p.page_size * p.hd;
+    if (head < p.nh + p.nkv) {         // keys lie [row][hd]
+      bf16_t* dst = p.k_pool + (size_t)page * p.page_stride + (size_t)(head - p.nh) * kv_head_stride + (size_t)row * p.hd;
+      dst[d] = f32_to_bf16(a);
+      dst[d + p.hd / 2] = f32_to_bf16(b);
+    } else {                           // values lie transposed, [hd][row]
+      bf16_t* dst = p.v_pool + (size_t)page * p.page_stride + (size_t)(head - p.nh - p.nkv) * kv_head_stride + row;
+      dst[(size_t)d * p.page_size] = f32_to_bf16(a);
+      dst[(size_t)(d + p.hd / 2) * p.page_size] = f32_to_bf16(b);
+    }
+  }
 }
 
 // ------------------------------------------------------------------------------------------ many rows
@@ -652,6 +752,32 @@ TQ_API int tq_gemm_mfma_pair(const int64_t* d1, const int64_t* d2, int splits2, 
   else if (out_act[0]) TQ_PAIR(false, true);
   else TQ_PAIR(false, false);
 #undef TQ_PAIR
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// Queries, keys and values of T <= 16 tokens in one launch: a [T][K] bfloat16 (row stride lda) times w [(nh + 2 nkv)
+// hd][K] plus bias, queries and keys rotated by positions[t] * inv_freq[d] on the pairs (d, d + hd / 2), queries to
+// q_out [T][nh hd], keys and values into the pages (k_pool / v_pool with the layer's offset added; null: only the
+// queries are made).  hd must be a multiple of 32 and the rotation span the whole head.
+TQ_API int tq_qkv_rope_write(const void* a, int64_t lda, const void* w, const void* bias, int bias_type, int T, int K,
+                             const int* positions, const int* seq_of_token, const int* block_table, int bt_stride,
+                             const float* inv_freq, void* q_out, void* k_pool, void* v_pool, int page_size,
+                             int64_t page_stride, int nh, int nkv, int hd, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (T > 16 || hd % 32 != 0 || hd <= 0 || nh <= 0 || nkv <= 0) return TQ_ERR_UNSUPPORTED;
+  if (K <= 0 || K % 8 != 0 || lda % 8 != 0 || ((uintptr_t)a | (uintptr_t)w) % 16 != 0) return TQ_ERR_BAD_ARG;
+  if ((k_pool == nullptr) != (v_pool == nullptr) || page_size <= 0) return TQ_ERR_BAD_ARG;
+  const int heads = k_pool ? nh + 2 * nkv : nh;
+  const int N = (nh + 2 * nkv) * hd;
+  MfmaGemmArgs g{(const bf16_t*)a, lda, nullptr, 1, (const bf16_t*)w, nullptr, 0, nullptr, nullptr, bias, bias_type,
+                 nullptr, 0, T, N, K, K, 0};
+  RopeWriteArgs p{positions, seq_of_token, block_table, bt_stride, inv_freq, (bf16_t*)q_out, (bf16_t*)k_pool,
+                  (bf16_t*)v_pool, page_size, page_stride, nh, nkv, hd};
+  int nw = split_k_waves(heads * hd / 2, K, false);
+  if (nw > 8) nw = 8;
+  const size_t shmem = (size_t)nw * 2 * 4 * 64 * sizeof(float);
+  hipLaunchKernelGGL(qkv_rope_write_kernel, dim3(heads * (hd / 32)), dim3(64 * nw), shmem, st, g, p);
   TQ_LAUNCH_CHECK();
   return 0;
 }

@@ -54,6 +54,8 @@ _OPTIONAL = {
     "tq_gemm_mfma_splits": [_c_int, _c_int, _c_int],
     "tq_gemm_mfma_pair_splits": [_c_int, _c_int, _c_int, _c_int, _c_int, _c_int],
     "tq_gemm_mfma_pair": [_c_ptr, _c_ptr, _c_int, _c_ptr],
+    "tq_qkv_rope_write": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr,
+                          _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_ptr],
     "tq_attention_decode_scratch": [_c_int, _c_int, _c_int, _c_int],
     "tq_attention_mfma": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int,
                           _c_int, _c_int, _c_int, _c_f32, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
@@ -249,6 +251,51 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torc
                                           block_table.shape[1], _ptr(inv_freq), pairing, rotary_dim, _ptr(q), kp, vp,
                                           page_size, page_stride, T, num_heads, num_kv_heads, head_dim, int(write),
                                           _ptr(cu), _ptr(slots), _ptr(start), B, max_new, _stream()))
+    return q
+
+
+def qkv_rope_write(a: torch.Tensor, qkv_weight: torch.Tensor, qkv_bias: torch.Tensor | None, positions: torch.Tensor,
+                   seq_of_token: torch.Tensor, block_table: torch.Tensor, inv_freq: torch.Tensor, pairing: int,
+                   rotary_dim: int, k_pages: torch.Tensor | None, v_pages: torch.Tensor | None, layer_offset: int,
+                   page_size: int, page_stride: int, num_heads: int, num_kv_heads: int, head_dim: int, act,
+                   runs: dict | None = None) -> torch.Tensor:
+    """``gemm(a, qkv_weight, bias=qkv_bias)`` followed by ``rope_kv_write``: the queries [T, nh*hd], keys and
+    values in their pages.  Up to 16 tokens in bfloat16, with heads rotated whole in "half" pairing, take one
+    launch (the product's workgroups rotate and store what they have summed); anything else is the two calls."""
+    k = "qkv_rope_write"
+    lib = library(act)
+    T, K = a.shape
+    fused = (hasattr(lib, "tq_qkv_rope_write") and T <= 16 and pairing == 0 and rotary_dim == head_dim
+             and head_dim % 32 == 0 and _use_mfma(act, a, qkv_weight, K)
+             and (qkv_bias is None or qkv_bias.dtype in _WTYPE))
+    if not fused:
+        qkv = gemm(a, qkv_weight, act, bias=qkv_bias)
+        return rope_kv_write(qkv, positions, seq_of_token, block_table, inv_freq, pairing, rotary_dim, k_pages, v_pages,
+                             layer_offset, page_size, page_stride, num_heads, num_kv_heads, head_dim, act, runs=runs)
+    adt = ACT_DTYPES[dtype_name(act)]
+    width = (num_heads + 2 * num_kv_heads) * head_dim
+    _check(a, k, "a", adt)
+    _need(a.stride(1) == 1, k, "a must have unit stride along its rows")
+    _check(qkv_weight, k, "qkv_weight", torch.bfloat16, (width, K))
+    if qkv_bias is not None:
+        _check(qkv_bias, k, "qkv_bias", tuple(_WTYPE), (width,))
+    _check(positions, k, "positions", torch.int32, (T,))
+    _check(seq_of_token, k, "seq_of_token", torch.int32, (T,))
+    _check(block_table, k, "block_table", torch.int32)
+    _need(block_table.dim() == 2, k, "block_table must be [B, pages]")
+    _check(inv_freq, k, "inv_freq", torch.float32, (head_dim // 2,))
+    q = torch.empty((T, num_heads * head_dim), dtype=adt, device=a.device)
+    kp = vp = None
+    if k_pages is not None:
+        _check(k_pages, k, "k_pages", adt)
+        _check(v_pages, k, "v_pages", adt)
+        _need(layer_offset + num_kv_heads * page_size * head_dim <= page_stride, k, "layer does not fit in a page")
+        esz = k_pages.element_size()
+        kp, vp = k_pages.data_ptr() + layer_offset * esz, v_pages.data_ptr() + layer_offset * esz
+    _run(k, lib.tq_qkv_rope_write(_ptr(a), a.stride(0), _ptr(qkv_weight), _ptr(qkv_bias),
+                                  _WTYPE[qkv_bias.dtype] if qkv_bias is not None else 0, T, K, _ptr(positions),
+                                  _ptr(seq_of_token), _ptr(block_table), block_table.shape[1], _ptr(inv_freq), _ptr(q),
+                                  kp, vp, page_size, page_stride, num_heads, num_kv_heads, head_dim, _stream()))
     return q
 
 

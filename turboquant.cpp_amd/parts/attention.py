@@ -64,12 +64,11 @@ class GroupedQueryAttention(Part):
 
     def forward(self, normed, ctx, entry):
         b, kv = ctx.batch, ctx.kv(entry)
-        qkv = ops.gemm(normed, self.qkv_weight, ctx.act, bias=self.qkv_bias)
-        q = ops.rope_kv_write(qkv, b.positions, b.slot_of_token, kv.table, self.position.table(ctx.device),
-                              self.position.pairing_code, self.position.rotary_dim,
-                              kv.k_pages if kv.owns else None, kv.v_pages if kv.owns else None,
-                              kv.layer_offset, kv.page_size, kv.page_stride,
-                              self.num_heads, self.num_kv_heads, self.head_dim, ctx.act, runs=b.runs())
+        q = ops.qkv_rope_write(normed, self.qkv_weight, self.qkv_bias, b.positions, b.slot_of_token, kv.table,
+                               self.position.table(ctx.device), self.position.pairing_code, self.position.rotary_dim,
+                               kv.k_pages if kv.owns else None, kv.v_pages if kv.owns else None,
+                               kv.layer_offset, kv.page_size, kv.page_stride,
+                               self.num_heads, self.num_kv_heads, self.head_dim, ctx.act, runs=b.runs())
         o = ops.attention(q, kv.k_pages, kv.v_pages, kv.layer_offset, b.positions, b.slot_of_token, kv.table,
                           kv.page_size, kv.page_stride, self.num_heads, self.num_kv_heads, self.head_dim,
                           self.window, self.scale, ctx.act, runs=b.runs())
