@@ -290,6 +290,10 @@ __device__ __forceinline__ void align_pairs(const int* ids, int n_pairs, int E, 
   const int per = ((n_pairs + AW - 1) / AW + TQ_WAVE - 1) / TQ_WAVE * TQ_WAVE;   // pairs per wave, whole batches
   const int seg_beg = wave * per, seg_end = min(n_pairs, seg_beg + per);
   int* mine = cnt + wave * E;
+  // with at most 64 pairs per wave a thread meets its pair again in the last loop (i == threadIdx.x both times):
+  // expert and rank stay in its registers and need not go through memory
+  const bool one_batch = per == TQ_WAVE;
+  int my_e = -1, my_rank = 0;
   for (int b = seg_beg; b < seg_end; b += TQ_WAVE) {
     const int i = b + lane;
     const bool valid = i < seg_end;
@@ -306,7 +310,12 @@ __device__ __forceinline__ void align_pairs(const int* ids, int n_pairs, int E, 
     __builtin_amdgcn_wave_barrier();       // every lane has read its count before the expert's first lane adds to it
     if (valid && lower == 0) mine[e] = base + __popcll(same);
     __builtin_amdgcn_wave_barrier();
-    if (valid) pair_slot[i] = rank;      // rank within (wave, expert) for now
+    if (one_batch) {
+      my_e = e;
+      my_rank = rank;
+    } else if (valid) {
+      pair_slot[i] = rank;      // rank within (wave, expert) for now
+    }
   }
   __syncthreads();
   // counts become each wave's first row within its expert; starts[e] first holds the expert's padded size
@@ -341,6 +350,15 @@ __device__ __forceinline__ void align_pairs(const int* ids, int n_pairs, int E, 
     if (lane == TQ_WAVE - 1) n_tiles[0] = incl / unit;
   }
   __syncthreads();
+  if (one_batch) {
+    if (my_e >= 0) {
+      const int i = threadIdx.x;
+      const int r = starts[my_e] + cnt[wave * E + my_e] + my_rank;
+      pair_slot[i] = r;
+      sorted_token[r] = i / topk;
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) {
     const int e = ids[i], w = i / per;
     const int r = starts[e] + cnt[w * E + e] + pair_slot[i];
