@@ -393,8 +393,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g)
   // has its own L2: so the tiles are numbered such that one die gets a contiguous run of them.  One matrix: a
   // run goes through bands of 8 row tiles, down a band's column of row tiles first, so that workgroups that run
   // at the same time on a die share their tiles of `a` and of `w` in that die's L2.  A matrix per expert: a run
-  // goes row tile by row tile through all columns, so that an expert's matrix is read by one die (by two where
-  // a run ends), and only the row tiles in use are dealt.
+  // goes expert by expert, so that an expert's matrix is read by one die (by two where a run ends), and within an
+  // expert column by column with the expert's row tiles side by side (measured against row tile by row tile: 6 to
+  // 12 % faster, the more the more row tiles an expert has); only the row tiles in use are dealt.
   int tile_m, tile_n;
   {
     const int gx = g.tile_group && g.n_tiles ? min(g.n_tiles[0], (int)gridDim.x) : (int)gridDim.x;
@@ -404,8 +405,15 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g)
     if (id / 8 >= q + (die < rem ? 1 : 0)) return;
     const int logical = die * q + min(die, rem) + id / 8;
     if (g.tile_group) {
-      tile_m = logical / gy;
-      tile_n = logical % gy;
+      // the expert whose row tiles [lo, hi) hold row tile logical / gy; within it column by column, the expert's
+      // row tiles of a column one after the other, so that they read that column's rows of w at the same time
+      const int t = logical / gy, e = g.tile_group[t];
+      int lo = t, hi = t + 1;
+      while (lo > 0 && g.tile_group[lo - 1] == e) --lo;
+      while (hi < gx && g.tile_group[hi] == e) ++hi;
+      const int local = logical - lo * gy, n_e = hi - lo;
+      tile_n = local / n_e;
+      tile_m = lo + local % n_e;
     } else {
       const int band = logical / (8 * gy), in_band = logical % (8 * gy);
       const int bh = min(8, gx - band * 8);
