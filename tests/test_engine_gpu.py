@@ -188,6 +188,44 @@ def test_first_tokens_and_long_decoding(name, act, engines):
         check_logits(lg, ref[:n], margins[:n], act, f"{name} {act} first {n} tokens")
 
 
+def test_the_layer_sizes_of_a_real_checkpoint(tmp_path):
+    """Two layers with the sizes of Qwen1.5-MoE-A2.7B (width 2,048, 16 heads of 128, 60 experts of 1,408, top 4, a
+    shared expert of 5,632; a small vocabulary) with random weights, against the plain implementation: three
+    prompts of unequal length in one step (one long enough for the tiled products), then steps of one token.
+    The tiny configurations of the other tests never reach the kernel variants of these sizes (rows of whole cache
+    lines, waves that split k, two products in one launch, head size 128, the product that rotates and stores)."""
+    from turboquant_cpp_amd.engine.model import load_model, write_random_model_dir
+    from turboquant_cpp_amd.engine.step import Engine
+    cfg = {"architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe", "vocab_size": 8000, "hidden_size": 2048,
+           "num_hidden_layers": 2, "num_attention_heads": 16, "num_key_value_heads": 16, "intermediate_size": 5632,
+           "moe_intermediate_size": 1408, "shared_expert_intermediate_size": 5632, "num_experts": 60,
+           "num_experts_per_tok": 4, "norm_topk_prob": False, "decoder_sparse_step": 1, "mlp_only_layers": [],
+           "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "use_sliding_window": False, "sliding_window": 32768,
+           "max_window_layers": 2, "max_position_embeddings": 4096, "tie_word_embeddings": False, "torch_dtype": "float32"}
+    g = torch.Generator().manual_seed(41)
+    n_fed = 4
+    seqs = [torch.randint(0, 8000, (n + n_fed,), generator=g).tolist() for n in (200, 70, 9)]
+    for act in ACTS:
+        d = write_random_model_dir(str(tmp_path / f"a27b_two_layers_{act}"), cfg, 3, 0.02, 0.02, act)
+        plain = PlainQwen2Moe(d)
+        refs = [plain_rows(plain, s) for s in seqs]
+        del plain
+        eng = Engine(load_model(d, act=act, device=DEV), max_tokens=64 * 8)
+        slots = eng.open(3)
+        prompts = [s[:-n_fed] for s in seqs]
+        first = eng.step(slots, prompts, [list(range(len(p))) for p in prompts]).cpu()
+        fed = [eng.step(slots, [[s[len(s) - n_fed + t]] for s in seqs]).cpu() for t in range(n_fed)]
+        eng.close(slots)
+        del eng
+        torch.cuda.empty_cache()
+        off = 0
+        for i, (s, (ref, margins)) in enumerate(zip(seqs, refs)):
+            n = len(s) - n_fed
+            got = torch.cat([first[off:off + n]] + [f[i:i + 1] for f in fed])
+            off += n
+            check_logits(got, ref, margins, act, f"real layer sizes, {act}, sequence of {len(s)}")
+
+
 @pytest.mark.parametrize("act", ACTS)
 def test_a_step_fed_from_the_device_is_the_step_fed_from_the_host(act, sharp_dirs):
     """Decode steps whose tokens come from a tensor on the device (eager, captured, replayed) give the bits of the
