@@ -13,6 +13,7 @@ them, and the rest must be close: nine in ten within 2 %, all within 10 % of the
 import json
 import math
 import os
+import shutil
 import subprocess
 import sys
 
@@ -218,6 +219,7 @@ def test_the_layer_sizes_of_a_real_checkpoint(tmp_path):
         eng.close(slots)
         del eng
         torch.cuda.empty_cache()
+        shutil.rmtree(d)              # gigabytes of weights: not kept for the next test session to find
         off = 0
         for i, (s, (ref, margins)) in enumerate(zip(seqs, refs)):
             n = len(s) - n_fed
