@@ -26,7 +26,11 @@ A27B = {
     "use_sliding_window": False, "sliding_window": 32768, "max_window_layers": 24, "max_position_embeddings": 8192,
     "tie_word_embeddings": False, "torch_dtype": "bfloat16",
 }
-FULL_LAYERS = 24
+# the other Qwen2-MoE checkpoint's sizes, about 115 GB of bfloat16 weights (`--sizes a14b`)
+A14B = dict(A27B, hidden_size=3584, num_hidden_layers=28, num_attention_heads=28, num_key_value_heads=4,
+            intermediate_size=18944, moe_intermediate_size=2560, shared_expert_intermediate_size=20480, num_experts=64,
+            num_experts_per_tok=8, sliding_window=131072, max_window_layers=28, max_position_embeddings=32768)
+SIZES = {"a27b": (A27B, "Qwen1.5-MoE-A2.7B"), "a14b": (A14B, "Qwen2-57B-A14B")}
 PEAK_HBM_GBS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 PREFILL_TOKENS = 2048
@@ -69,7 +73,8 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--layers", type=int, default=FULL_LAYERS)
+    ap.add_argument("--sizes", default="a27b", choices=sorted(SIZES), help="whose layer sizes (default: the headline model's)")
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (default: all)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=8192)
     ap.add_argument("--points-context", type=int, default=2048)
@@ -87,7 +92,9 @@ def main() -> int:
     from turboquant_cpp_amd.engine.step import Engine
     from turboquant_cpp_amd.sampling.sampler import TokenFetch
 
-    cfg = dict(A27B)
+    cfg, model_name = dict(SIZES[args.sizes][0]), SIZES[args.sizes][1]
+    full_layers = cfg["num_hidden_layers"]
+    args.layers = full_layers if args.layers is None else args.layers
     cfg["num_hidden_layers"] = args.layers
     cfg["max_window_layers"] = args.layers
     cfg["max_position_embeddings"] = max(args.context, args.points_context, PREFILL_TOKENS)
@@ -191,12 +198,12 @@ def main() -> int:
             s, _, _ = run_decode(b, args.points_context, 32, 4)
             points[f"decode_b{b}"] = round(b / s, 1)
     out = {
-        "metric": f"decode tok/s at batch {args.batch}, context {args.context} (Qwen1.5-MoE-A2.7B layer sizes, random weights)",
+        "metric": f"decode tok/s at batch {args.batch}, context {args.context} ({model_name} layer sizes, random weights)",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": short, "data": "synthetic",
         "config": {
-            "model": "Qwen1.5-MoE-A2.7B sizes", "layers": args.layers, "layers_of_full_model": FULL_LAYERS,
+            "model": f"{model_name} sizes", "layers": args.layers, "layers_of_full_model": full_layers,
             "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
             "head_dim": cfg["hidden_size"] // cfg["num_attention_heads"], "vocab": V, "experts": cfg["num_experts"],
             "top_k": cfg["num_experts_per_tok"], "expert_inner": cfg["moe_intermediate_size"],
