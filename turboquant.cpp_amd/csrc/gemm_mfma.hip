@@ -364,8 +364,8 @@ __global__ __launch_bounds__(512) void qkv_rope_write_kernel(MfmaGemmArgs g, Rop
 }
 
 // ------------------------------------------------------------------------------------------ many rows
-// grid (row tiles of BM, ceil(N / 128)); block of 8 waves laid WM x WN over the tile: BM = 128 as 4 x 2 (a wave
-// owns 32 x 64 outputs), BM = 64 as 2 x 4 (32 x 32).  Eight waves of small tiles beat four of large ones here:
+// grid (row tiles of BM, ceil(N / BN)); block of 8 waves laid WM x WN over the tile of BM x BN outputs (BN = 128
+// unless said): BM = 128 as 4 x 2 (a wave owns 32 x 64 outputs, or 32 x 96 with BN = 192), BM = 64 as 2 x 4 (32 x 32).  Eight waves of small tiles beat four of large ones here:
 // the step is bound by the way through LDS, and twice the waves hide twice the latency.
 #define TBN 128
 #define TBK 64
@@ -375,20 +375,20 @@ __global__ __launch_bounds__(512) void qkv_rope_write_kernel(MfmaGemmArgs g, Rop
 // 128 bytes per clock; XOR with bits 0..2 at 107, no swizzle at 31.
 __device__ __forceinline__ int swz(int row, int chunk) { return row * TBK + ((chunk ^ ((row >> 1) & 7)) << 3); }
 
-template <int BM, int WM, int WN, bool DUAL, bool OUT_ACT>
+template <int BM, int WM, int WN, bool DUAL, bool OUT_ACT, int BN = TBN>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g) {
   constexpr int NT = 64 * WM * WN;
   constexpr int MI = BM / WM / 32;               // 32-high row tiles per wave
-  constexpr int NI = TBN / WN / 32;              // 32-wide column tiles per wave
+  constexpr int NI = BN / WN / 32;              // 32-wide column tiles per wave
   constexpr int A_CH = BM * 8 / NT;              // 16-byte chunks of the a tile per thread
-  constexpr int W_CH = TBN * 8 / NT;
-  static_assert(MI >= 1 && NI >= 1 && A_CH >= 1 && W_CH >= 1 && BM * 8 % NT == 0 && TBN * 8 % NT == 0, "tile layout");
+  constexpr int W_CH = BN * 8 / NT;
+  static_assert(MI >= 1 && NI >= 1 && A_CH >= 1 && W_CH >= 1 && BM * 8 % NT == 0 && BN * 8 % NT == 0, "tile layout");
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   // two buffers, each a tile of `a`, one of `w` and (gated pair) one of `w2`
-  constexpr int BUF = (BM + TBN * (DUAL ? 2 : 1)) * TBK;
+  constexpr int BUF = (BM + BN * (DUAL ? 2 : 1)) * TBK;
   bf16_t* As = (bf16_t*)smem;
   bf16_t* Ws = As + BM * TBK;
-  bf16_t* Vs = Ws + TBN * TBK;
+  bf16_t* Vs = Ws + BN * TBK;
   // Which tile this workgroup takes.  Workgroups are dealt to the chip's 8 dies in turn (id % 8), and each die
   // has its own L2: so the tiles are numbered such that one die gets a contiguous run of them.  One matrix: a
   // run goes through bands of 8 row tiles, down a band's column of row tiles first, so that workgroups that run
@@ -424,7 +424,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g)
   const int group = g.tile_group ? g.tile_group[tile_m] : 0;
   const bf16_t* w = g.w + (size_t)group * g.group_stride;
   const bf16_t* w2 = DUAL ? g.w2 + (size_t)group * g.group_stride : nullptr;
-  const int m0 = tile_m * BM, n0 = tile_n * TBN;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int wm = wave / WN, wn = wave % WN;
   // this workgroup's run of k: k_lo .. k_lo + Kl (all of k unless the product is split), and where its sums go
@@ -603,16 +603,17 @@ static int launch_stream(MfmaGemmArgs g, bool dual, bool out_act, int row_tiles,
   return 0;
 }
 
-template <int BM, int WM, int WN>
+template <int BM, int WM, int WN, int BN = TBN>
 static int launch_tile(const MfmaGemmArgs& g, bool dual, bool out_act, int splits, hipStream_t st) {
-  const dim3 grid((g.M + BM - 1) / BM, (g.N + TBN - 1) / TBN, splits);
-  const size_t shmem = (size_t)2 * (BM + TBN * (dual ? 2 : 1)) * TBK * sizeof(bf16_t);
+  const dim3 grid((g.M + BM - 1) / BM, (g.N + BN - 1) / BN, splits);
+  const size_t shmem = (size_t)2 * (BM + BN * (dual ? 2 : 1)) * TBK * sizeof(bf16_t);
 #define TQ_TILE(D, O)                                                                                  \
   do {                                                                                                 \
     if (shmem > 48 * 1024)                                                                             \
-      hipFuncSetAttribute((const void*)gemm_tile_kernel<BM, WM, WN, D, O>,                             \
+      hipFuncSetAttribute((const void*)gemm_tile_kernel<BM, WM, WN, D, O, BN>,                         \
                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);                     \
-    hipLaunchKernelGGL((gemm_tile_kernel<BM, WM, WN, D, O>), grid, dim3(64 * WM * WN), shmem, st, g);  \
+    hipLaunchKernelGGL((gemm_tile_kernel<BM, WM, WN, D, O, BN>), grid, dim3(64 * WM * WN), shmem, st,  \
+                       g);                                                                             \
   } while (0)
   if (dual && out_act)
     TQ_TILE(true, true);
@@ -630,6 +631,16 @@ static int launch_tile(const MfmaGemmArgs& g, bool dual, bool out_act, int split
 // tiles of 128 columns (a vocabulary).  The tiles read `a` through LDS once per 128 columns, the streaming kernel
 // once per 32 (measured at 151,936 x 2,048 and 64 rows: 159 us against 466 with 16 columns a wave).
 static bool wide_enough_for_tiles(int N) { return (N + TBN - 1) / TBN >= 512 && (N + TBN - 1) / TBN <= 65535; }
+
+// Tiles of 128 x 192 instead of 128 x 128 for a plain product: the chip holds 512 workgroups of either at a time
+// (256 compute units, two to each), a tile of 192 columns takes one and a half times as long, and what counts is
+// how many times the chip is filled.  2,048 rows by 6,144 columns are 768 tiles of 128 (two fillings, the second
+// half empty) or 512 of 192 (one).
+static bool wider_tiles_take_fewer_rounds(int M, int N, int splits) {
+  const int64_t rows = (int64_t)((M + 127) / 128) * splits;
+  const int64_t fill_128 = (rows * ((N + 127) / 128) + 511) / 512, fill_192 = (rows * ((N + 191) / 192) + 511) / 512;
+  return 3 * fill_192 < 2 * fill_128;
+}
 
 // Into how many runs of k a plain product of M rows may be split when its partial sums are wanted apart.  Many
 // rows: a product whose tiles do not fill the chip twice, and that has k enough, goes faster in 2 to 4 runs, each
@@ -688,8 +699,12 @@ TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gat
     rc = launch_stream<4>(g, dual, out_act, 1, st, splits);
   } else {
     if ((N + TBN - 1) / TBN > 65535) return TQ_ERR_UNSUPPORTED;
-    rc = M <= 64 * 16 && !dual ? launch_tile<64, 2, 4>(g, dual, out_act, splits, st)
-                               : launch_tile<128, 4, 2>(g, dual, out_act, splits, st);
+    if (M <= 64 * 16 && !dual)
+      rc = launch_tile<64, 2, 4>(g, dual, out_act, splits, st);
+    else if (!dual && wider_tiles_take_fewer_rounds(M, N, splits))
+      rc = launch_tile<128, 4, 2, 192>(g, dual, out_act, splits, st);
+    else
+      rc = launch_tile<128, 4, 2>(g, dual, out_act, splits, st);
   }
   if (rc) return rc;
   TQ_LAUNCH_CHECK();
