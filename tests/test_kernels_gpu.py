@@ -84,7 +84,7 @@ def ref_gemm(a, w, bias=None, w2=None):
 
 @pytest.mark.parametrize("act", ACTS)
 @pytest.mark.parametrize("M,N,K", [(5, 33, 50), (1, 50, 72), (5, 130, 200), (16, 64, 64), (17, 33, 136), (40, 257, 264),
-                                   (64, 96, 1000), (65, 130, 72), (200, 300, 520), (300, 129, 64), (1130, 7400, 136)])
+                                   (64, 96, 1000), (65, 130, 72), (200, 300, 520), (300, 129, 64), (1130, 7400, 136), (2048, 4096, 72)])
 @pytest.mark.parametrize("mode", ["plain", "bias", "gated"])
 def test_gemm_dense(ops, act, M, N, K, mode):
     a = rnd((M, K), adt(act), 10)

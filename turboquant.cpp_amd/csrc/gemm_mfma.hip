@@ -365,8 +365,8 @@ __global__ __launch_bounds__(512) void qkv_rope_write_kernel(MfmaGemmArgs g, Rop
 
 // ------------------------------------------------------------------------------------------ many rows
 // grid (row tiles of BM, ceil(N / BN)); block of 8 waves laid WM x WN over the tile of BM x BN outputs (BN = 128
-// unless said): BM = 128 as 4 x 2 (a wave owns 32 x 64 outputs, or 32 x 96 with BN = 192), BM = 64 as 2 x 4 (32 x 32).  Eight waves of small tiles beat four of large ones here:
-// the step is bound by the way through LDS, and twice the waves hide twice the latency.
+// unless said): BM = 128 as 4 x 2 (a wave owns 32 x 64 outputs, or 32 x 96 with BN = 192), BM = 256 as 4 x 2 (64 x 64
+// or 64 x 96), BM = 64 as 2 x 4 (32 x 32).  Eight waves beat four here: twice the waves hide twice the latency.
 #define TBN 128
 #define TBK 64
 
@@ -632,14 +632,28 @@ static int launch_tile(const MfmaGemmArgs& g, bool dual, bool out_act, int split
 // once per 32 (measured at 151,936 x 2,048 and 64 rows: 159 us against 466 with 16 columns a wave).
 static bool wide_enough_for_tiles(int N) { return (N + TBN - 1) / TBN >= 512 && (N + TBN - 1) / TBN <= 65535; }
 
-// Tiles of 128 x 192 instead of 128 x 128 for a plain product: the chip holds 512 workgroups of either at a time
-// (256 compute units, two to each), a tile of 192 columns takes one and a half times as long, and what counts is
-// how many times the chip is filled.  2,048 rows by 6,144 columns are 768 tiles of 128 (two fillings, the second
-// half empty) or 512 of 192 (one).
-static bool wider_tiles_take_fewer_rounds(int M, int N, int splits) {
-  const int64_t rows = (int64_t)((M + 127) / 128) * splits;
-  const int64_t fill_128 = (rows * ((N + 127) / 128) + 511) / 512, fill_192 = (rows * ((N + 191) / 192) + 511) / 512;
-  return 3 * fill_192 < 2 * fill_128;
+// Which tile a plain product of many rows takes: 128 x 128, 128 x 192, 256 x 128 or 256 x 192 outputs (0..3).  The
+// larger the tile, the fewer bytes pass through LDS per multiply-add (measured on products that fill the chip
+// evenly: 1.06, 1.05 and 1.12 times the rate of 128 x 128); against that stand the compute units left idle when
+// the tiles do not divide evenly among the 256 of them, and the rows and columns of padding at the edges.  2,048
+// rows by 6,144 columns are 768, 512, 384 or 256 tiles: three, two, one and a half, or one to a compute unit.
+static int plain_tile_choice(int M, int N, int splits) {
+  static const int bm[4] = {128, 128, 256, 256}, bn[4] = {128, 192, 128, 192};
+  static const double rate[4] = {1.0, 1.06, 1.05, 1.12};
+  int best = 0;
+  double best_score = 0.0;
+  for (int c = 0; c < 4; ++c) {
+    const double rows = (M + bm[c] - 1) / bm[c], cols = (N + bn[c] - 1) / bn[c];
+    const double per_cu = rows * cols * splits / 256.0;
+    const double even = per_cu / (double)(int64_t)(per_cu + 0.999999);
+    const double useful = ((double)M * N) / (rows * bm[c] * cols * bn[c]);
+    const double score = rate[c] * even * useful;
+    if (score > best_score * 1.0001) {
+      best = c;
+      best_score = score;
+    }
+  }
+  return best;
 }
 
 // Into how many runs of k a plain product of M rows may be split when its partial sums are wanted apart.  Many
@@ -701,10 +715,15 @@ TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gat
     if ((N + TBN - 1) / TBN > 65535) return TQ_ERR_UNSUPPORTED;
     if (M <= 64 * 16 && !dual)
       rc = launch_tile<64, 2, 4>(g, dual, out_act, splits, st);
-    else if (!dual && wider_tiles_take_fewer_rounds(M, N, splits))
-      rc = launch_tile<128, 4, 2, 192>(g, dual, out_act, splits, st);
-    else
+    else if (dual)
       rc = launch_tile<128, 4, 2>(g, dual, out_act, splits, st);
+    else
+      switch (plain_tile_choice(M, N, splits)) {
+        case 1: rc = launch_tile<128, 4, 2, 192>(g, dual, out_act, splits, st); break;
+        case 2: rc = launch_tile<256, 4, 2, 128>(g, dual, out_act, splits, st); break;
+        case 3: rc = launch_tile<256, 4, 2, 192>(g, dual, out_act, splits, st); break;
+        default: rc = launch_tile<128, 4, 2>(g, dual, out_act, splits, st);
+      }
   }
   if (rc) return rc;
   TQ_LAUNCH_CHECK();
