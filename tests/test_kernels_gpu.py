@@ -2,6 +2,7 @@
 at sizes other than the engine's: widths and vocabularies that are no power of two, head sizes in steps
 of 16, odd numbers of heads and groups, rows that do not fill a tile."""
 import math
+import numpy as np
 
 import pytest
 import torch
@@ -653,12 +654,59 @@ def test_sample_topp_against_plain(ops):
             return self.u
 
     g = torch.Generator().manual_seed(120)
-    for V, T, P in [(4, 0.7, 0.9), (97, 0.7, 0.9), (1000, 1.3, 0.5), (5000, 0.3, 0.95), (300, 0.7, 1.0)]:
+    # (the last: logits in steps of 1/2, so that many probabilities are equal and the order of indices decides)
+    for V, T, P, step in [(4, 0.7, 0.9, 0), (97, 0.7, 0.9, 0), (1000, 1.3, 0.5, 0), (5000, 0.3, 0.95, 0),
+                          (300, 0.7, 1.0, 0), (2000, 1.5, 0.97, 0.5)]:
         logits = 3 * torch.randn((16, V), generator=g)
+        if step:
+            logits = torch.round(logits / step) * step
         u = torch.rand((16,), generator=g)
         got = ops.sample_topp(logits.to(DEV), T, P, u.to(DEV), "float32").cpu().tolist()
         want = [sample_topp(logits[r].numpy(), T, P, Fixed(float(u[r]))) for r in range(16)]
         assert got == want, (V, T, P)
+
+
+def sorted_walk_in_float64(logits, T, P, u, tol):
+    """The reference's walk (/root/reference/src/engine/tq_generate.c:81-156) with every sum in float64: the
+    token, and whether the same token comes out when every running sum is off by up to tol of itself (the place
+    where top_p is reached may then move, and with it the sum that the draw is scaled by)."""
+    l = logits.astype(np.float64)
+    p = np.where(l >= l.max() - 16.0 * T, np.exp((l - l.max()) / T), 0.0)
+    p /= p.sum()
+    order = np.argsort(-p, kind="stable")
+    cum = np.cumsum(p[order])
+
+    def first_reaching(x):
+        return int(np.argmax(cum >= x)) if (cum >= x).any() else len(cum) - 1
+
+    r = u * cum[first_reaching(P)]
+    k = first_reaching(r)
+    r_lo = u * cum[first_reaching(P * (1 - tol))] * (1 - tol)
+    r_hi = u * cum[first_reaching(P * (1 + tol))] * (1 + tol)
+    return int(order[k]), first_reaching(r_lo) == k and first_reaching(r_hi) == k
+
+
+def test_sample_topp_of_a_long_row(ops):
+    """Rows of a real vocabulary's length, a length that is no multiple of 4, lengths that exceed what a workgroup
+    loads at once, and logits in steps of 1/2 (many equal probabilities: the order of indices decides).  The plain
+    float32 walk adds 100,000 terms one after the other and is itself off by 1e-5 or so there, so the kernel is
+    held to the walk in float64 wherever that walk does not turn on 4e-6 of a sum, which is most rows.  (The
+    kernel adds at most 20 values in a thread, then 6 + 4 + 32 partial sums: 62 roundings of 2^-24 each at worst.)"""
+    g = torch.Generator().manual_seed(121)
+    for V, T, P, step in [(151936, 0.7, 0.9, 0), (70001, 1.0, 0.8, 0), (4000, 1.5, 0.97, 0.5), (151936, 1.0, 1.0, 0),
+                          (300000, 0.4, 0.95, 0)]:
+        logits = 3 * torch.randn((24, V), generator=g)
+        if step:
+            logits = torch.round(logits / step) * step
+        u = torch.rand((24,), generator=g)
+        got = ops.sample_topp(logits.to(DEV), T, P, u.to(DEV), "float32").cpu().tolist()
+        clear = 0
+        for r in range(24):
+            want, is_clear = sorted_walk_in_float64(logits[r].numpy(), T, P, float(u[r]), 4e-6)
+            if is_clear:
+                clear += 1
+                assert got[r] == want, (V, T, P, r)
+        assert clear >= 18, (V, clear)
 
 
 def test_sample_topp_distribution(ops):

@@ -45,7 +45,8 @@ _SIGNATURES = {
                  _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
     "tq_argmax": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr],
     "tq_rep_penalty": [_c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_ptr, _c_f32, _c_ptr],
-    "tq_sample_topp": [_c_ptr, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+    "tq_sample_topp_scratch": [_c_int],
+    "tq_sample_topp": [_c_ptr, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
 }
 # entry points that only the bfloat16 library has
 _OPTIONAL = {
@@ -95,6 +96,7 @@ def library(dtype) -> ctypes.CDLL:
         if hasattr(lib, fn):
             f = getattr(lib, fn)
             f.argtypes, f.restype = sig, _c_int
+    lib.tq_sample_topp_scratch.restype = _c_i64
     if hasattr(lib, "tq_attention_decode_scratch"):
         lib.tq_attention_decode_scratch.restype = _c_i64
     _LIBS[name] = lib
@@ -600,6 +602,8 @@ def sample_topp(logits: torch.Tensor, temperature: float, top_p: float, uniforms
     _need(temperature > 0 and top_p > 0, k, "temperature and top_p must be positive (else use argmax)")
     probs = torch.empty((R, V), dtype=torch.float32, device=logits.device)
     out = torch.empty((R,), dtype=torch.int32, device=logits.device)
-    _run(k, library(act).tq_sample_topp(_ptr(logits), R, V, float(temperature), float(top_p), _ptr(uniforms),
-                                        _ptr(probs), _ptr(out), _stream()))
+    lib = library(act)
+    scratch = torch.empty((lib.tq_sample_topp_scratch(R),), dtype=torch.float32, device=logits.device)
+    _run(k, lib.tq_sample_topp(_ptr(logits), R, V, float(temperature), float(top_p), _ptr(uniforms), _ptr(probs),
+                               _ptr(scratch), _ptr(out), _stream()))
     return out
