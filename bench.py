@@ -68,6 +68,42 @@ def prefill_flops(c, layers: int, T: int, rows_out: int = 1) -> float:
     return layers * per_layer + 2 * rows_out * H * c["vocab_size"]
 
 
+def probe() -> int:
+    """The measured counterparts of the published peaks: one JSON line."""
+    import torch
+    from turboquant_cpp_amd.csrc import ops
+    dev = "cuda:0"
+
+    def timed(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) * 1e-3 / reps
+
+    buf = torch.randint(0, 2 ** 31 - 1, (2 ** 28,), dtype=torch.int32, device=dev)      # 1 GiB
+    nbytes = buf.numel() * 4
+    out = {"metric": "measured peaks", "read_bytes": nbytes}
+    for name, once in (("read_GBs", False), ("read_once_hint_GBs", True)):
+        out[name] = round(nbytes / timed(lambda: ops.probe_stream(buf, once), 10) / 1e9, 0)
+    del buf
+    for shape in (32, 16):
+        for name, seed in (("same_values", 0), ("random_values", 12345)):
+            flop = [0.0]
+
+            def run():
+                flop[0] = ops.probe_mfma(shape, 512, 20000, seed, dev)
+            t = timed(run, 3)
+            out[f"mfma_{shape}_{name}_TFLOPs"] = round(flop[0] / t / 1e12, 0)
+    out["published"] = {"hbm_GBs": PEAK_HBM_GBS, "bf16_TFLOPs": PEAK_FLOPS["bf16"] / 1e12}
+    print(json.dumps(out))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -81,10 +117,14 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true")
     ap.add_argument("--prefill-only", action="store_true", help="time only the prompt step (for profiles)")
+    ap.add_argument("--probe", action="store_true",
+                    help="no model: what this GPU reaches on a plain read of memory and on the matrix instructions alone")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single device)")
         return 2
+    if args.probe:
+        return probe()
 
     import torch
     from turboquant_cpp_amd.csrc import ops

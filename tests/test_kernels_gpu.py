@@ -771,3 +771,14 @@ def test_attention_tiled(ops, nh, nkv, hd, window, page):
     assert run([0, 7, 100, 300]) < tol(act, 2)                   # runs that go on from a cached prefix
     assert run([n - 1 for n in lens]) < tol(act, 2)              # one token each: the split kernel
     assert run([1, 18, 149, 200]) < tol(act, 2)                  # mixed: not all single tokens
+
+
+def test_probes_run(ops):
+    """The two kernels behind `bench.py --probe` (a plain read, the matrix instructions alone) launch and finish;
+    the second reports how many operations it did."""
+    buf = torch.arange(1 << 20, dtype=torch.int32, device=DEV)
+    for once in (False, True):
+        ops.probe_stream(buf, once)
+    assert ops.probe_mfma(32, 4, 10, 1, DEV) == 4 * 8 * 10 * 196608.0
+    assert ops.probe_mfma(16, 4, 10, 0, DEV) == 4 * 8 * 10 * 196608.0
+    torch.cuda.synchronize()

@@ -20,7 +20,7 @@ CSRC = os.path.dirname(os.path.abspath(__file__))
 COMMON_SOURCES = ["elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "moe.hip", "sampling.hip"]
 SOURCES = {
     "float32": COMMON_SOURCES,
-    "bfloat16": COMMON_SOURCES + ["gemm_mfma.hip", "attention_mfma.hip"],
+    "bfloat16": COMMON_SOURCES + ["gemm_mfma.hip", "attention_mfma.hip", "probe.hip"],
 }
 HEADERS = ["common.h", "mfma.h"]
 DEFINES = {"float32": "-DTQ_ACT_F32", "bfloat16": "-DTQ_ACT_BF16"}

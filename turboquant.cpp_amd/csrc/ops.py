@@ -57,6 +57,8 @@ _OPTIONAL = {
     "tq_gemm_mfma_pair": [_c_ptr, _c_ptr, _c_int, _c_ptr],
     "tq_qkv_rope_write": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr,
                           _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_ptr],
+    "tq_probe_stream": [_c_ptr, _c_i64, _c_int, ctypes.c_uint, _c_ptr, _c_ptr],
+    "tq_probe_mfma": [_c_int, _c_int, _c_int, ctypes.c_uint, _c_ptr, _c_ptr],
     "tq_attention_decode_scratch": [_c_int, _c_int, _c_int, _c_int],
     "tq_attention_mfma": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int,
                           _c_int, _c_int, _c_int, _c_f32, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
@@ -607,3 +609,22 @@ def sample_topp(logits: torch.Tensor, temperature: float, top_p: float, uniforms
     _run(k, lib.tq_sample_topp(_ptr(logits), R, V, float(temperature), float(top_p), _ptr(uniforms), _ptr(probs),
                                _ptr(scratch), _ptr(out), _stream()))
     return out
+
+
+# ------------------------------------------------------------------------------------------------ probes
+def probe_stream(buf: torch.Tensor, once: bool) -> None:
+    """One read of all of ``buf`` (whole lines of 128 bytes per instruction; ``once``: with the read-once hint)."""
+    k = "probe_stream"
+    _need(buf.is_cuda and buf.is_contiguous(), k, "buf must be a contiguous tensor on the GPU")
+    nbytes = buf.numel() * buf.element_size()
+    out = torch.zeros((1,), dtype=torch.int32, device=buf.device)
+    _run(k, library("bfloat16").tq_probe_stream(_ptr(buf), nbytes, int(once), 0x9e3779b9, _ptr(out), _stream()))
+
+
+def probe_mfma(shape: int, workgroups: int, iters: int, seed: int, device) -> float:
+    """A loop of bfloat16 matrix instructions alone (shape 32: 32x32x16, 16: 16x16x32); returns the number of
+    floating-point operations that the launch does."""
+    k = "probe_mfma"
+    out = torch.empty((workgroups * 512,), dtype=torch.float32, device=device)
+    _run(k, library("bfloat16").tq_probe_mfma(shape, workgroups, iters, seed, _ptr(out), _stream()))
+    return float(workgroups) * 8 * iters * 196608.0
