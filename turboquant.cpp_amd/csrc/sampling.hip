@@ -156,14 +156,15 @@ __device__ __forceinline__ float candidate(uint32_t lo_b, uint32_t hi_b, int j) 
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-// NB units of VEC floats for this thread, all asked for before any is used.  Unit u starts at element
-// first + unit_of(u) * VEC; what lies at or beyond `end` reads as `pad`.  (With VEC 4, first and end are multiples
-// of 4 and the row is aligned to 16 bytes.)
+// A thread fetches NB units of VEC floats at a time, all asked for before any is used.  Where unit u starts,
+// counted from `first`: with OWN_RUN a thread's units follow one another, else the threads' units interleave (a
+// wave's loads take whole lines).
 template <int VEC, bool OWN_RUN>
 __device__ __forceinline__ int unit_start(int first, int u) {
-  // OWN_RUN: a thread's units follow one another; else the threads' units interleave (whole lines per wave)
   return first + (OWN_RUN ? (int)threadIdx.x * NB + u : u * SB + (int)threadIdx.x) * VEC;
 }
+// What lies at or beyond `end` reads as `pad`.  (With VEC 4, first and end are multiples of 4 and the row is aligned
+// to 16 bytes.)
 template <int VEC, bool OWN_RUN>
 __device__ __forceinline__ void load_units(const float* __restrict__ base, int first, int end, float pad,
                                            float (&v)[NB][VEC]) {
