@@ -117,6 +117,9 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true")
     ap.add_argument("--prefill-only", action="store_true", help="time only the prompt step (for profiles)")
+    ap.add_argument("--one-stream", action="store_true",
+                    help="no second stream in prompt steps: kernels run one after the other, so that a profile shows "
+                         "each kernel's own time")
     ap.add_argument("--probe", action="store_true",
                     help="no model: what this GPU reaches on a plain read of memory and on the matrix instructions alone")
     args = ap.parse_args()
@@ -208,6 +211,8 @@ def main() -> int:
 
     def run_prefill(T: int):
         engine = Engine(model, max_tokens=T + 64, page_size=64, max_slots=1)
+        if args.one_stream:
+            engine.side_stream = None
         prompt = torch.randint(0, V, (T,), generator=gen).tolist()
         times = []
         for i in range(3):
