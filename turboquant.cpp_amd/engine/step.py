@@ -131,8 +131,7 @@ class Engine:
         return starts
 
     def _eager(self, batch) -> torch.Tensor:
-        # a second stream for what does not depend on the main line: the shared expert runs beside the routing
-        # kernels, which are short and leave the chip empty (5 % of a prompt step of 2,048 tokens)
+        # a second stream for what does not depend on the main line (the parts decide what they put there)
         ctx = StepContext(batch=batch, cache=self.cache, act=self.model.act, device=self.device,
                           side_stream=self.side_stream)
         return self.model.forward(ctx)
