@@ -275,19 +275,20 @@ TQ_API int tq_router_topk(const float* x, const void* wr, const void* shared_w, 
 // number), gives it its rank among them in order of lane and adds their number to its count of the expert.
 // After a barrier the counts of all waves give every expert's first row and every wave's first row within
 // the expert, and each pair's row is that plus its rank.
-#define AW 16   // waves
+#define AW 16   // waves (one where a single token is ordered: the result does not depend on their number)
 
-// ids may lie in LDS or in memory; cnt: (AW + 1) * E ints of LDS ([AW][E] counts, then E starts).  All AW waves
+// ids may lie in LDS or in memory; cnt: (NW + 1) * E ints of LDS ([NW][E] counts, then E starts).  All NW waves
 // of the workgroup call it together.
+template <int NW>
 __device__ __forceinline__ void align_pairs(const int* ids, int n_pairs, int E, int topk, int unit, int cap,
                                             int* __restrict__ sorted_token, int* __restrict__ pair_slot,
                                             int* __restrict__ tile_expert, int* __restrict__ n_tiles, int* cnt) {
-  int* starts = cnt + AW * E;
+  int* starts = cnt + NW * E;
   const int wave = threadIdx.x / TQ_WAVE, lane = threadIdx.x % TQ_WAVE;
   for (int i = threadIdx.x; i < cap; i += blockDim.x) sorted_token[i] = -1;
-  for (int i = threadIdx.x; i < AW * E; i += blockDim.x) cnt[i] = 0;
+  for (int i = threadIdx.x; i < NW * E; i += blockDim.x) cnt[i] = 0;
   __syncthreads();
-  const int per = ((n_pairs + AW - 1) / AW + TQ_WAVE - 1) / TQ_WAVE * TQ_WAVE;   // pairs per wave, whole batches
+  const int per = ((n_pairs + NW - 1) / NW + TQ_WAVE - 1) / TQ_WAVE * TQ_WAVE;   // pairs per wave, whole batches
   const int seg_beg = wave * per, seg_end = min(n_pairs, seg_beg + per);
   int* mine = cnt + wave * E;
   // with at most 64 pairs per wave a thread meets its pair again in the last loop (i == threadIdx.x both times):
@@ -321,7 +322,7 @@ __device__ __forceinline__ void align_pairs(const int* ids, int n_pairs, int E, 
   // counts become each wave's first row within its expert; starts[e] first holds the expert's padded size
   for (int e = threadIdx.x; e < E; e += blockDim.x) {
     int total = 0;
-    for (int w = 0; w < AW; ++w) {
+    for (int w = 0; w < NW; ++w) {
       const int c = cnt[w * E + e];
       cnt[w * E + e] = total;
       total += c;
@@ -374,12 +375,13 @@ __global__ __launch_bounds__(64 * AW) void moe_align_kernel(const int* __restric
                                                             int* __restrict__ tile_expert,
                                                             int* __restrict__ n_tiles) {
   extern __shared__ int cnt[];
-  align_pairs(ids, n_pairs, E, topk, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles, cnt);
+  align_pairs<AW>(ids, n_pairs, E, topk, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles, cnt);
 }
 
-// The choice and the order of pairs in one workgroup, for up to AW tokens (decoding): wave w chooses for token w,
+// The choice and the order of pairs in one workgroup of NW waves, for up to NW tokens (decoding): wave w chooses for token w,
 // then all waves order the pairs; the same device functions and so the same results as the two kernels.
-__global__ __launch_bounds__(64 * AW) void select_align_kernel(const float* __restrict__ logits, int rows, int E,
+template <int NW>
+__global__ __launch_bounds__(64 * NW) void select_align_kernel(const float* __restrict__ logits, int rows, int E,
                                                                int topk, int renorm, int* __restrict__ ids,
                                                                float* __restrict__ weights,
                                                                float* __restrict__ shared_gate, int T, int unit,
@@ -387,16 +389,16 @@ __global__ __launch_bounds__(64 * AW) void select_align_kernel(const float* __re
                                                                int* __restrict__ pair_slot,
                                                                int* __restrict__ tile_expert,
                                                                int* __restrict__ n_tiles) {
-  extern __shared__ int sm_i[];       // (AW + 1) * E ints for the order, AW * topk ids, AW * E floats for the choice
+  extern __shared__ int sm_i[];       // (NW + 1) * E ints for the order, NW * topk ids, NW * E floats for the choice
   int* cnt = sm_i;
-  int* ids_l = cnt + (AW + 1) * E;
-  float* lg = (float*)(ids_l + AW * topk);
+  int* ids_l = cnt + (NW + 1) * E;
+  float* lg = (float*)(ids_l + NW * topk);
   const int wave = threadIdx.x / TQ_WAVE;
   if (wave < T)
     select_token(logits + (size_t)wave * rows, rows, E, topk, renorm, lg + wave * E, ids + (size_t)wave * topk,
                  ids_l + wave * topk, weights + (size_t)wave * topk, shared_gate + wave);
   __syncthreads();
-  align_pairs(ids_l, T * topk, E, topk, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles, cnt);
+  align_pairs<NW>(ids_l, T * topk, E, topk, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles, cnt);
 }
 
 // cap: rows that sorted_token holds, a multiple of unit and at least n_pairs + min(E, n_pairs) * (unit - 1);
@@ -430,9 +432,16 @@ TQ_API int tq_route(const float* x, const void* wr, const void* shared_w, int wt
   if (unit < 1 || cap % unit != 0 || cap < n_pairs + (E < n_pairs ? E : n_pairs) * (unit - 1)) return TQ_ERR_BAD_ARG;
   const int rc = launch_router_logits(x, wr, shared_w, wtype, E, logits, T, H, st);
   if (rc) return rc;
+  if (T == 1) {      // one wave: its barriers cost nothing
+    const size_t shmem1 = ((size_t)2 * E + topk + E) * 4;
+    hipLaunchKernelGGL(select_align_kernel<1>, dim3(1), dim3(64), shmem1, st, logits, E + (shared_w ? 1 : 0), E, topk,
+                       renorm, ids, weights, shared_gate, T, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles);
+    TQ_LAUNCH_CHECK();
+    return 0;
+  }
   if (shmem > 48 * 1024)
-    hipFuncSetAttribute((const void*)select_align_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
-  hipLaunchKernelGGL(select_align_kernel, dim3(1), dim3(64 * AW), shmem, st, logits, E + (shared_w ? 1 : 0), E, topk,
+    hipFuncSetAttribute((const void*)select_align_kernel<AW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+  hipLaunchKernelGGL(select_align_kernel<AW>, dim3(1), dim3(64 * AW), shmem, st, logits, E + (shared_w ? 1 : 0), E, topk,
                      renorm, ids, weights, shared_gate, T, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles);
   TQ_LAUNCH_CHECK();
   return 0;
