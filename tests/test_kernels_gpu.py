@@ -566,12 +566,14 @@ def test_attention_finds_a_far_key(ops, act):
 
 @pytest.mark.parametrize("window", [None, 3000])
 def test_decoding_over_long_caches(ops, window):
-    """One token per sequence at positions on both sides of every length at which the split kernel changes the
-    length of its runs (2048, 4096, 6144) and well beyond, in one batch; in each sequence one far key stands out a
-    little, so that a run that is skipped or joined twice shows.  Against the plain formula for the last token."""
+    """One token per sequence at positions on both sides of the length at which the split kernel changes the
+    length of its runs (4096), of other multiples of 2048 and well beyond, in one batch: the sequences of 3,500 and
+    4,095 tokens have more runs (one per 64 positions) than the longest one (one per 192), after which the grid is
+    sized.  In each sequence one far key stands out a little, so that a run that is skipped or joined twice shows.
+    Against the plain formula for the last token."""
     act = "bfloat16"
     nh, nkv, hd, page = 6, 2, 64, 64
-    lens = [2047, 2048, 2049, 4095, 4097, 6143, 6145, 9001, 130]
+    lens = [2047, 2048, 2049, 4095, 4097, 6143, 6145, 9001, 130, 3500]
     table, slots, page_stride, kp, vp = paged_setup(lens, page, nkv, hd, 1, act, 95)
     scale = 1.0 / math.sqrt(hd)
     g = torch.Generator().manual_seed(96)
@@ -606,7 +608,7 @@ def test_decoding_over_long_caches(ops, window):
     err = (out.double() - torch.stack(want)).abs().max(dim=1).values
     assert err.max() < 2e-2, err
     # each sequence alone gives the same bits: what a run is depends on the token's position only
-    for i in (1, 4, 7):
+    for i in (1, 3, 4, 7):
         runs1 = {"cu_seqlens": torch.tensor([0, 1], dtype=torch.int32).to(DEV), "slots": torch.tensor([slots[i]], dtype=torch.int32).to(DEV),
                  "start": positions[i:i + 1].to(DEV), "max_new": 1, "max_end": lens[i], "decode": True}
         alone = ops.attention(qs[i].reshape(1, nh * hd).to(DEV), kp.to(DEV), vp.to(DEV), 0, positions[i:i + 1].to(DEV),

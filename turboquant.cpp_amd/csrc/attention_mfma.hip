@@ -17,7 +17,7 @@
 //
 // Two entry points share this: whole prompts (columns = 16 consecutive tokens of a sequence, one head; four
 // waves per workgroup) and decoding (columns = the query heads that share one kv head, one token; the cache is
-// split into runs of 1 to 3 tiles, one wave each, and a second kernel joins the runs in order).  Tiles start at
+// split into runs of 1 or 3 tiles, one wave each, and a second kernel joins the runs in order).  Tiles start at
 // multiples of 64 positions and runs at multiples of the run length, so the order of every sum depends only on
 // the token's own position.
 #include "common.h"
@@ -30,13 +30,15 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 #define TILE 64
 #define LOG2E 1.4426950408889634f
 // Tiles per run when decoding a token at position p: short sequences are cut finer, so that a small batch still
-// gives the chip hundreds of waves; a function of the token's own position only.  Measured at position 8191 with
-// 16 kv heads: 3 tiles per run beat 4 by 15 % at 8 sequences and lose 2 to 4 % from 16 on.
-__host__ __device__ __forceinline__ int tiles_per_run(int p) { return p >= 2 * 2048 ? 3 : p / 2048 + 1; }
+// gives the chip hundreds of waves; a function of the token's own position only.  Measured with 16 kv heads: at
+// position 8191, 3 tiles per run beat 4 by 15 % at 8 sequences and lose 2 to 4 % from 16 on, 2 lose 9 % and 1 loses
+// 22 %; at positions 3000 and 4000, 1 tile per run beats 2 by 25 % and 9 % at 8 sequences (4 % and -2 % at 64).
+__host__ __device__ __forceinline__ int tiles_per_run(int p) { return p >= 2 * 2048 ? 3 : 1; }
+__host__ __device__ __forceinline__ int runs_at(int p) { return p / TILE / tiles_per_run(p) + 1; }
 // Most runs that a token at a position below max_end can have.
 static int most_runs(int max_end) {
   const int tiles = (max_end + 63) / 64;
-  const int short_runs = tiles < 32 ? tiles : 32;          // below position 4096 no token has more than 32
+  const int short_runs = tiles < 64 ? tiles : 64;          // below position 4096 no token has more than 64
   const int long_runs = (tiles + 2) / 3;
   return short_runs > long_runs ? short_runs : long_runs;
 }
@@ -405,20 +407,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 }
 
 // ------------------------------------------------------------------------------------------ decoding
-// One new token per sequence at position start[b].  grid (max_runs, nkv * ceil(g / 16), B), block 64: the wave
+// One new token per sequence at position start[b].  grid (runs, nkv * ceil(g / 16), B), block 64: the wave
 // takes run x (tiles S x .. S x + S - 1, S = tiles_per_run(position)) for up to 16 of the g = nh / nkv heads of one kv head and
-// writes their unnormalised sums with maximum and denominator.
+// writes their unnormalised sums with maximum and denominator.  The grid has the runs of the step's longest
+// sequence, so that no wave is started for nothing where all sequences are about as long (a wave that finds no run
+// costs as much to start as one that does: a third more of them made the kernel a fifth slower).  A shorter
+// sequence of the same step may still have more runs than that, positions below 4096 being cut finer: the wave of
+// the grid's last run then takes all of the sequence's further runs, one after the other, each into its own place.
 template <int DT, bool EXACT>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DT > 8 ? 2 : 3))) void attn_decode_kernel(AttnArgs a) {
-  const int b = blockIdx.z, run = blockIdx.x;
+  const int b = blockIdx.z;
   const int g = a.nh / a.nkv, ngc = (g + 15) / 16;
   const int kvh = blockIdx.y / ngc, cg = blockIdx.y % ngc;
   const int lane = threadIdx.x, r = lane % 16, c = lane / 16;
   const int p = a.start[b];
   const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
-  const int S = tiles_per_run(p);
-  const int tile_beg = max(run * S, lo / TILE), tile_end = min((run + 1) * S, p / TILE + 1);
-  if (tile_beg >= tile_end) return;
+  const int S = tiles_per_run(p), n_runs = runs_at(p);
+  if ((int)blockIdx.x >= n_runs) return;
   const int hg = cg * 16 + r;                 // head within the group
   const bool valid = hg < g;
   const int h = kvh * g + (valid ? hg : 0);
@@ -428,24 +433,29 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DT > 8 ? 2 :
 
   bf16x8 qf[1][(DT + 1) / 2];
   load_query<DT>(qf[0], a.q + ((size_t)t * a.nh + h) * a.hd, a.hd, valid);
-  f32x4 o[1][DT];
+  const int run_end = blockIdx.x + 1 == gridDim.x ? n_runs : (int)blockIdx.x + 1;
+  for (int run = blockIdx.x; run < run_end; ++run) {
+    const int tile_beg = max(run * S, lo / TILE), tile_end = min((run + 1) * S, p / TILE + 1);
+    if (tile_beg >= tile_end) continue;       // all of the run lies before the window
+    f32x4 o[1][DT];
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) o[0][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m_run[1] = {-INFINITY}, l_run[1] = {0.f};
-  attend<DT, EXACT>(o, m_run, l_run, qf, a.k_pool + head_off, a.v_pool + head_off, table, a.page_size, a.page_stride, a.hd,
-             tile_beg, tile_end, p, valid, lo, a.scale * LOG2E);
-  if (!valid) return;
-  float* out = a.partial + (((size_t)b * a.nh + h) * a.max_runs + run) * (a.hd + 2);
+    for (int dt = 0; dt < DT; ++dt) o[0][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run[1] = {-INFINITY}, l_run[1] = {0.f};
+    attend<DT, EXACT>(o, m_run, l_run, qf, a.k_pool + head_off, a.v_pool + head_off, table, a.page_size, a.page_stride,
+                      a.hd, tile_beg, tile_end, p, valid, lo, a.scale * LOG2E);
+    if (!valid) continue;
+    float* out = a.partial + (((size_t)b * a.nh + h) * a.max_runs + run) * (a.hd + 2);
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) {
-    if (16 * dt < a.hd) {
+    for (int dt = 0; dt < DT; ++dt) {
+      if (16 * dt < a.hd) {
 #pragma unroll
-      for (int v = 0; v < 4; ++v) out[16 * dt + 4 * c + v] = o[0][dt][v];
+        for (int v = 0; v < 4; ++v) out[16 * dt + 4 * c + v] = o[0][dt][v];
+      }
     }
-  }
-  if (c == 0) {
-    out[a.hd] = m_run[0];
-    out[a.hd + 1] = l_run[0];
+    if (c == 0) {
+      out[a.hd] = m_run[0];
+      out[a.hd + 1] = l_run[0];
+    }
   }
 }
 
@@ -510,9 +520,9 @@ static int launch_prefill(const AttnArgs& a, int B, int max_new, hipStream_t st)
   return 0;
 }
 template <int DT, bool EXACT>
-static void launch_decode(const AttnArgs& a, int B, hipStream_t st) {
+static void launch_decode(const AttnArgs& a, int B, int grid_runs, hipStream_t st) {
   const int g = a.nh / a.nkv;
-  hipLaunchKernelGGL((attn_decode_kernel<DT, EXACT>), dim3(a.max_runs, a.nkv * ((g + 15) / 16), B), dim3(64), 0, st, a);
+  hipLaunchKernelGGL((attn_decode_kernel<DT, EXACT>), dim3(grid_runs, a.nkv * ((g + 15) / 16), B), dim3(64), 0, st, a);
   hipLaunchKernelGGL(attn_join_kernel, dim3(a.nh, B), dim3(64), 0, st, a);
 }
 
@@ -539,12 +549,13 @@ TQ_API int tq_attention_mfma(const void* q, const void* k_pool, const void* v_po
   // head sizes 64, 128 and 256 have kernels of their own in which nothing depends on hd at run time
   if (decode) {
     if (!partial) return TQ_ERR_BAD_ARG;
-    if (dt == 4) launch_decode<4, true>(a, B, st);
-    else if (dt == 8) launch_decode<8, true>(a, B, st);
-    else if (dt == 16) launch_decode<16, true>(a, B, st);
-    else if (dt < 4) launch_decode<4, false>(a, B, st);
-    else if (dt < 8) launch_decode<8, false>(a, B, st);
-    else launch_decode<16, false>(a, B, st);
+    const int grid_runs = runs_at(max_end > 0 ? max_end - 1 : 0);      // the runs of the step's longest sequence
+    if (dt == 4) launch_decode<4, true>(a, B, grid_runs, st);
+    else if (dt == 8) launch_decode<8, true>(a, B, grid_runs, st);
+    else if (dt == 16) launch_decode<16, true>(a, B, grid_runs, st);
+    else if (dt < 4) launch_decode<4, false>(a, B, grid_runs, st);
+    else if (dt < 8) launch_decode<8, false>(a, B, grid_runs, st);
+    else launch_decode<16, false>(a, B, grid_runs, st);
   } else {
     // two groups of 16 tokens per wave, which halves the reads from LDS per product, when that still leaves
     // the chip two workgroups per compute unit and registers allow; else one group
