@@ -76,8 +76,8 @@ class SparseMoE(Part):
                                       dict(a=hs, w=self.shared_down, partial_sums=True), ctx.act)
             return ops.GatheredSum(y, pair_slot, weights, shared, gate)
         # The shared expert needs nothing from the router: it may run on a second stream beside the routed experts.
-        # That pays while its products are a few rounds of tiles over the chip, whose ends the other stream's work
-        # fills (2,048 tokens of width 5,632: 5 % of the step; 512 tokens: 10 %); with eight rounds and more the two
+        # That pays while its products are a few passes of tiles over the chip, whose ends the other stream's work
+        # fills (2,048 tokens of width 5,632: 5 % of the step; 512 tokens: 10 %); with eight passes and more the two
         # only disturb each other (2,048 tokens of width 20,480: 2 % slower).
         shared, side = None, None
         if self.shared_size > 0:
