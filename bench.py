@@ -120,6 +120,9 @@ def main() -> int:
     ap.add_argument("--one-stream", action="store_true",
                     help="no second stream in prompt steps: kernels run one after the other, so that a profile shows "
                          "each kernel's own time")
+    ap.add_argument("--generate", action="store_true",
+                    help="time the generation loop instead of bare steps: --batch prompts of 512 tokens, 256 new tokens "
+                         "each, greedy and with the default sampling (temperature 0.7, top-p 0.9, repetition penalty)")
     ap.add_argument("--probe", action="store_true",
                     help="no model: what this GPU reaches on a plain read of memory and on the matrix instructions alone")
     args = ap.parse_args()
@@ -152,6 +155,25 @@ def main() -> int:
           f"({model.weight_bytes / 1e9:.1f} GB)", file=sys.stderr, flush=True)
     V = cfg["vocab_size"]
     gen = torch.Generator().manual_seed(2)
+
+    if args.generate:
+        from turboquant_cpp_amd.engine.generate import GenerationOptions, generate
+        P, N, B = 512, 256, args.batch
+        engine = Engine(model, max_tokens=(P + N + 64) * B, page_size=64, max_slots=B)
+        prompts = [torch.randint(0, V, (P,), generator=gen).tolist() for _ in range(B)]
+        out = {"metric": f"generated tok/s, {B} prompts of {P} tokens, {N} new tokens each ({model_name}, random weights)",
+               "unit": "tok/s", "dtype": short, "layers": args.layers}
+        for name, opts in (("greedy", dict(temperature=0.0, rep_penalty=1.0)), ("default_sampling", dict())):
+            for _ in range(2):      # the first pass loads kernels and captures the decode step
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                res = generate(engine, prompts, GenerationOptions(max_tokens=N, max_batch=B, loop_detection=False, **opts))
+                torch.cuda.synchronize()
+                dt = time.perf_counter() - t0
+            n = sum(len(r.tokens) for r in res)
+            out[name] = {"value": round(n / dt, 1), "tokens": n, "seconds": round(dt, 3)}
+        print(json.dumps(out))
+        return 0
 
     def run_decode(batch: int, context: int, steps: int, warmup: int):
         """Prefills `batch` prompts so that the timed steps end at `context`, then times `steps` decode steps."""
