@@ -642,6 +642,20 @@ def test_rep_penalty(ops):
     apply_rep_penalty(ref[0], [3, 7, 3], 4, 1.1)       # token 3 twice: penalised twice
     apply_rep_penalty(ref[1], [2, 1, 0, 49], 4, 1.1)
     assert (d.cpu() - torch.from_numpy(ref)).abs().max() < 1e-6
+    # histories of 100 entries (a thread per entry) and of 200 (one thread walks them), tokens drawn from 20 so that
+    # most occur several times; the same bits as the walk in float32
+    g = torch.Generator().manual_seed(111)
+    for window in (100, 200):
+        logits = rnd((3, V), torch.float32, 112)
+        recent = torch.randint(0, 20, (3, window), generator=g).to(torch.int32)
+        counts = torch.tensor([window, window // 2, 0], dtype=torch.int32)
+        d = logits.clone().to(DEV)
+        ops.rep_penalty(d, recent.to(DEV), counts.to(DEV), 1.3, "float32")
+        ref = logits.numpy().copy()
+        for r in range(3):
+            n = int(counts[r])
+            apply_rep_penalty(ref[r], recent[r, :n].tolist()[::-1], window, 1.3)
+        assert torch.equal(d.cpu(), torch.from_numpy(ref)), window
 
 
 def test_sample_topp_against_plain(ops):

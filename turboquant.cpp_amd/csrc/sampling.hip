@@ -64,8 +64,35 @@ TQ_API int tq_argmax(const float* logits, int R, int V, int* out, hipStream_t st
 // ---------------------------------------------------------------- repetition penalty
 // For each of the last `count` tokens of a row's history, once per occurrence: a positive logit is
 // divided by the penalty, any other multiplied (/root/reference/src/engine/tq_generate.c:387-400).
-__global__ void rep_penalty_kernel(float* __restrict__ logits, int V, const int* __restrict__ recent, int window,
-                                   const int* __restrict__ counts, float penalty) {
+// One workgroup per row, a thread per entry of the history: the thread that holds a token's first entry counts the
+// token's entries and applies the penalty that many times, one after the other as the walk over the history would
+// (the sign of a logit does not change on the way, so the order of the entries does not matter).
+#define RP_MAX 128      // entries of history per row that the parallel kernel takes
+__global__ __launch_bounds__(RP_MAX) void rep_penalty_kernel(float* __restrict__ logits, int V,
+                                                             const int* __restrict__ recent, int window,
+                                                             const int* __restrict__ counts, float penalty) {
+  __shared__ int toks[RP_MAX];
+  float* row = logits + (size_t)blockIdx.x * V;
+  const int n = min(counts[blockIdx.x], window), r = threadIdx.x;
+  const int tok = r < n ? recent[blockIdx.x * window + r] : -1;
+  toks[r] = tok;
+  __syncthreads();
+  if (tok < 0 || tok >= V) return;
+  int times = 0;
+  for (int j = 0; j < n; ++j) {
+    if (toks[j] == tok) {
+      if (j < r) return;      // an earlier entry holds the token and does the work
+      ++times;
+    }
+  }
+  float v = row[tok];
+  for (int t = 0; t < times; ++t) v = v > 0.f ? v / penalty : v * penalty;
+  row[tok] = v;
+}
+
+// The same for longer histories: one thread walks the row's history.
+__global__ void rep_penalty_walk_kernel(float* __restrict__ logits, int V, const int* __restrict__ recent, int window,
+                                        const int* __restrict__ counts, float penalty) {
   if (threadIdx.x != 0) return;
   float* row = logits + (size_t)blockIdx.x * V;
   const int n = min(counts[blockIdx.x], window);
@@ -78,7 +105,10 @@ __global__ void rep_penalty_kernel(float* __restrict__ logits, int V, const int*
 TQ_API int tq_rep_penalty(float* logits, int R, int V, const int* recent, int window, const int* counts,
                           float penalty, hipStream_t st) {
   if (R <= 0) return 0;
-  hipLaunchKernelGGL(rep_penalty_kernel, dim3(R), dim3(64), 0, st, logits, V, recent, window, counts, penalty);
+  if (window <= RP_MAX)
+    hipLaunchKernelGGL(rep_penalty_kernel, dim3(R), dim3(RP_MAX), 0, st, logits, V, recent, window, counts, penalty);
+  else
+    hipLaunchKernelGGL(rep_penalty_walk_kernel, dim3(R), dim3(64), 0, st, logits, V, recent, window, counts, penalty);
   TQ_LAUNCH_CHECK();
   return 0;
 }

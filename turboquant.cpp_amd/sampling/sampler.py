@@ -44,6 +44,22 @@ class Sampler:
     def __init__(self, options: SamplingOptions, act: str, device):
         self.options, self.act, self.device = options, act, device
         self.window = max(0, min(options.rep_window, 128))    # the reference caps the window at 128 (:367)
+        self._staging = None
+
+    def _staged(self, rows: int) -> dict:
+        """Host arrays that the step's small inputs (recent tokens, their counts, the uniform draws) are written
+        into before they go to the device: pinned where there is a GPU, so that the copies are issued without the
+        host waiting for the stream (a copy from ordinary memory returns only when everything issued before it has
+        run, the whole decode step included).  They are written again at the next ``launch``; by then the tokens of
+        this one have been fetched, so its copies have run."""
+        if self._staging is None or self._staging["rows"] < rows:
+            pin = self.device is not None and torch.device(self.device).type == "cuda"
+            n = max(rows, 8)
+            self._staging = {"rows": n,
+                             "recent": torch.empty((n, max(self.window, 1)), dtype=torch.int32, pin_memory=pin),
+                             "counts": torch.empty((n,), dtype=torch.int32, pin_memory=pin),
+                             "uniforms": torch.empty((n,), dtype=torch.float32, pin_memory=pin)}
+        return self._staging
 
     def new_sequence(self, index: int, prompt: list[int]) -> SequenceSampling:
         st = SequenceSampling(XorShift64Star(stream_seed(self.options.seed, index)))
@@ -61,19 +77,22 @@ class Sampler:
         """Issues the choice and returns the tokens as int32 [R] on the device; ``finish`` must be told the
         tokens before the next ``launch`` for the same sequences."""
         o, R = self.options, logits.shape[0]
+        staged = self._staged(R)
         if o.rep_penalty > 1.0 and self.window > 0:
-            recent = np.full((R, self.window), -1, dtype=np.int32)
-            counts = np.zeros(R, dtype=np.int32)
+            recent, counts = staged["recent"][:R], staged["counts"][:R]
+            recent_np, counts_np = recent.numpy(), counts.numpy()
+            recent_np.fill(-1)
             for i, st in enumerate(states):
                 tail = st.recent[-self.window:][::-1]      # newest first, the reference's order
-                recent[i, :len(tail)] = tail
-                counts[i] = len(tail)
-            ops.rep_penalty(logits, torch.from_numpy(recent).to(self.device), torch.from_numpy(counts).to(self.device),
+                recent_np[i, :len(tail)] = tail
+                counts_np[i] = len(tail)
+            ops.rep_penalty(logits, recent.to(self.device, non_blocking=True), counts.to(self.device, non_blocking=True),
                             o.rep_penalty, self.act)
         if o.greedy:
             return ops.argmax(logits, self.act)
-        u = np.array([st.rng.next_float() for st in states], dtype=np.float32)
-        return ops.sample_topp(logits, o.temperature, o.top_p, torch.from_numpy(u).to(self.device), self.act)
+        u = staged["uniforms"][:R]
+        u.numpy()[:] = [st.rng.next_float() for st in states]
+        return ops.sample_topp(logits, o.temperature, o.top_p, u.to(self.device, non_blocking=True), self.act)
 
     def finish(self, tokens: list[int], states: list[SequenceSampling]) -> None:
         for st, t in zip(states, tokens):
