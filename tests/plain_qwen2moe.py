@@ -321,19 +321,35 @@ def apply_rep_penalty(logits: np.ndarray, recent: list, window: int, penalty: fl
 
 
 def generate(model: PlainQwen2Moe, prompt, max_tokens: int, temperature: float = 0.0, top_p: float = 0.9,
-             seed: int = 42, rep_penalty: float = 1.0, rep_window: int = 32, stop_tokens=()) -> list:
-    """The reference's loop for one prompt (/root/reference/src/engine/tq_generate.c:386-630) without its
-    4-gram stop: penalty, sample; while fewer than max_tokens are out: stop on an end token, emit, run,
-    penalty, sample.  Every step recomputes the whole sequence."""
+             seed: int = 42, rep_penalty: float = 1.0, rep_window: int = 32, stop_tokens=(),
+             loop_detection: bool = False) -> list:
+    """The reference's loop for one prompt (/root/reference/src/engine/tq_generate.c:363-630): penalty, sample;
+    while fewer than max_tokens are out: stop on an end token, emit, run, penalty, sample, and (``loop_detection``)
+    stop when the 4-gram that the new token closes has been seen three times before (:611-629; the tokens
+    hashed are the prompt's last ``rep_window`` and every sampled one, :381-384, and the first sampled token,
+    drawn before the loop, is not looked at, :403-410).  Every step recomputes the whole sequence."""
     rng = PlainRng(seed)
     seq = list(prompt)
+    rep_window = min(rep_window, 128)                                     # :367
     recent = list(prompt[-rep_window:]) if rep_window else []
-    out = []
+    out, ring, n_hashed = [], [], 0
     while len(out) < max_tokens:
         logits = model.logits(seq)[-1].to(torch.float32).numpy().copy()
         apply_rep_penalty(logits, recent, rep_window, rep_penalty)
         nxt = sample_topp(logits, temperature, top_p, rng)
         recent.append(nxt)
+        if loop_detection and len(seq) > len(prompt) and len(recent) >= 4:
+            h = 0
+            for t in recent[-4:]:
+                h = (h * 31 + t) % (1 << 32)
+            matches = sum(1 for x in ring if x == h)
+            if len(ring) < 64:
+                ring.append(h)
+            else:
+                ring[n_hashed % 64] = h
+            n_hashed += 1
+            if matches >= 3:
+                break
         if nxt in stop_tokens:
             break
         out.append(nxt)

@@ -320,3 +320,70 @@ def test_generate_ends_a_sequence_when_the_cache_is_full(cpu_engine):
     assert r.finish_reason == "context" and len(r.tokens) == 4 and eng.cache.n_live == 0
     r = generate(eng, [[1] * 65], GenerationOptions(max_tokens=5))[0]
     assert r.finish_reason == "context" and r.tokens == []
+
+
+def test_a_refused_step_leaves_its_slots_usable(cpu_engine):
+    eng = cpu_engine("A", max_tokens=128, max_slots=2)
+    s = eng.open(2)
+    with pytest.raises(StepError, match="wanted place"):
+        eng.step(s, [[1, 2], [3]], [[0], [1]])
+    with pytest.raises(CacheFull):
+        eng.step(s, [[1] * 70, [2] * 70])              # three pages would be needed, two exist
+    assert all(g.pool.n_free == g.pool.n_pages for g in eng.cache.groups)
+    lg = eng.step(s, [[1, 2], [3]])                    # the same slots step as if nothing had happened
+    assert lg.shape == (2, 256) and eng.length(s[0]) == 2 and eng.length(s[1]) == 1
+    eng.close(s)
+
+
+def test_generate_survives_a_full_pool(cpu_engine):
+    """Two pages, two sequences of 60 tokens: at position 64 both need a page and none is free.  One ends with
+    reason "context" (with the token that found no room as its last), its page lets the other go on, and the
+    other's tokens are what it generates alone."""
+    eng = cpu_engine("A", max_tokens=128, max_slots=2)
+    greedy = dict(temperature=0.0, rep_penalty=1.0, loop_detection=False)
+    a, b = [3] * 60, [5, 9] * 30
+    alone = [generate(eng, [p], GenerationOptions(max_tokens=12, **greedy))[0] for p in (a, b)]
+    both = generate(eng, [a, b], GenerationOptions(max_tokens=12, **greedy))
+    assert [r.finish_reason for r in both] == ["context", "length"]
+    assert both[0].tokens == alone[0].tokens[:5] and both[1].tokens == alone[1].tokens and len(both[1].tokens) == 12
+    assert eng.cache.n_live == 0 and all(g.pool.n_free == g.pool.n_pages for g in eng.cache.groups)
+
+
+def test_prompts_that_do_not_fit_together_run_one_after_the_other(cpu_engine):
+    eng = cpu_engine("A", max_tokens=192, max_slots=2)
+    greedy = dict(temperature=0.0, rep_penalty=1.0, loop_detection=False)
+    a, b, c = [3] * 100, [5, 9] * 50, [7] * 300
+    alone = [generate(eng, [p], GenerationOptions(max_tokens=6, **greedy))[0] for p in (a, b)]
+    res = generate(eng, [a, b, c], GenerationOptions(max_tokens=6, max_batch=2, **greedy))
+    assert [r.tokens for r in res[:2]] == [r.tokens for r in alone] and all(len(r.tokens) == 6 for r in res[:2])
+    assert res[2].tokens == [] and res[2].finish_reason == "context"        # four pages are needed, three exist
+    assert eng.cache.n_live == 0
+
+
+def test_a_limit_of_positions_per_sequence_binds(cpu_engine):
+    eng = cpu_engine("A", max_tokens=1024, max_slots=2, max_positions=100)
+    assert eng.cache.max_positions == 100
+    r = generate(eng, [[1] * 90, [2] * 101], GenerationOptions(max_tokens=50, temperature=0.0, rep_penalty=1.0,
+                                                               loop_detection=False))
+    assert r[0].finish_reason == "context" and len(r[0].tokens) == 10
+    assert r[1].finish_reason == "context" and r[1].tokens == []
+
+
+def test_generate_with_the_default_options_matches_the_plain_loop(cpu_engine, model_dirs):
+    """Loop detection, repetition penalty and sampling as the options default to them; greedy decoding of a
+    tiny model soon repeats itself, so the 4-gram stop fires."""
+    from plain_qwen2moe import PlainQwen2Moe, generate as plain_generate
+    eng = cpu_engine("A")
+    plain = PlainQwen2Moe(model_dirs("A"))
+    reasons = []
+    for prompt, opts in (([3, 3, 3, 3, 3, 3], dict(temperature=0.0, rep_penalty=1.0)),
+                         ([1, 2, 3, 4] * 4, dict(temperature=0.0, rep_penalty=1.0)),
+                         ([9, 8, 7], dict())):
+        o = GenerationOptions(max_tokens=40, **opts)
+        assert o.loop_detection
+        got = generate(eng, [prompt], o)[0]
+        want = plain_generate(plain, prompt, max_tokens=40, loop_detection=True,
+                              **{**dict(temperature=0.7, top_p=0.9, rep_penalty=1.1), **opts})
+        assert got.tokens == want
+        reasons.append(got.finish_reason)
+    assert "loop" in reasons

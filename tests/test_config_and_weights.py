@@ -243,3 +243,38 @@ def test_random_weights_mode_writes_a_folder_that_the_seed_fixes(tmp_path):
         assert abs(float(n.mean()) - 1.0) < 0.01 and 0.01 < float(n.std()) < 0.03
     with SafetensorsFolder(write_random_model_dir(str(tmp_path / "d"), TINY_A, seed=0, dtype="bfloat16")) as fd:
         assert fd.read("model.norm.weight").dtype == torch.bfloat16 and bool((fd.read("model.norm.weight") == 1).all())
+
+
+def test_tensors_that_the_model_does_not_read_are_a_warning_not_an_error():
+    from turboquant_cpp_amd.weights.loader import UnexpectedTensors
+    model = model_from_config(TINY_A, "float32")
+    tensors = {n: torch.zeros(s) for n, (s, _r) in model.tensor_table().items()}
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
+    with pytest.warns(UnexpectedTensors, match="rotary_emb.inv_freq"):
+        load_bindings(model.bindings, TensorDict(tensors), "float32", "cpu")
+    assert model.blocks[0].mixer.qkv_weight.shape == (3 * 64, 64)
+
+
+def test_random_weights_are_a_function_of_seed_tensor_and_element(tmp_path):
+    """The generator's integer steps against splitmix64's published first outputs for state 0, pieces of a tensor
+    against the whole, and a model drawn in memory against the folder written for the same seed."""
+    from turboquant_cpp_amd.engine.model import random_model
+    from turboquant_cpp_amd.weights import random_init as ri
+    assert ri.splitmix64(0, 0) == 0xE220A8397B1DCDAF and ri.splitmix64(0, 1) == 0x6E789E6AA1B965F4
+    words = ri.splitmix64_mix(torch.tensor([ri._signed(ri._GAMMA), ri._signed(2 * ri._GAMMA)]))
+    assert [w % (1 << 64) for w in words.tolist()] == [0xE220A8397B1DCDAF, 0x6E789E6AA1B965F4]
+    key = ri.tensor_key(5, 3)
+    whole = ri.standard_normal(key, 0, 1000)
+    assert torch.equal(torch.cat([ri.standard_normal(key, 0, 333), ri.standard_normal(key, 333, 667)]), whole)
+    assert not torch.equal(ri.standard_normal(ri.tensor_key(5, 4), 0, 1000), whole)
+    z = ri.standard_normal(key, 0, 400000)
+    assert abs(float(z.mean())) < 0.01 and abs(float(z.var()) - 1) < 0.01 and abs(float((z ** 4).mean()) - 3) < 0.05
+    assert abs(float((z[:-1] * z[1:]).mean())) < 0.01
+    for dtype in ("float32", "bfloat16"):
+        d = write_random_model_dir(str(tmp_path / dtype), TINY_B, seed=1, std=0.02, norm_std=0.02, dtype=dtype)
+        drawn = random_model(TINY_B, 1, act=dtype, device="cpu", std=0.02, norm_std=0.02)
+        loaded = model_from_config(TINY_B, dtype)
+        with SafetensorsFolder(d) as f:
+            loaded.load(f, "cpu")
+        for a, b in zip(drawn.bindings, loaded.bindings):
+            assert torch.equal(getattr(a.owner, a.attr), getattr(b.owner, b.attr)), a.path

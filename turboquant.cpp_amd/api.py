@@ -18,8 +18,9 @@ class Model:
     """A loaded model ready to generate.
 
     ``path``: a folder with ``config.json`` and ``model.safetensors``.  ``dtype``: ``"bfloat16"`` (serving
-    kernels) or ``"float32"`` (everything in true 32-bit).  ``context_length``: positions per sequence the
-    cache is sized for (0: the model's ``max_position_embeddings``, at most 4096 as in the reference,
+    kernels) or ``"float32"`` (everything in true 32-bit).  ``context_length``: the most positions (prompt and
+    generated tokens) of a sequence, which the cache is sized for; a sequence that reaches it ends with reason
+    ``"context"`` (0: the model's ``max_position_embeddings``, at most 4096 as in the reference,
     /root/reference/src/engine/tq_model.c:2951).  ``max_batch``: sequences that generate together.
     """
 
@@ -56,7 +57,9 @@ class Model:
             stop_tokens=tuple(stop_tokens) if stop_tokens is not None else tuple(plan.stop_tokens), max_batch=max_batch)
         page = 64
         per_seq = -(-ctx // page) * page
-        self._engine = Engine(self._model, max_tokens=per_seq * max_batch, page_size=page, max_slots=max_batch)
+        # the cache holds ``max_batch`` sequences of ``context_length`` positions, and no sequence may grow beyond that
+        self._engine = Engine(self._model, max_tokens=per_seq * max_batch, page_size=page, max_slots=max_batch,
+                              max_positions=ctx)
 
     # ------------------------------------------------------------ generation
     def generate(self, prompts, **overrides) -> list[list[int]]:

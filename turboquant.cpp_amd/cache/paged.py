@@ -10,11 +10,13 @@ blocks on demand with create / append / seq_len / free calls and status checks
 * A *slot* stands for one live sequence: its length, its pages, its row of every state tensor.
   Slots are opened when a batch starts, closed when its sequence ends, and handed out again.
 * Keys and values live in *pages* of ``page_size`` positions.  Layers whose needs agree (kv heads,
-  head size, window) form a *group* with storage of its own: one pool of pages, each page holding the
-  rows of all the group's layers for ``page_size`` positions of one sequence: keys laid out
-  ``[layer][kv head][row][head_dim]``, values transposed, ``[layer][kv head][head_dim][row]`` (both as the
-  attention kernels' operands want them).  A group that keeps a window gives back the pages that have
-  fallen out of every later token's window, so its sequences hold pages for the window only.
+  width of a key row, width of a value row, window) form a *group* with storage of its own: one pool of
+  pages, each page holding the rows of all the group's layers for ``page_size`` positions of one sequence:
+  keys laid out ``[layer][kv head][row][head_dim]``, values transposed, ``[layer][kv head][value_dim][row]``
+  (both as the attention kernels' operands want them).  Keys and values have pools of their own, so their
+  rows may differ in width, and a group whose layers keep one row per position only (``value_dim`` 0) has no
+  value pool at all.  A group that keeps a window gives back the pages that have fallen out of every later
+  token's window, so its sequences hold pages for the window only.
 * The page table of a group, ``[slot][logical page] -> page`` (-1: none), lives on the device and is
   updated only when pages change hands; kernels find a token's rows through its slot.
 * A schedule entry that reads another entry's cache gets a view of that entry's storage and none
@@ -70,20 +72,24 @@ class PagePool:
 class GroupKey:
     num_kv_heads: int
     head_dim: int
+    value_dim: int
     window: int | None
 
 
 @dataclass
 class KVView:
     """What a mixer needs to reach its keys and values."""
-    k_pages: torch.Tensor | None      # flat pool of the group
-    v_pages: torch.Tensor | None
+    k_pages: torch.Tensor | None      # flat pool of the group's keys
+    v_pages: torch.Tensor | None      # flat pool of the group's values (None: the group keeps keys only)
     table: torch.Tensor | None        # int32 [slots, logical pages]
-    layer_offset: int                 # offset of the layer's rows inside a page, in elements
+    layer_offset: int                 # offset of the layer's key rows inside a key page, in elements
     page_size: int
-    page_stride: int                  # elements per page
+    page_stride: int                  # elements per key page
     window: int | None
     owns: bool                        # False: this run reads another run's keys and values and writes none
+    v_layer_offset: int = 0           # the same for values; equal to the keys' when both rows are as wide
+    v_page_stride: int = 0
+    value_dim: int = 0
 
 
 class CacheGroup:
@@ -93,23 +99,29 @@ class CacheGroup:
         self.entries = entries
         self.page_size = page_size
         self.layer_elems = key.num_kv_heads * page_size * key.head_dim
+        self.v_layer_elems = key.num_kv_heads * page_size * key.value_dim
         self.page_stride = len(entries) * self.layer_elems
+        self.v_page_stride = len(entries) * self.v_layer_elems
         self.pool = PagePool(n_pages)
         self.max_pages_per_seq = max_pages_per_seq
         self.host_table = np.full((max_slots, max_pages_per_seq), -1, dtype=np.int32)
         self.dirty: set[int] = set()
         self.device = device
+        self._staging = None
+        self.k_pages = self.v_pages = self.table = None     # without a device: bookkeeping only
         if device is not None:
             # zeroed once: rows beyond a sequence's length are read by tiled kernels (and masked), so they
             # must always hold finite numbers; pages that come back from a sequence do
             self.k_pages = torch.zeros(n_pages * self.page_stride, dtype=dtype, device=device)
-            self.v_pages = torch.zeros(n_pages * self.page_stride, dtype=dtype, device=device)
+            if self.v_page_stride:
+                self.v_pages = torch.zeros(n_pages * self.v_page_stride, dtype=dtype, device=device)
             self.table = torch.full((max_slots, max_pages_per_seq), -1, dtype=torch.int32, device=device)
-        else:   # bookkeeping only
-            self.k_pages = self.v_pages = self.table = None
 
     def offset_of(self, entry: int) -> int:
         return self.entries.index(entry) * self.layer_elems
+
+    def v_offset_of(self, entry: int) -> int:
+        return self.entries.index(entry) * self.v_layer_elems
 
     def first_needed_page(self, length: int) -> int:
         """Lowest logical page that a token at position >= length can still attend to."""
@@ -118,14 +130,33 @@ class CacheGroup:
         return max(0, length - self.key.window + 1) // self.page_size
 
     def sync(self) -> None:
-        """Sends the rows of the page table that changed to the device."""
+        """Sends the rows of the page table that changed to the device.  On a GPU they go through pinned memory
+        with copies that the host does not wait for (a copy from ordinary memory returns only when everything
+        issued before it has run, a decode step that was issued ahead included); the pinned rows are written again
+        only after an event behind the last copies has passed."""
         if not self.dirty or self.table is None:
             self.dirty.clear()
             return
         rows = sorted(self.dirty)
-        idx = torch.tensor(rows, dtype=torch.int64, device=self.device)
-        self.table[idx] = torch.from_numpy(self.host_table[rows]).to(self.device)
         self.dirty.clear()
+        n = len(rows)
+        if torch.device(self.device).type != "cuda":
+            self.table[torch.tensor(rows, dtype=torch.int64)] = torch.from_numpy(self.host_table[rows])
+            return
+        st = self._staging
+        if st is None or st["rows"].shape[0] < n:
+            cap = max(n, 8)
+            st = self._staging = {"rows": torch.empty((cap, self.max_pages_per_seq), dtype=torch.int32).pin_memory(),
+                                  "idx": torch.empty((cap,), dtype=torch.int64).pin_memory(),
+                                  "copied": torch.cuda.Event()}
+        else:
+            st["copied"].synchronize()
+        st["rows"].numpy()[:n] = self.host_table[rows]
+        st["idx"].numpy()[:n] = rows
+        dev_rows = st["rows"][:n].to(self.device, non_blocking=True)
+        dev_idx = st["idx"][:n].to(self.device, non_blocking=True)
+        st["copied"].record()
+        self.table.index_copy_(0, dev_idx, dev_rows)
 
 
 @dataclass
@@ -151,7 +182,7 @@ class PagedCache:
         self.n_pages = -(-max_tokens // page_size)
         self.max_slots = min(self.n_pages, 4096) if max_slots is None else max_slots
         per_seq = self.n_pages if max_positions is None else min(self.n_pages, -(-max_positions // page_size))
-        self.max_positions = per_seq * page_size
+        self.max_positions = per_seq * page_size if max_positions is None else min(per_seq * page_size, max_positions)
         self.dtype, self.device = dtype, device
         self.slots = [Slot(i) for i in range(self.max_slots)]
         self._free_slots = list(range(self.max_slots - 1, -1, -1))
@@ -161,24 +192,29 @@ class PagedCache:
         self._needs = list(needs)
         for e, (cache_need, _state, cache_of) in enumerate(self._needs):
             if cache_need is not None and cache_of is None:
-                by_key.setdefault(GroupKey(cache_need.num_kv_heads, cache_need.head_dim, cache_need.window), []).append(e)
+                by_key.setdefault(GroupKey(cache_need.num_kv_heads, cache_need.head_dim, cache_need.value_width,
+                                           cache_need.window), []).append(e)
         self.groups: list[CacheGroup] = [
             CacheGroup(key, entries, self.n_pages, page_size, self.max_slots, per_seq, dtype, device)
             for key, entries in by_key.items()]
+        self._v_offset: dict[int, int] = {}
         for g in self.groups:
             for e in g.entries:
                 self._entry_group[e] = (g, g.offset_of(e), True)
+                self._v_offset[e] = g.v_offset_of(e)
         for e, (cache_need, _state, cache_of) in enumerate(self._needs):
             if cache_need is not None and cache_of is not None:
                 if cache_of not in self._entry_group or not self._entry_group[cache_of][2]:
                     raise CacheError(f"schedule entry {e} reads the cache of entry {cache_of}, which keeps none of its own")
                 g, off, _ = self._entry_group[cache_of]
                 src = self._needs[cache_of][0]
-                if (src.num_kv_heads, src.head_dim) != (cache_need.num_kv_heads, cache_need.head_dim):
+                if (src.num_kv_heads, src.head_dim, src.value_width) != \
+                        (cache_need.num_kv_heads, cache_need.head_dim, cache_need.value_width):
                     raise CacheError(f"schedule entry {e} reads the cache of entry {cache_of} but their head counts or sizes differ")
                 if src.window is not None and (cache_need.window is None or cache_need.window > src.window):
                     raise CacheError(f"schedule entry {e} looks further back than entry {cache_of}, whose cache it reads, keeps")
                 self._entry_group[e] = (g, off, False)
+                self._v_offset[e] = self._v_offset[cache_of]
 
         self.states: dict[int, torch.Tensor] = {}
         for e, (_cache, state_need, _of) in enumerate(self._needs):
@@ -246,7 +282,20 @@ class PagedCache:
         s.reserved = n_new
         return s.length
 
-    def _undo_reserve(self, slot: int, failed: CacheGroup) -> None:
+    def needs_page(self, slot: int, n_new: int = 1) -> bool:
+        """Whether ``n_new`` more positions would take a page that the sequence does not hold yet."""
+        s = self._live(slot)
+        first_page, last_page = s.length // self.page_size, (s.length + n_new - 1) // self.page_size
+        if last_page >= self.groups[0].max_pages_per_seq if self.groups else False:
+            return True
+        return any((g.host_table[slot][first_page:last_page + 1] < 0).any() for g in self.groups)
+
+    @property
+    def n_free_slots(self) -> int:
+        return len(self._free_slots)
+
+    def _undo_reserve(self, slot: int, failed: CacheGroup | None) -> None:
+        """Gives back the pages beyond the sequence's length, in the groups before ``failed`` (None: in all)."""
         s = self.slots[slot]
         keep_upto = (s.length - 1) // self.page_size if s.length else -1
         for g in self.groups:
@@ -258,6 +307,12 @@ class PagedCache:
                 g.pool.give_back(row[extra].tolist())
                 row[extra] = -1
                 g.dirty.add(slot)
+
+    def cancel(self, slot: int) -> None:
+        """The step that reserved positions did not run: they do not count, and pages taken for them go back."""
+        s = self._live(slot)
+        s.reserved = 0
+        self._undo_reserve(slot, None)
 
     def commit(self, slot: int) -> None:
         """The step that reserved positions has run: they now count, and pages that no later token's
@@ -284,7 +339,8 @@ class PagedCache:
         if entry not in self._entry_group:
             raise CacheError(f"schedule entry {entry} keeps no keys and values")
         g, off, owns = self._entry_group[entry]
-        return KVView(g.k_pages, g.v_pages, g.table, off, g.page_size, g.page_stride, self._needs[entry][0].window, owns)
+        return KVView(g.k_pages, g.v_pages, g.table, off, g.page_size, g.page_stride, self._needs[entry][0].window, owns,
+                      self._v_offset[entry], g.v_page_stride, g.key.value_dim)
 
     def state(self, entry: int) -> torch.Tensor:
         if entry not in self.states:
@@ -298,6 +354,7 @@ class PagedCache:
     def bytes(self) -> int:
         n = 0
         for g in self.groups:
-            if g.k_pages is not None:
-                n += 2 * g.k_pages.numel() * g.k_pages.element_size()
+            for pages in (g.k_pages, g.v_pages):
+                if pages is not None:
+                    n += pages.numel() * pages.element_size()
         return n

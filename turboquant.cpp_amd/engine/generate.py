@@ -6,11 +6,15 @@ emit, run the token, apply the repetition penalty, sample, and stop when the sam
 times (:611-629).  Here the same decisions are taken per sequence of a batch: all prompts of a batch run
 in one step, then every live sequence decodes one token per step; a sequence that ends gives its slot
 and pages back at once and the others go on; when more requests wait than a batch holds, batch follows
-batch.  The decisions are kept apart from the device work (``Decision`` and ``SequenceTrack``) so that
-they are tested without one.
+batch.  Where the reference shifts a full context (:456-514), a sequence here ends with reason ``"context"``:
+when it reaches the positions a sequence may hold, and also when the cache's pages run out while several
+sequences grow (the longest of those that need a page ends, its pages let the others go on); a prompt that
+finds no room beside the others of its batch waits for the next batch.  The decisions are kept apart from
+the device work (``SequenceTrack``) so that they are tested without one.
 """
 from __future__ import annotations
 
+from collections import deque
 from dataclasses import dataclass, field
 from typing import Callable, Sequence
 
@@ -75,9 +79,17 @@ class SequenceTrack:
     options: GenerationOptions
     max_positions: int
     out: list[int] = field(default_factory=list)
-    history: list[int] = field(default_factory=list)    # prompt tail and sampled tokens, for the loop detector
+    # the last tokens of the prompt (as many as the repetition window, tq_generate.c:381-384) and every sampled
+    # token: what the loop detector hashes its 4-grams from
+    history: list[int] = field(default_factory=list)
     detector: LoopDetector = field(default_factory=LoopDetector)
     finish_reason: str | None = None
+    n_sampled: int = 0
+
+    @classmethod
+    def start(cls, request: int, prompt: Sequence[int], options: GenerationOptions, max_positions: int) -> "SequenceTrack":
+        window = max(0, min(options.rep_window, 128))
+        return cls(request, len(prompt), options, max_positions, history=list(prompt[-window:]) if window else [])
 
     def room_after_next(self) -> bool:
         """Whether the sequence can go on after its next token, as far as that does not depend on the token:
@@ -89,7 +101,14 @@ class SequenceTrack:
         False if the sequence has ended (``finish_reason`` says why)."""
         o = self.options
         self.history.append(token)
-        looped = o.loop_detection and self.detector.push(self.history)
+        del self.history[:-128]
+        self.n_sampled += 1
+        # the reference looks for a loop right after it has sampled a token in its loop, not after the first
+        # token, which it samples before the loop (tq_generate.c:403-410, :603-629); the token that closes a loop
+        # is not emitted
+        if o.loop_detection and self.n_sampled > 1 and self.detector.push(self.history):
+            self.finish_reason = "loop"
+            return False
         if token in o.stop_tokens:
             self.finish_reason = "stop"          # the end token is not emitted
             return False
@@ -98,9 +117,6 @@ class SequenceTrack:
             o.on_token(self.request, token)
         if len(self.out) >= o.max_tokens:
             self.finish_reason = "length"
-            return False
-        if looped:
-            self.finish_reason = "loop"
             return False
         if self.prompt_len + len(self.out) >= self.max_positions:
             self.finish_reason = "context"       # no room for another position; the reference would shift (:456-514)
@@ -120,27 +136,56 @@ def generate(engine, prompts: Sequence[Sequence[int]], options: GenerationOption
     o = options or GenerationOptions()
     if any(len(p) == 0 for p in prompts):
         raise ValueError("every prompt needs at least one token")
+    if o.max_batch < 1:
+        raise ValueError("max_batch must be at least 1")
     if o.max_tokens < 1:
         return [GenerationResult([], "length") for _ in prompts]
     sampler = Sampler(o.sampling(), engine.model.act, engine.device)
     results: list[GenerationResult | None] = [None] * len(prompts)
     max_pos = engine.cache.max_positions
-    for batch in plan_batches(len(prompts), o.max_batch):
-        too_long = [r for r in batch if len(prompts[r]) > max_pos]
-        for r in too_long:
-            results[r] = GenerationResult([], "context")
-        batch = [r for r in batch if r not in too_long]
+    waiting = deque(range(len(prompts)))
+
+    def end(r, tracks, slot_of, reason=None):
+        if reason is not None:
+            tracks[r].finish_reason = reason
+        engine.close([slot_of.pop(r)])
+        results[r] = GenerationResult(tracks[r].out, tracks[r].finish_reason)
+
+    while waiting:
+        batch = []
+        room = min(o.max_batch, engine.cache.n_free_slots)
+        if room < 1:
+            raise CacheFull("no slot is free to start a batch with")
+        while waiting and len(batch) < room:
+            r = waiting.popleft()
+            if len(prompts[r]) > max_pos:
+                results[r] = GenerationResult([], "context")
+            else:
+                batch.append(r)
         if not batch:
             continue
         slots = engine.open(len(batch))
-        tracks = {r: SequenceTrack(r, len(prompts[r]), o, max_pos) for r in batch}
+        tracks = {r: SequenceTrack.start(r, prompts[r], o, max_pos) for r in batch}
         samp = {r: sampler.new_sequence(r, list(prompts[r])) for r in batch}
         slot_of = dict(zip(batch, slots))
         live = list(batch)
         fetch = TokenFetch(engine.device, len(batch))
         try:
-            logits = engine.step([slot_of[r] for r in live], [list(prompts[r]) for r in live])
-            while True:
+            logits = None
+            while live:
+                try:
+                    logits = engine.step([slot_of[r] for r in live], [list(prompts[r]) for r in live])
+                    break
+                except CacheFull:
+                    # the prompts of this batch do not fit into the cache together: the last one waits for the
+                    # next batch; a prompt that does not even fit alone has no room at all
+                    r = live.pop()
+                    if live:
+                        engine.close([slot_of.pop(r)])
+                        waiting.appendleft(r)
+                    else:
+                        end(r, tracks, slot_of, "context")
+            while live:
                 states = [samp[r] for r in live]
                 ids = sampler.launch(logits, states)
                 fetch.start(ids)
@@ -164,13 +209,20 @@ def generate(engine, prompts: Sequence[Sequence[int]], options: GenerationOption
                     if tracks[r].accept(t):
                         going.append(i)
                     else:
-                        engine.close([slot_of.pop(r)])
-                        results[r] = GenerationResult(tracks[r].out, tracks[r].finish_reason)
-                if not going:
-                    break
-                if not ahead:
-                    logits = engine.step([slot_of[live[i]] for i in going], [[tokens[i]] for i in going])
-                else:
+                        end(r, tracks, slot_of)
+                if going and not ahead:
+                    while going:
+                        try:
+                            logits = engine.step([slot_of[live[i]] for i in going], [[tokens[i]] for i in going])
+                            break
+                        except CacheFull:
+                            # the pages have run out: of the sequences that need one, the longest ends here, and
+                            # what it held lets the others go on
+                            needy = [i for i in going if engine.cache.needs_page(slot_of[live[i]], 1)]
+                            i = max(needy or going, key=lambda i: engine.length(slot_of[live[i]]))
+                            going.remove(i)
+                            end(live[i], tracks, slot_of, "context")
+                elif going:
                     rows = [ahead.index(i) for i in going]       # a sequence that goes on was run ahead
                     logits = next_logits if rows == list(range(len(ahead))) else \
                         next_logits[torch.tensor(rows, dtype=torch.int64, device=next_logits.device)]

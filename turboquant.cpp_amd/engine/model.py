@@ -101,9 +101,12 @@ class CausalLM:
             needs.append((block.cache_need(), block.state_need(), e.cache_of))
         return needs
 
-    def new_cache(self, max_tokens: int, page_size: int = 64, max_slots: int | None = None) -> PagedCache:
+    def new_cache(self, max_tokens: int, page_size: int = 64, max_slots: int | None = None,
+                  max_positions: int | None = None) -> PagedCache:
+        """``max_positions``: the most positions a sequence may reach, if that is to be fewer than the model allows."""
+        limit = self.plan.max_positions if max_positions is None else min(max_positions, self.plan.max_positions)
         return PagedCache(self.cache_needs(), max_tokens, self.act_dtype, self.device, page_size=page_size,
-                          max_slots=max_slots, max_positions=self.plan.max_positions)
+                          max_slots=max_slots, max_positions=limit)
 
     # ------------------------------------------------------------ forward
     def forward(self, ctx: StepContext) -> torch.Tensor:
@@ -135,12 +138,13 @@ def load_model(model_dir: str, act: str = "bfloat16", device="cuda:0") -> Causal
 
 
 def random_model(config_json: dict, seed: int, act: str = "bfloat16", device="cuda:0", std: float = 0.02,
-                 norm_std: float = 0.0, on_device: bool = True) -> CausalLM:
-    """A model with random weights made in memory (the values differ from those of a written folder when
-    they are drawn on the device)."""
+                 norm_std: float = 0.0, on_device: bool = True, dtype: str | None = None) -> CausalLM:
+    """A model with random weights drawn in memory, tensor by tensor, where the model lives: the values of the
+    folder that ``write_random_model_dir`` writes for the same configuration, seed and ``dtype`` (the type the
+    folder's tensors would have; default: the activation type)."""
     model = model_from_config(config_json, act)
     table = model.tensor_table()
-    dtype = torch.float32 if model.act == "float32" else torch.bfloat16
+    dtype = {"float32": torch.float32, "bfloat16": torch.bfloat16}[ACT_NAMES[dtype] if dtype else model.act]
     gen_device = device if on_device else "cpu"
 
     class _Lazy:

@@ -27,9 +27,10 @@ class Engine:
     each sequence rounded up to whole pages of ``page_size``."""
 
     def __init__(self, model: CausalLM, max_tokens: int, page_size: int = 64, max_slots: int | None = None,
-                 use_graphs: bool = True):
+                 use_graphs: bool = True, max_positions: int | None = None):
+        """``max_positions``: the most positions one sequence may reach (default and upper bound: the model's)."""
         self.model = model
-        self.cache = model.new_cache(max_tokens, page_size=page_size, max_slots=max_slots)
+        self.cache = model.new_cache(max_tokens, page_size=page_size, max_slots=max_slots, max_positions=max_positions)
         self.device = model.device
         self.vocab_size = model.plan.vocab_size
         # decode steps are replayed as HIP graphs where a GPU runs them
@@ -70,27 +71,33 @@ class Engine:
             raise StepError("a slot appears twice in one step")
         if wants is None:
             wants = [[len(t) - 1] for t in token_lists]
+        if len(wants) != len(slots):
+            raise StepError("a step needs as many lists of wanted places as slots")
         V = self.vocab_size
-        for i, toks in enumerate(token_lists):
+        for i, (toks, want) in enumerate(zip(token_lists, wants)):
             if len(toks) == 0:
                 raise StepError(f"sequence {i} of the step brings no token")
             bad = [t for t in toks if not 0 <= t < V]
             if bad:
                 raise StepError(f"sequence {i} brings token {bad[0]}, outside the vocabulary of {V}")
+            bad = [w for w in want if not 0 <= w < len(toks)]
+            if bad:
+                raise StepError(f"wanted place {bad[0]} is outside the {len(toks)} tokens that sequence {i} brings")
         starts = self._reserve(slots, [len(t) for t in token_lists])
-        logits = None
-        if self.graphs is not None and all(len(t) == 1 for t in token_lists):
-            for i, w in enumerate(wants):
-                if any(x != 0 for x in w):
-                    raise ValueError(f"wanted place {w} is outside the 1 token that sequence {i} brings")
-            all_rows = self.graphs.run(slots, starts, [t[0] for t in token_lists])
-            if all_rows is not None:       # the graph gives every row; hand out a copy of the wanted ones
-                rows = [i for i, w in enumerate(wants) for _ in w]
-                logits = all_rows.clone() if rows == list(range(len(slots))) else \
-                    all_rows[torch.tensor(rows, dtype=torch.int64, device=self.device)] if rows else \
-                    torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
-        if logits is None:
-            logits = self._eager(pack_step(slots, starts, token_lists, wants, self.device))
+        try:
+            logits = None
+            if self.graphs is not None and all(len(t) == 1 for t in token_lists):
+                all_rows = self.graphs.run(slots, starts, [t[0] for t in token_lists])
+                if all_rows is not None:       # the graph gives every row; hand out a copy of the wanted ones
+                    rows = [i for i, w in enumerate(wants) for _ in w]
+                    logits = all_rows.clone() if rows == list(range(len(slots))) else \
+                        all_rows[torch.tensor(rows, dtype=torch.int64, device=self.device)] if rows else \
+                        torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
+            if logits is None:
+                logits = self._eager(pack_step(slots, starts, token_lists, wants, self.device))
+        except BaseException:
+            self._unreserve(slots)
+            raise
         for slot in slots:
             self.cache.commit(slot)
         return logits
@@ -107,11 +114,15 @@ class Engine:
                 (self.device is not None and tokens.device != torch.device(self.device)):
             raise StepError(f"tokens must be int32 [{len(slots)}] on the model's device")
         starts = self._reserve(slots, [1] * len(slots))
-        logits = self.graphs.run(slots, starts, tokens) if self.graphs is not None else None
-        if logits is None:
-            batch = pack_step(slots, starts, [[0]] * len(slots), [[0]] * len(slots), self.device)
-            batch.tokens.copy_(tokens)
-            logits = self._eager(batch)
+        try:
+            logits = self.graphs.run(slots, starts, tokens) if self.graphs is not None else None
+            if logits is None:
+                batch = pack_step(slots, starts, [[0]] * len(slots), [[0]] * len(slots), self.device)
+                batch.tokens.copy_(tokens)
+                logits = self._eager(batch)
+        except BaseException:
+            self._unreserve(slots)
+            raise
         for slot in slots:
             self.cache.commit(slot)
         return logits
@@ -124,11 +135,16 @@ class Engine:
                 starts.append(self.cache.reserve(slot, n))
                 reserved.append(slot)
         except CacheError:
-            for slot in reserved:
-                self.cache.slots[slot].reserved = 0
+            self._unreserve(reserved)
             raise
         self.cache.sync()
         return starts
+
+    def _unreserve(self, slots) -> None:
+        """A step that did not run: its positions do not count and the pages taken for them go back."""
+        for slot in slots:
+            self.cache.cancel(slot)
+        self.cache.sync()
 
     def _eager(self, batch) -> torch.Tensor:
         # a second stream for what does not depend on the main line (the parts decide what they put there)

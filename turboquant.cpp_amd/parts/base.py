@@ -43,10 +43,17 @@ class ParamSpec:
 
 @dataclass(frozen=True)
 class CacheNeed:
-    """Keys and values per position: ``window`` None keeps all positions, else the last ``window``."""
+    """Keys and values per position: ``window`` None keeps all positions, else the last ``window``.
+    ``head_dim`` is the width of a key row; ``value_dim`` that of a value row (None: the same; 0: no values are
+    kept, one row per position and kv head only)."""
     num_kv_heads: int
     head_dim: int
     window: int | None = None
+    value_dim: int | None = None
+
+    @property
+    def value_width(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
 
 
 @dataclass(frozen=True)

@@ -3,11 +3,14 @@
 In the manner of the reference's loader (/root/reference/src/engine/tq_model.c:847-1666): tensors are looked up
 by name (:324-360), bfloat16 stays bfloat16 and float32 stays float32 (:367-412, :440-451).  Unlike it, a
 tensor that is not there is never a silent NULL (tq_model.c:418-423): everything is checked before
-anything is copied, and one error lists all missing tensors, all unexpected ones and all wrong shapes.
+anything is copied, and one error lists all missing tensors, all wrong shapes and, beside them, the tensors
+that the model does not read.  A checkpoint whose only difference is such extra tensors (a stray buffer) loads,
+with a warning that names them.
 Experts stored one tensor each are stacked, and q, k, v are joined, as the plan's sources say.
 """
 from __future__ import annotations
 
+import warnings
 from dataclasses import dataclass
 
 import torch
@@ -32,6 +35,10 @@ class WeightError(ValueError):
         for o in self.other:
             lines.append("  " + o)
         super().__init__("\n".join(lines))
+
+
+class UnexpectedTensors(UserWarning):
+    """The checkpoint holds tensors that the model does not read."""
 
 
 @dataclass
@@ -78,8 +85,12 @@ def check(bindings: list[Binding], available: dict[str, tuple[tuple[int, ...], t
     wrong = [(n, available[n][0], want[n][0]) for n in want if n in available and tuple(available[n][0]) != want[n][0]]
     other = [f"tensor {n} has type {available[n][1]}, which no kernel takes" for n in want
              if n in available and available[n][1] not in (torch.float32, torch.bfloat16, torch.float16, torch.int32, torch.int64)]
-    if missing or unexpected or wrong or other:
+    if missing or wrong or other:
         raise WeightError(missing, unexpected, wrong, other)
+    if unexpected:
+        warnings.warn(f"checkpoint holds {len(unexpected)} tensors that the model does not read: "
+                      + ", ".join(unexpected[:20]) + (" ..." if len(unexpected) > 20 else ""), UnexpectedTensors,
+                      stacklevel=3)
 
 
 def stored_dtype(dtypes: list[torch.dtype], act: str) -> torch.dtype:
