@@ -22,7 +22,7 @@ SOURCES = {
     "float32": COMMON_SOURCES,
     "bfloat16": COMMON_SOURCES + ["gemm_mfma.hip", "attention_mfma.hip", "probe.hip"],
 }
-HEADERS = ["common.h"]
+HEADERS = ["common.h", "no_alloc.h"]
 DEFINES = {"float32": "-DTQ_ACT_F32", "bfloat16": "-DTQ_ACT_BF16"}
 FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-fno-gpu-rdc",
          # keep the compiler from forming packed 32-bit float instructions

@@ -1,6 +1,8 @@
 // Choice of the next token from rows of logits: greedy, temperature with top-p, repetition penalty.
 // Nothing is sorted.
 #include "common.h"
+#include "no_alloc.h"
+#include <mutex>
 
 #define ST 1024   // threads per row
 
@@ -484,14 +486,8 @@ TQ_API int64_t tq_sample_topp_scratch(int R) {
   return (int64_t)R * 2 * (STATE_FLOATS + SC * PW);
 }
 
-// probs: scratch of R * V floats; scratch: tq_sample_topp_scratch(R) floats.  temperature > 0 and top_p > 0 (the
-// caller takes the greedy path otherwise).  out[r] is written for every row unless a probability is NaN; it is
-// set to 0 first.
-TQ_API int tq_sample_topp(const float* logits, int R, int V, float temperature, float top_p, const float* uniforms,
-                          float* probs, float* scratch, int* out, hipStream_t st) {
-  if (R <= 0) return 0;
-  if (!(temperature > 0.f) || !(top_p > 0.f) || !scratch) return TQ_ERR_BAD_ARG;
-  if (R > 65535) return TQ_ERR_UNSUPPORTED;
+static int launch_sample_topp(const float* logits, int R, int V, float temperature, float top_p, const float* uniforms,
+                              float* probs, float* scratch, int* out, hipStream_t st) {
   RowState* state[2] = {(RowState*)scratch, (RowState*)(scratch + (size_t)R * STATE_FLOATS)};
   float* part[2] = {scratch + (size_t)R * 2 * STATE_FLOATS, nullptr};
   part[1] = part[0] + (size_t)R * SC * PW;
@@ -503,4 +499,66 @@ TQ_API int tq_sample_topp(const float* logits, int R, int V, float temperature, 
                        state[(stage + 1) % 2], state[stage % 2], part[(stage + 1) % 2], part[stage % 2], out);
   TQ_LAUNCH_CHECK();
   return 0;
+}
+
+// probs: scratch of R * V floats; scratch: tq_sample_topp_scratch(R) floats.  temperature > 0 and top_p > 0 (the
+// caller takes the greedy path otherwise).  out[r] is written for every row unless a probability is NaN; it is
+// set to 0 first.
+TQ_API int tq_sample_topp(const float* logits, int R, int V, float temperature, float top_p, const float* uniforms,
+                          float* probs, float* scratch, int* out, hipStream_t st) {
+  if (R <= 0) return 0;
+  if (!(temperature > 0.f) || !(top_p > 0.f) || !scratch) return TQ_ERR_BAD_ARG;
+  if (R > 65535) return TQ_ERR_UNSUPPORTED;
+  return launch_sample_topp(logits, R, V, temperature, top_p, uniforms, probs, scratch, out, st);
+}
+
+// ---------------------------------------------------------------- the same choice without any allocation
+// The probabilities and the passes' partial results live in an array that is part of the library's image on every
+// GPU, TQ_STATIC_SAMPLE_BYTES of it (see no_alloc.h).  The array's name is only the host's handle for it: the
+// address that kernels can use is looked up once per device and kept.  Nothing in the array has to start at zero:
+// the first pass writes every field that a later pass reads.
+#define STATIC_SCRATCH_FLOATS (TQ_STATIC_SAMPLE_MAX_ROWS * 2 * (STATE_FLOATS + SC * PW))
+static __device__ __align__(256) float scratch[TQ_STATIC_SAMPLE_MAX_PROBS + STATIC_SCRATCH_FLOATS];
+static_assert(sizeof(scratch) <= TQ_STATIC_SAMPLE_BYTES, "the array has outgrown the size that no_alloc.h states");
+
+#define STATIC_MAX_DEVICES 64
+static std::mutex static_lock;
+static float* static_ptr[STATIC_MAX_DEVICES];      // device address of `scratch` on each GPU, once looked up
+
+TQ_API int tq_sample_topp_static_init(void) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= STATIC_MAX_DEVICES) return TQ_ERR_UNSUPPORTED;
+  std::lock_guard<std::mutex> hold(static_lock);
+  if (static_ptr[dev]) return 0;
+  float* ptr = nullptr;
+  e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+  if (e != hipSuccess) return (int)e;
+  if (!ptr) return TQ_ERR_BAD_ARG;
+  static_ptr[dev] = ptr;
+  return 0;
+}
+
+TQ_API int tq_sample_topp_static(const float* logits, int R, int V, float temperature, float top_p,
+                                 const float* uniforms, int* out, hipStream_t st) {
+  if (R <= 0) return 0;
+  if (!(temperature > 0.f) || !(top_p > 0.f) || V <= 0) return TQ_ERR_BAD_ARG;
+  if (R > TQ_STATIC_SAMPLE_MAX_ROWS || (int64_t)R * V > TQ_STATIC_SAMPLE_MAX_PROBS) return TQ_ERR_UNSUPPORTED;
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= STATIC_MAX_DEVICES) return TQ_ERR_UNSUPPORTED;
+  float* base;
+  {
+    std::lock_guard<std::mutex> hold(static_lock);
+    base = static_ptr[dev];
+  }
+  if (!base) {
+    const int rc = tq_sample_topp_static_init();
+    if (rc != 0) return rc;
+    std::lock_guard<std::mutex> hold(static_lock);
+    base = static_ptr[dev];
+  }
+  return launch_sample_topp(logits, R, V, temperature, top_p, uniforms, base, base + TQ_STATIC_SAMPLE_MAX_PROBS, out, st);
 }
