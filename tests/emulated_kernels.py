@@ -91,7 +91,9 @@ def attention(q, k_pages, v_pages, layer_offset, positions, slot_of_token, block
 
 
 def gemm(a, w, act, bias=None, w2=None, out_act=False, a_rows=None, tile_group=None, n_tiles=None, tile_rows=None,
-         gather=True, partial_sums=False):
+         gather=True, partial_sums=False, activation="silu"):
+    gate = {"silu": torch.nn.functional.silu, "relu2": lambda v: torch.relu(v) ** 2,
+            "gelu_tanh": lambda v: torch.nn.functional.gelu(v, approximate="tanh")}[activation]
     if partial_sums:
         return gemm(a, w, act, bias=bias).unsqueeze(0)
     af = a.float()
@@ -101,7 +103,7 @@ def gemm(a, w, act, bias=None, w2=None, out_act=False, a_rows=None, tile_group=N
         if bias is not None:
             y = y + bias.float()
         if w2 is not None:
-            y = torch.nn.functional.silu(y) * (src @ w2.float().T)
+            y = gate(y) * (src @ w2.float().T)
     else:
         P, N = a_rows.numel(), w.shape[1]
         y = torch.full((P, N), float("nan"))
@@ -114,7 +116,7 @@ def gemm(a, w, act, bias=None, w2=None, out_act=False, a_rows=None, tile_group=N
                 row = af[r] if gather else af[m]
                 v = w[g].float() @ row
                 if w2 is not None:
-                    v = torch.nn.functional.silu(v) * (w2[g].float() @ row)
+                    v = gate(v) * (w2[g].float() @ row)
                 y[m] = v
     return y.to(ACT[act]) if out_act else y
 

@@ -102,22 +102,28 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: int | N
     return out
 
 
-def route(x: torch.Tensor, router: torch.Tensor, top_k: int, renormalize: bool):
+def route(x: torch.Tensor, router: torch.Tensor, top_k: int, renormalize: bool, other_side=None):
     """x [H].  logits = router x; top-k by k passes of a scan with >=, so among equals the highest index
     wins and ids come out by descending logit (/root/reference/src/engine/tq_moe.c:611-645).
     renormalize true: softmax over the selected logits (tq_moe.c:648-678).
     renormalize false (no formula in the reference, which always renormalises): softmax over all experts,
-    the selected probabilities kept as they are."""
+    the selected probabilities kept as they are.
+    ``other_side`` = (i, j): the choice that an arithmetic with other rounding makes when the expert of rank i (one
+    of the chosen, 0 the best) and the expert of rank j (one of those left out) nearly tie: the latter takes the
+    former's place."""
     logits = matvec_rows(router, x)
     E = logits.shape[0]
     used, ids = [False] * E, []
-    for _ in range(top_k):
+    for _ in range(top_k if other_side is None else other_side[1] + 1):
         best, best_val = -1, -math.inf
         for e in range(E):
             if not used[e] and logits[e].item() >= best_val:
                 best_val, best = logits[e].item(), e
         used[best] = True
         ids.append(best)
+    if other_side is not None:
+        i, j = other_side
+        ids = ids[:i] + [ids[j]] + ids[i + 1:top_k]
     sel = logits[ids]
     if renormalize:
         w = softmax(sel)
@@ -142,13 +148,26 @@ def swiglu_mlp(x: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torc
     return matvec_rows(down, silu(matvec_rows(gate, x)) * matvec_rows(up, x))
 
 
-def moe(x: torch.Tensor, w: dict, top_k: int, renormalize: bool, margins: list | None = None) -> torch.Tensor:
+def near_swaps(x: torch.Tensor, router: torch.Tensor, top_k: int, reach: int = 3) -> list:
+    """(gap, i, j) for every chosen rank i and every rank j among the ``reach`` best left out, the gap being the
+    difference of their logits in units of the logits' spread, smallest first."""
+    logits = matvec_rows(router, x)
+    top = torch.sort(logits, descending=True).values
+    spread = float(logits.std()) + 1e-30
+    out = [(float(top[i] - top[j]) / spread, i, j) for i in range(top_k) for j in range(top_k, min(top_k + reach, len(top)))]
+    return sorted(out)
+
+
+def moe(x: torch.Tensor, w: dict, top_k: int, renormalize: bool, margins: list | None = None,
+        other_side=None, swaps: list | None = None) -> torch.Tensor:
     """x [T, H].  out = sum over the selected experts, in the order selected, of weight * expert(x)
     (/root/reference/src/engine/tq_moe.c:720,864-999); then + sigmoid(x . shared_scale) * shared(x)
     (tq_moe.c:1005-1058)."""
     out = torch.zeros_like(x)
     for t in range(x.shape[0]):
-        ids, wts = route(x[t], w["router"], top_k, renormalize)
+        ids, wts = route(x[t], w["router"], top_k, renormalize, other_side=(other_side or {}).get(t))
+        if swaps is not None:
+            swaps.append(near_swaps(x[t], w["router"], top_k))
         if margins is not None:
             margins.append(route_margin(x[t], w["router"], top_k))
         acc = torch.zeros_like(x[t])
@@ -184,6 +203,8 @@ class PlainQwen2Moe:
         self.hd = c.get("head_dim") or self.H // self.nh
         self.eps, self.theta = c["rms_norm_eps"], c["rope_theta"]
         self.margins: dict[int, list] = {}      # per sparse layer, the routing margin of every token of the last call
+        self.swaps: dict[int, list] = {}        # per sparse layer and token, the nearest exchanges of two experts
+        self.other_side: dict = {}              # (layer, position) -> (i, j): near-ties that calls decide the other way
 
     def layer_is_sparse(self, l: int) -> bool:
         """No rule in the reference (it looks for a router tensor, /root/reference/src/engine/tq_model.c:3440-3444);
@@ -225,8 +246,9 @@ class PlainQwen2Moe:
         if c["shared_expert_intermediate_size"] > 0:
             w["shared"] = {n: t[f"{p}shared_expert.{n}_proj.weight"] for n in ("gate", "up", "down")}
             w["shared_scale"] = t[p + "shared_expert_gate.weight"]
-        self.margins[l] = []
-        return moe(xb, w, c["num_experts_per_tok"], c.get("norm_topk_prob", False), self.margins[l])
+        self.margins[l], self.swaps[l] = [], []
+        return moe(xb, w, c["num_experts_per_tok"], c.get("norm_topk_prob", False), self.margins[l],
+                   other_side={pos: ij for (layer, pos), ij in self.other_side.items() if layer == l}, swaps=self.swaps[l])
 
     def logits(self, tokens) -> torch.Tensor:
         """Logits [T, vocab] at every position of one sequence (step order of
@@ -241,6 +263,15 @@ class PlainQwen2Moe:
         x = rmsnorm(x, t["model.norm.weight"], self.eps)                                      # :2922
         head = t["lm_head.weight"] if "lm_head.weight" in t else t["model.embed_tokens.weight"]   # tq_model.c:1499-1516
         return matvec_rows(head, x)                                                           # :2931-2942
+
+    def near_ties(self, bound: float, position: int | None = None) -> list:
+        """(gap, layer, position, i, j) of every exchange of a chosen expert (rank i) for one left out (rank j) in
+        the last ``logits`` call whose gap is under ``bound``, at ``position`` or at all positions, smallest first."""
+        out = []
+        for l in sorted(self.swaps):
+            for p in (range(len(self.swaps[l])) if position is None else [position]):
+                out += [(gap, l, p, i, j) for gap, i, j in self.swaps[l][p] if gap < bound]
+        return sorted(out)
 
     def min_margins(self) -> torch.Tensor:
         """For every token of the last ``logits`` call, its smallest routing margin over the sparse layers."""

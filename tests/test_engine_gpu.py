@@ -3,13 +3,24 @@ whole, with the last 32 tokens one by one, in batches of unequal lengths one aft
 ``bin/trace_run``, as a user runs it); long decoding; the first tokens; generation through the entry point;
 each part alone; and a toy mixer with state of its own that is registered from here.
 
-How results are compared.  In 32-bit every logit must lie within 1e-4 of the plain implementation's.  In
-bfloat16 every rounding is about 2^-9 of a value, which through the layers comes to about a hundredth of the
-largest logit; but where two experts' router logits nearly tie, that rounding changes which expert runs and the
-logits of that position move by much more.  The plain model reports each position's routing margin; positions
-with a margin under 0.02 (in units of the router logits' spread) are left out, there may not be many of
-them, and the rest must be close: nine in ten within 2 %, all within 10 % of the largest logit.
+How results are compared.  A routing decision is a comparison of two router logits, and where the plain model
+(float64) finds the last expert chosen and the best one left out close together, an arithmetic with other
+rounding may order them the other way; then another expert runs, and the logits of that position and of every
+later position of the sequence (which attend to it) move by far more than rounding.  So wherever all positions of
+a sequence are observed, results are compared with the plain model *after it has taken the engine's side at such
+near-ties*, found like this (``check_sequence``): at the first position that differs, the plain model's near-ties at
+that position (a chosen expert and one left out whose router logits differ by less than F32_TIE = 1e-5 of the
+logits' spread in 32-bit, BF16_TIE = 0.08 in bfloat16) are decided the other way, one at a time or one in each of
+two layers, and the one way that brings the position within the
+bound is kept; a difference that no near-tie of that very position explains is a failure, and so is any position
+that stays beyond the bound.  No position is left out.  The bounds: 1e-4 in 32-bit; in bfloat16, where every
+rounding is about 2^-9 of a value, 4 % of the largest logit at every position and 1.5 % at nine in ten.
+Where only some positions are observed (decoded tokens after a long prompt), near-ties of the unobserved part
+cannot be found that way: 32-bit is still held to 1e-4 (the fixed seeds have no near-tie there), bfloat16 to the
+looser ``check_logits``: positions with a margin under 0.02 are left out, there may not be many of them, and the
+rest must lie within 10 % of the largest logit, nine in ten within 2 %.
 """
+import itertools
 import json
 import math
 import os
@@ -29,6 +40,8 @@ DEV = "cuda:0"
 SHARP = 0.1        # weights this wide make attention and routing matter; 0.02 leaves softmaxes nearly flat
 ACTS = ["float32", "bfloat16"]
 MARGIN = 0.02
+F32_TIE = 1e-5     # routing margin under which float32 and float64 may order two experts differently
+BF16_TIE = 0.08    # the same for bfloat16 activations
 
 
 @pytest.fixture(scope="module")
@@ -84,6 +97,50 @@ def check_logits(got, ref, margins, act, what):
     assert rel.quantile(0.9) < 0.02, f"{what}: a tenth of the bfloat16 logits differ by more than {rel.quantile(0.9):.1%}"
 
 
+def check_sequence(got, plain, prompt, act, what):
+    """``got``: the engine's logits at every position of one sequence.  They must agree with the plain model once
+    it has decided its near-ties as the engine did (see the top of this file).  Returns how many decisions were
+    turned."""
+    got = got.double().cpu()
+    assert got.shape[0] == len(prompt), what
+    tie = F32_TIE if act == "float32" else BF16_TIE
+    plain.other_side = {}
+    try:
+        ref = plain.logits(prompt)
+        scale = ref.abs().max().item()
+        tol = 1e-4 if act == "float32" else 0.04 * scale
+        for _ in range(len(prompt)):
+            err = (got - ref).abs().max(dim=-1).values
+            bad = (err > tol).nonzero()
+            if bad.numel() == 0:
+                break
+            p = int(bad[0])
+            swaps = [(l, i, j) for _gap, l, _p, i, j in plain.near_ties(tie, p) if (l, p) not in plain.other_side]
+            tries = [(s,) for s in swaps] + [c for c in itertools.combinations(swaps[:6], 2) if c[0][0] != c[1][0]]
+            settled = False
+            for combo in tries:
+                for l, i, j in combo:
+                    plain.other_side[(l, p)] = (i, j)
+                ref2 = plain.logits(prompt)
+                if (got[p] - ref2[p]).abs().max().item() <= tol:
+                    ref, settled = ref2, True
+                    break
+                for l, i, j in combo:
+                    del plain.other_side[(l, p)]
+            if not settled:
+                plain.logits(prompt)
+                raise AssertionError(f"{what}: {act} logits at position {p} differ by {err[p]:.2e} (bound {tol:.2e}) and no "
+                                     f"near-tie of that position explains it (nearest exchanges {plain.near_ties(1.0, p)[:4]})")
+        err = (got - ref).abs().max(dim=-1).values
+        assert err.max() <= tol, f"{what}: position {int(err.argmax())} differs by {err.max():.2e}"
+        if act != "float32":
+            q90 = err.quantile(0.9).item() / scale
+            assert q90 < 0.015, f"{what}: a tenth of the bfloat16 logits differ by more than {q90:.1%} of the largest logit"
+        return len(plain.other_side)
+    finally:
+        plain.other_side = {}
+
+
 def plain_rows(plain, prompt):
     ref = plain.logits(prompt)
     return ref, plain.min_margins() if plain.margins else torch.full((len(prompt),), math.inf)
@@ -127,7 +184,7 @@ def build_trace(prompts):
         ids = {i: f"b{b}:{i}" for i in members}
         cut = {i: max(1, len(prompts[i]) - 5 - 3 * j) for j, i in enumerate(members)}
         done = [i for i in members if cut[i] == len(prompts[i])]
-        emit([(ids[i], prompts[i][:cut[i]], [cut[i] - 1], 0) for i in members], [ids[i] for i in done])
+        emit([(ids[i], prompts[i][:cut[i]], list(range(cut[i])), 0) for i in members], [ids[i] for i in done])
         pos = dict(cut)
         going = [i for i in members if i not in done]
         while going:
@@ -136,11 +193,32 @@ def build_trace(prompts):
             for i in going:
                 pos[i] += 1
             going = [i for i in going if i not in done]
+    # 4. cuts that the step function takes beyond what the replay format promises: a prompt fed as chunks of several
+    #    tokens (a run of tokens that does not start at position 0), and steps in which one request brings a whole
+    #    prompt or a chunk while others go on by one token
+    big = max(range(len(prompts)), key=lambda i: len(prompts[i]))
+    p = prompts[big]
+    a, b = max(1, len(p) // 3), max(2, 2 * len(p) // 3)
+    if len(p) >= 3:
+        emit([(f"m:{big}", p[:a], list(range(a)), 0)], [])
+        emit([(f"m:{big}", p[a:b], list(range(b - a)), a)], [])
+        emit([(f"m:{big}", p[b:], list(range(len(p) - b)), b)], [f"m:{big}"])
+    others = [i for i in range(len(prompts)) if i != big and len(prompts[i]) >= 6][:2]
+    if others:
+        ids = {i: f"m2:{i}" for i in others}
+        cut = {i: len(prompts[i]) - 4 for i in others}
+        emit([(ids[i], prompts[i][:cut[i]], list(range(cut[i])), 0) for i in others], [])
+        # the big request's first chunk arrives while the others decode; then its next chunk; then all go on by one
+        emit([(ids[i], [prompts[i][cut[i]]], [0], cut[i]) for i in others] + [(f"m2:{big}", p[:a], list(range(a)), 0)], [])
+        emit([(f"m2:{big}", p[a:b], list(range(b - a)), a)] + [(ids[i], [prompts[i][cut[i] + 1]], [0], cut[i] + 1) for i in others], [])
+        emit([(ids[i], [prompts[i][cut[i] + 2]], [0], cut[i] + 2) for i in others] + [(f"m2:{big}", [p[b]], [0], b)], [])
+        emit([(ids[i], [prompts[i][cut[i] + 3]], [0], cut[i] + 3) for i in others] + [(f"m2:{big}", p[b + 1:], list(range(len(p) - b - 1)), b + 1)],
+             list(ids.values()) + [f"m2:{big}"])
     return lines, expect, peak
 
 
 @pytest.mark.parametrize("act", ACTS)
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_replay(name, act, sharp_dirs, tmp_path):
     d, plain = sharp_dirs(name, act)
     prompts = prompts_for(name, [1, 7, 33, 70, 150], seed=11)
@@ -151,22 +229,24 @@ def test_replay(name, act, sharp_dirs, tmp_path):
     run = subprocess.run(cmd, input="\n".join(lines) + "\n", capture_output=True, text=True, timeout=600)
     assert run.returncode == 0, run.stderr[-2000:]
     assert [l for l in run.stdout.splitlines() if l.startswith("done ")] == [f"done {s}" for s in range(len(lines))]
-    refs = [plain_rows(plain, p) for p in prompts]
     V = TINY[name][0]["vocab_size"]
-    got, want, margins = {"w": [], "d": [], "b": []}, {"w": [], "d": [], "b": []}, {"w": [], "d": [], "b": []}
     steps_with_output = sorted(int(f[:-4]) for f in os.listdir(out) if f.endswith(".f32"))
     assert steps_with_output == sorted(expect)
-    for s, rows in expect.items():
-        data = torch.frombuffer(bytearray((out / f"{s}.f32").read_bytes()), dtype=torch.float32).view(-1, V)
+    seen = {}                      # request id -> {position: logits}
+    for s_, rows in expect.items():
+        data = torch.frombuffer(bytearray((out / f"{s_}.f32").read_bytes()), dtype=torch.float32).view(-1, V)
         assert data.shape[0] == len(rows)
-        kind = json.loads(lines[s])["entries"][0]["id"][0]
-        for r, (req, posn) in enumerate(rows):
-            got[kind].append(data[r])
-            want[kind].append(refs[int(req)][0][posn])
-            margins[kind].append(refs[int(req)][1][posn])
-    for kind, what in (("w", "whole"), ("d", "last 32 one by one"), ("b", "unequal batches")):
-        check_logits(torch.stack(got[kind]), torch.stack(want[kind]), torch.stack(margins[kind]).float(), act,
-                     f"{name} {act} {what}")
+        ids = [e["id"] for e in json.loads(lines[s_])["entries"] for _ in e["want"]]
+        for r, ((req, posn), rid) in enumerate(zip(rows, ids)):
+            seen.setdefault(rid, {})[posn] = data[r]
+    names = {"w": "whole", "d": "last 32 one by one", "b": "unequal batches", "m": "chunks", "m2": "mixed steps"}
+    assert {rid.split(":")[0].rstrip("0123456789") for rid in seen} == {"w", "d", "b", "m"}
+    for rid, rows in seen.items():
+        tag, req = rid.split(":")
+        prompt = prompts[int(req)]
+        assert sorted(rows) == list(range(len(prompt))), f"{rid}: the trace does not ask for every position"
+        check_sequence(torch.stack([rows[i] for i in range(len(prompt))]), plain, prompt, act,
+                       f"{name} {act} {names[tag if tag == 'm2' else tag[0]]} request {req}")
 
 
 # ------------------------------------------------------------------------------------------------ in process
@@ -175,18 +255,17 @@ def test_replay(name, act, sharp_dirs, tmp_path):
 def test_first_tokens_and_long_decoding(name, act, engines):
     eng, plain = engines(name, act)
     (seq,) = prompts_for(name, [330], seed=12)
-    ref, margins = plain_rows(plain, seq)
     slot = eng.open(1)
     rows = [eng.step(slot, [seq[:3]], [[0, 1, 2]])]                 # the first tokens of a sequence, in one step
     for t in range(3, len(seq)):
         rows.append(eng.step(slot, [[seq[t]]]))
     eng.close(slot)
-    check_logits(torch.cat(rows), ref, margins, act, f"{name} {act} long decoding")
+    check_sequence(torch.cat(rows), plain, seq, act, f"{name} {act} long decoding")
     for n in (1, 2):                                                # and as the whole of a very short sequence
         slot = eng.open(1)
         lg = eng.step(slot, [seq[:n]], [list(range(n))])
         eng.close(slot)
-        check_logits(lg, ref[:n], margins[:n], act, f"{name} {act} first {n} tokens")
+        check_sequence(lg, plain, seq[:n], act, f"{name} {act} first {n} tokens")
 
 
 def test_the_layer_sizes_of_a_real_checkpoint(tmp_path):
@@ -209,8 +288,6 @@ def test_the_layer_sizes_of_a_real_checkpoint(tmp_path):
     for act in ACTS:
         d = write_random_model_dir(str(tmp_path / f"a27b_two_layers_{act}"), cfg, 3, 0.02, 0.02, act)
         plain = PlainQwen2Moe(d)
-        refs = [plain_rows(plain, s) for s in seqs]
-        del plain
         eng = Engine(load_model(d, act=act, device=DEV), max_tokens=64 * 8)
         slots = eng.open(3)
         prompts = [s[:-n_fed] for s in seqs]
@@ -221,11 +298,12 @@ def test_the_layer_sizes_of_a_real_checkpoint(tmp_path):
         torch.cuda.empty_cache()
         shutil.rmtree(d)              # gigabytes of weights: not kept for the next test session to find
         off = 0
-        for i, (s, (ref, margins)) in enumerate(zip(seqs, refs)):
+        for i, s in enumerate(seqs):
             n = len(s) - n_fed
             got = torch.cat([first[off:off + n]] + [f[i:i + 1] for f in fed])
             off += n
-            check_logits(got, ref, margins, act, f"real layer sizes, {act}, sequence of {len(s)}")
+            check_sequence(got, plain, s, act, f"real layer sizes, {act}, sequence of {len(s)}")
+        del plain
 
 
 @pytest.mark.parametrize("act", ACTS)
@@ -289,9 +367,8 @@ def test_a_request_does_not_feel_its_batch_or_its_place_in_the_cache(act, engine
     if act == "float32":
         assert diff < 2e-5
     else:
-        ref, margins = plain_rows(plain, prompts[0])
-        check_logits(torch.cat(rows), ref, margins, act, "in a batch")
-        check_logits(alone, ref, margins, act, "alone")
+        check_sequence(torch.cat(rows), plain, prompts[0], act, "in a batch")
+        check_sequence(alone, plain, prompts[0], act, "alone")
     assert eng.cache.n_live == 0
 
 

@@ -130,6 +130,23 @@ def test_gemm_partial_sums(ops, act, M, N, K, bias):
 
 
 @pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("activation", ["silu", "gelu_tanh", "relu2"])
+@pytest.mark.parametrize("M,N,K", [(3, 40, 72), (40, 130, 264), (150, 200, 136), (9, 33, 50)])
+def test_gated_products_take_the_activation_as_a_parameter(ops, act, activation, M, N, K):
+    """The gate of a gated pair is a parameter of the products' epilogues: every kernel family (few rows, tiles,
+    plain multiply-adds where K is no multiple of 4 or 8) with each activation."""
+    a, w, w2 = rnd((M, K), adt(act), 22), rnd((N, K), adt(act), 23, 0.3), rnd((N, K), adt(act), 24, 0.3)
+    y = ops.gemm(a.to(DEV), w.to(DEV), act, w2=w2.to(DEV), activation=activation).cpu().double()
+    g = a.double() @ w.double().T
+    gate = {"silu": g / (1 + torch.exp(-g)), "relu2": torch.relu(g) ** 2,
+            "gelu_tanh": 0.5 * g * (1 + torch.tanh(math.sqrt(2 / math.pi) * (g + 0.044715 * g ** 3)))}[activation]
+    ref = gate * (a.double() @ w2.double().T)
+    assert (y - ref).abs().max() < (1e-5 * math.sqrt(K) if act == "float32" else 4e-3) * ref.abs().max()
+    with pytest.raises(ops.KernelError, match="unknown activation"):
+        ops.gemm(a.to(DEV), w.to(DEV), act, w2=w2.to(DEV), activation="swish")
+
+
+@pytest.mark.parametrize("act", ACTS)
 def test_gemm_float32_weights_on_the_bfloat16_path(ops, act):
     """A matrix the checkpoint stores in 32 bits stays so and still multiplies."""
     a = rnd((9, 72), adt(act), 20)

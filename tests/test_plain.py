@@ -244,3 +244,20 @@ def test_repetition_penalty_counts_every_occurrence():
     assert l.tolist() == [0.25, -4.0, 3.0, 1.0]
     P.apply_rep_penalty(l, [0], window=32, penalty=1.0)
     assert l[0] == 0.25
+
+
+def test_a_near_tie_decided_the_other_way_exchanges_two_experts():
+    """``route(..., other_side=(i, j))`` puts the expert of rank j in the place of rank i; ``near_swaps`` lists the
+    exchanges by the gap of their logits."""
+    router = torch.zeros(6, 4, dtype=torch.float64)
+    for e, v in enumerate([5.0, 1.0, 4.0, 3.99, 3.0, 3.98]):
+        router[e, 0] = v
+    x = torch.tensor([1.0, 0, 0, 0], dtype=torch.float64)
+    ids, w = P.route(x, router, 2, True)
+    assert ids == [0, 2] and abs(float(w.sum()) - 1) < 1e-12
+    ids2, w2 = P.route(x, router, 2, True, other_side=(1, 2))
+    assert ids2 == [0, 3] and abs(float(w2[1] / w2[0]) - math.exp(3.99 - 5.0)) < 1e-12
+    assert P.route(x, router, 2, True, other_side=(1, 3))[0] == [0, 5]
+    assert P.route(x, router, 2, True, other_side=(0, 2))[0] == [3, 2]
+    swaps = P.near_swaps(x, router, 2)
+    assert [(i, j) for _, i, j in swaps[:2]] == [(1, 2), (1, 3)] and swaps[0][0] < swaps[1][0] < 0.02

@@ -1,0 +1,235 @@
+"""Schedules and entry points that the other GPU tests do not reach: a window whose pages are given back and used
+again while decoding goes on; decode steps of 17 to 64 sequences, replayed and eager; sequences that cross the
+positions at which decode graphs and attention runs change shape; the command line; a context length that binds;
+and float32 routing near-ties."""
+import copy
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from plain_qwen2moe import PlainQwen2Moe, generate as plain_generate
+from test_engine_gpu import (ACTS, DEV, F32_TIE, ROOT, SHARP, check_logits, check_sequence, plain_rows,
+                             prompts_for)
+from tiny_configs import TINY
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def sharp(tmp_path_factory):
+    from turboquant_cpp_amd.engine.model import load_model, write_random_model_dir
+    made = {}
+
+    def get(name, act, **changes):
+        key = (name, act, tuple(sorted(changes.items())))
+        if key not in made:
+            cfg, init = TINY[name]
+            cfg = dict(copy.deepcopy(cfg), **changes)
+            d = str(tmp_path_factory.mktemp(f"sched_{name}_{act}"))
+            write_random_model_dir(d, cfg, init["seed"], SHARP, init["norm_std"], act)
+            made[key] = (d, PlainQwen2Moe(d), load_model(d, act=act, device=DEV))
+        return made[key]
+    return get
+
+
+# ------------------------------------------------------------------------------------------------ a window's pages
+@pytest.mark.parametrize("act", ACTS)
+def test_a_window_gives_pages_back_and_a_second_sequence_uses_them(act, sharp):
+    """Configuration C: heads of 32 (the matrix-core attention in bfloat16), a window of 40 on layers 1 and 2.  A
+    sequence decodes far past window + page, so that the windowed group hands its early pages back; a second
+    sequence then starts in those pages and both go on.  Replayed and eager steps must agree bit for bit, and
+    both with the plain model."""
+    from turboquant_cpp_amd.engine.step import Engine
+    d, plain, model = sharp("C", act)
+    first, second = prompts_for("C", [260, 150], seed=21)
+    out = {}
+    for graphs in (True, False):
+        eng = Engine(model, max_tokens=64 * 8, max_slots=2, use_graphs=graphs)
+        assert (eng.graphs is not None) == graphs
+        full, win = eng.cache.groups if eng.cache.groups[0].key.window is None else eng.cache.groups[::-1]
+        a = eng.open(1)[0]
+        rows_a = [eng.step([a], [first[:30]], [list(range(30))])]
+        for t in range(30, 200):
+            rows_a.append(eng.step([a], [[first[t]]]).clone())
+        held_by_a = set(win.host_table[a][win.host_table[a] >= 0].tolist())
+        assert len(held_by_a) <= 2 and (full.host_table[a] >= 0).sum() == 4      # window 40: at most two pages of 64
+        b = eng.open(1)[0]
+        rows_b = [eng.step([b], [second[:100]], [list(range(100))])]
+        used_again = set(win.host_table[b][win.host_table[b] >= 0].tolist())
+        assert used_again and not (used_again & held_by_a)
+        for t in range(50):
+            lg = eng.step([a, b], [[first[200 + t]], [second[100 + t]]]).clone()
+            rows_a.append(lg[0:1])
+            rows_b.append(lg[1:2])
+        eng.close([b])
+        for t in range(250, 260):
+            rows_a.append(eng.step([a], [[first[t]]]).clone())
+        eng.close([a])
+        assert all(g.pool.n_free == g.pool.n_pages for g in eng.cache.groups)
+        out[graphs] = (torch.cat(rows_a), torch.cat(rows_b))
+    for x, y in zip(out[True], out[False]):
+        assert torch.equal(x, y), "replayed steps differ from eager steps"
+    check_sequence(out[True][0], plain, first, act, f"C {act} windowed decoding, first sequence")
+    check_sequence(out[True][1], plain, second, act, f"C {act} windowed decoding, second sequence")
+
+
+# ------------------------------------------------------------------------------------------------ many sequences
+@pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("name,n_seqs", [("A", 40), ("B", 17), ("C", 64)])
+def test_decode_steps_of_many_sequences(name, n_seqs, act, sharp):
+    """More than 16 sequences decode together: the feed-forward leaves the launches it uses for a handful of tokens
+    and puts the shared expert on a second stream, which a captured graph records as a fork and a join.  Replays
+    are compared with eager steps bit for bit, and both with the plain model."""
+    from turboquant_cpp_amd.engine.step import Engine
+    d, plain, model = sharp(name, act)
+    g = torch.Generator().manual_seed(23)
+    lens = [int(torch.randint(1, 40, (1,), generator=g)) for _ in range(n_seqs)]
+    n_dec = 7
+    seqs = prompts_for(name, [n + n_dec for n in lens], seed=24)
+    out = {}
+    for graphs in (True, False):
+        eng = Engine(model, max_tokens=64 * n_seqs, max_slots=n_seqs, use_graphs=graphs)
+        slots = eng.open(n_seqs)
+        first = eng.step(slots, [s[:n] for s, n in zip(seqs, lens)], [list(range(n)) for n in lens])
+        rows = []
+        for t in range(n_dec):
+            rows.append(eng.step(slots, [[s[n + t]] for s, n in zip(seqs, lens)]).clone())
+            if t == 3:
+                torch.cuda.synchronize()
+        eng.close(slots)
+        if graphs:
+            assert len(eng.graphs.graphs) == 1
+        out[graphs] = (first, torch.stack(rows))    # [prompt rows, vocab], [step, sequence, vocab]
+    assert torch.equal(out[True][1], out[False][1]), "replayed steps differ from eager steps"
+    assert torch.equal(out[True][0], out[False][0])
+    starts = [sum(lens[:i]) for i in range(n_seqs)]
+    for i in range(0, n_seqs, 5):
+        got = torch.cat([out[True][0][starts[i]:starts[i] + lens[i]], out[True][1][:, i]])
+        check_sequence(got, plain, seqs[i], act, f"{name} {act} sequence {i} of {n_seqs}")
+
+
+# ------------------------------------------------------------------------------------------------ long sequences
+@pytest.mark.parametrize("act", ACTS)
+def test_sequences_cross_the_positions_where_steps_change_shape(act, sharp):
+    """Decode graphs are kept per 2,048 positions of the longest sequence, and from position 4,096 on attention
+    joins runs of three tiles instead of one: a sequence is decoded across 2,048 and another across 4,096 (with a
+    short one beside it), through the engine, replayed and eager, against the plain model."""
+    from turboquant_cpp_amd.engine.step import Engine
+    d, plain, model = sharp("A", act, max_position_embeddings=8192)
+    long, short = prompts_for("A", [4110, 40], seed=25)
+    ref, margins = plain_rows(plain, long)
+    ref_s, margins_s = plain_rows(plain, short)
+    out = {}
+    for graphs in (True, False):
+        eng = Engine(model, max_tokens=64 * 100, max_slots=2, use_graphs=graphs)
+        rows, where, rows_s = [], [], []
+        for start, n in ((2040, 16), (4088, 16)):
+            a, b = eng.open(2)
+            eng.step([a, b], [long[:start], short[:20]], [[], []])
+            for t in range(n):
+                lg = eng.step([a, b], [[long[start + t]], [short[20 + t]]]).clone()
+                rows.append(lg[0])
+                where.append(start + t)
+                rows_s.append(lg[1])
+            eng.close([a, b])
+        if graphs:
+            assert sorted(k[1] for k in eng.graphs.graphs) == [2048, 4096, 6144]
+        out[graphs] = (torch.stack(rows), torch.stack(rows_s))
+    for x, y in zip(out[True], out[False]):
+        assert torch.equal(x, y), "replayed steps differ from eager steps"
+    check_logits(out[True][0], ref[where], margins[where], act, f"A {act} across 2,048 and 4,096")
+    check_logits(out[True][1], torch.cat([ref_s[20:36]] * 2), torch.cat([margins_s[20:36]] * 2), act, f"A {act} the short one beside it")
+
+
+# ------------------------------------------------------------------------------------------------ entry points
+@pytest.mark.parametrize("act", ACTS)
+def test_the_command_line_generates(act, sharp):
+    """``bin/quant DIR -p ... -n 8 -T 0 --json`` in a process of its own, with the options' defaults otherwise
+    (repetition penalty 1.1, loop detection): float32 gives the plain loop's tokens; bfloat16 tokens are each, by
+    the plain model's logits after the same penalty, the best or within rounding of it."""
+    d, plain, _ = sharp("B", act)
+    prompts = prompts_for("B", [5, 12, 3], seed=26)
+    text = ";".join(",".join(str(t) for t in p) for p in prompts)
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "quant"), d, "-p", text, "-n", "8", "-T", "0", "--json",
+           "--dtype", act, "--stop-id", "383"]
+    run = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr[-2000:]
+    res = json.loads(run.stdout.strip().splitlines()[-1])
+    assert "tok/s" in run.stderr and len(res) == 3
+    for p, r in zip(prompts, res):
+        want = plain_generate(plain, p, max_tokens=8, rep_penalty=1.1, stop_tokens=(383,), loop_detection=True)
+        if act == "float32":
+            assert r["tokens"] == want and r["finish_reason"] in ("length", "stop", "loop")
+        else:
+            import plain_qwen2moe as P
+            assert 1 <= len(r["tokens"]) <= 8
+            lg = plain.logits(p + r["tokens"])
+            recent = list(p[-32:])
+            for j, tok in enumerate(r["tokens"]):
+                row = lg[len(p) - 1 + j].to(torch.float32).numpy().copy()
+                P.apply_rep_penalty(row, recent, 32, 1.1)
+                assert row[tok] >= row.max() - 0.05 * float(lg.abs().max()), (j, tok)
+                recent.append(tok)
+    info = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "quant"), d, "--info"], capture_output=True, text=True)
+    assert info.returncode == 0 and "Qwen2MoeForCausalLM" in info.stdout
+
+
+def test_a_context_length_binds_and_a_full_cache_ends_sequences(sharp):
+    from turboquant_cpp_amd import Model
+    d, plain, _ = sharp("A", "float32")
+    prompts = prompts_for("A", [100, 60, 20, 127, 128, 129], seed=27)
+    with Model(d, dtype="float32", temperature=0.0, rep_penalty=1.0, max_tokens=200, context_length=128, max_batch=4,
+               stop_tokens=()) as m:
+        assert m.context_length == 128 and m.engine.cache.max_positions == 128
+        res = m.generate_detailed(prompts, loop_detection=False)
+        assert m.engine.cache.n_live == 0
+    # a sequence of n positions has run n - 1 generated tokens' worth of room: the token sampled at the last
+    # position is still emitted; a prompt that fills the context gives one token, a longer one none
+    assert all(r.finish_reason == "context" for r in res)
+    assert [len(r.tokens) for r in res] == [28, 68, 108, 1, 1, 0]
+    want = plain_generate(plain, prompts[0], max_tokens=28)
+    assert res[0].tokens == want
+
+
+# ------------------------------------------------------------------------------------------------ float32 near-ties
+def test_a_float32_near_tie_is_decided_either_way_and_nothing_else_differs(tmp_path):
+    """Two router rows that differ in the last bit of one element: their logits differ by less than float32 sums
+    resolve, so float32 sees a tie (the higher index wins) where float64 sees an order.  Where the two experts lie
+    on either side of the cut, another expert runs and the logits differ by far more than 1e-4; the comparison has
+    to find exactly that and accept nothing else."""
+    from turboquant_cpp_amd.engine.model import load_model, write_random_model_dir
+    from turboquant_cpp_amd.engine.step import Engine
+    from turboquant_cpp_amd.weights.safetensors_io import SafetensorsFolder, write_safetensors
+    cfg = dict(copy.deepcopy(TINY["A"][0]), num_experts=4, num_experts_per_tok=2)
+    d = write_random_model_dir(str(tmp_path / "ties"), cfg, 9, SHARP, 0.0, "float32")
+    with SafetensorsFolder(d) as f:
+        tensors = {n: f.read(n).clone() for n in f.names()}
+    r = tensors["model.layers.0.mlp.gate.weight"]
+    r[3] = r[2]
+    j = int(r[2].abs().argmin())
+    r[3, j] = torch.nextafter(r[3, j], torch.tensor(float("inf")))       # one bit in the smallest element
+    write_safetensors(os.path.join(d, "model.safetensors"), tensors)
+    plain = PlainQwen2Moe(d)
+    eng = Engine(load_model(d, act="float32", device=DEV), max_tokens=64 * 4)
+    turned, exact, ties = 0, 0, 0
+    for prompt in prompts_for("A", [10] * 8, seed=28):
+        slot = eng.open(1)
+        got = eng.step(slot, [prompt], [list(range(len(prompt)))])
+        eng.close(slot)
+        n = check_sequence(got, plain, prompt, "float32", "near-ties")
+        plain.logits(prompt)
+        ties += len(plain.near_ties(F32_TIE))
+        turned += n
+        exact += n == 0
+    assert ties > 0 and turned > 0, "the test's weights make no near-tie that float32 decides the other way"
+    # a real difference is not excused by a near-tie elsewhere
+    prompt = prompts_for("A", [10], seed=29)[0]
+    slot = eng.open(1)
+    got = eng.step(slot, [prompt], [list(range(len(prompt)))])
+    eng.close(slot)
+    with pytest.raises(AssertionError):
+        check_sequence(got + 1e-3, plain, prompt, "float32", "a shifted result")

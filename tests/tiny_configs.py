@@ -1,4 +1,4 @@
-"""Two tiny Qwen2-MoE configurations that differ in every size and option."""
+"""Tiny Qwen2-MoE configurations that differ in every size and option."""
 
 # MHA, head 16, theta 1e4, eps 1e-6, no window, 8 experts top-2 un-normalised, every layer sparse, norm weights 1
 TINY_A = {
@@ -25,4 +25,18 @@ TINY_B = {
 }
 TINY_B_INIT = dict(seed=1, std=0.02, norm_std=0.02)
 
-TINY = {"A": (TINY_A, TINY_A_INIT), "B": (TINY_B, TINY_B_INIT)}
+# heads of 32 on 2 kv heads (the matrix-core attention takes them; hidden size is not heads x head size), a window of
+# 40 from layer 1 (smaller than a page of the cache and no multiple of anything), one expert per token out of 5,
+# normalised, no shared expert, layer 1 dense, tied embeddings, theta 5e4
+TINY_C = {
+    "architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe",
+    "vocab_size": 200, "hidden_size": 96, "num_hidden_layers": 3, "num_attention_heads": 6,
+    "num_key_value_heads": 2, "head_dim": 32, "intermediate_size": 112, "moe_intermediate_size": 40,
+    "shared_expert_intermediate_size": 0, "num_experts": 5, "num_experts_per_tok": 1, "norm_topk_prob": True,
+    "decoder_sparse_step": 1, "mlp_only_layers": [1], "rope_theta": 50000.0, "rms_norm_eps": 1e-6,
+    "use_sliding_window": True, "sliding_window": 40, "max_window_layers": 1, "max_position_embeddings": 2048,
+    "tie_word_embeddings": True, "torch_dtype": "float32",
+}
+TINY_C_INIT = dict(seed=5, std=0.02, norm_std=0.02)
+
+TINY = {"A": (TINY_A, TINY_A_INIT), "B": (TINY_B, TINY_B_INIT), "C": (TINY_C, TINY_C_INIT)}

@@ -5,7 +5,7 @@
 // every weight type the matrix-core kernels do not take; each output element is summed over k in
 // ascending order by one thread, so a row's result does not depend on which other rows are in
 // the product.  One kernel covers the plain product, the product with bias, the gated pair
-// silu(a w_gate) * (a w_up) (/root/reference/src/engine/tq_transformer.c:2770-2794), and the
+// gate(a w_gate) * (a w_up), gate being silu or another activation (/root/reference/src/engine/tq_transformer.c:2770-2794), and the
 // same over groups of rows that each use their own matrix (experts,
 // /root/reference/src/engine/tq_moe.c:864-999): rows are then taken from `a` through a_rows and
 // row tile i uses matrix tile_group[i].
@@ -29,9 +29,8 @@ struct GemmArgs {
   void* out;               // [M][N] float, or act_t when OUT_ACT
   int64_t ldc;
   int M, N, K;
+  int gate;                // activation of the gated pair
 };
-
-__device__ __forceinline__ float silu(float x) { return x / (1.0f + expf(-x)); }
 
 template <class W, int TM, bool DUAL, bool OUT_ACT>
 __global__ __launch_bounds__(256) void gemm_generic_kernel(GemmArgs g) {
@@ -108,7 +107,7 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(GemmArgs g) {
       if (n >= g.N) continue;
       float v = acc[i][j];
       if (g.bias) v += g.bias_type == TQ_F32 ? ((const float*)g.bias)[n] : to_f32(((const bf16_t*)g.bias)[n]);
-      if (DUAL) v = silu(v) * acc2[i][j];
+      if (DUAL) v = gate_fn(v, g.gate) * acc2[i][j];
       if (OUT_ACT)
         ((act_t*)g.out)[(size_t)m * g.ldc + n] = from_f32<act_t>(v);
       else
@@ -135,11 +134,12 @@ static void launch(const GemmArgs& g, bool dual, bool out_act, hipStream_t st) {
 TQ_API int tq_gemm_generic(const void* a, int64_t lda, const int* a_rows, int a_gather, const void* w, const void* w2, int wtype,
                            int64_t group_stride, const int* tile_group, const int* n_tiles, const void* bias,
                            int bias_type, void* out, int64_t ldc, int out_is_act, int M, int N, int K, int tile_rows,
-                           hipStream_t st) {
+                           int gate, hipStream_t st) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || (tile_rows != 16 && tile_rows != 64)) return TQ_ERR_BAD_ARG;
   if ((N + BN - 1) / BN > 65535) return TQ_ERR_UNSUPPORTED;
-  GemmArgs g{(const act_t*)a, lda, a_rows, a_gather, w, w2, group_stride, tile_group, n_tiles, bias, bias_type, out, ldc, M, N, K};
+  if (gate < 0 || gate >= TQ_GATE_COUNT) return TQ_ERR_BAD_ARG;
+  GemmArgs g{(const act_t*)a, lda, a_rows, a_gather, w, w2, group_stride, tile_group, n_tiles, bias, bias_type, out, ldc, M, N, K, gate};
   TQ_DISPATCH_W(wtype, {
     if (tile_rows == 16)
       launch<W, 1>(g, w2 != nullptr, out_is_act != 0, st);

@@ -1,7 +1,7 @@
 // Matrix products out[m, n] = sum_k a[m, k] * w[n, k] on the matrix cores, bfloat16 in, float sums.
 //
 // Same contract as the plain product (gemm_generic.hip): optional bias, optional gated pair
-// silu(a w^T) * (a w2^T), optional row gather and per-row-tile matrices for experts.  Two kernels:
+// gate(a w^T) * (a w2^T) (gate: silu or another activation), optional row gather and per-row-tile matrices for experts.  Two kernels:
 //
 //  * gemm_stream_kernel, for few rows (decoding): the work is reading w once.  A wave owns 16 rows of w
 //    and streams them straight from memory into the operand registers of v_mfma_f32_16x16x32_bf16 (lane
@@ -43,9 +43,8 @@ struct MfmaGemmArgs {
   int M, N, K;
   int k_per;                // k is split into runs of k_per, run z going to out + z * split_stride (float)
   int64_t split_stride;
+  int gate;                 // activation of the gated pair
 };
-
-__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
 
 // For bytes that are read once (a matrix streamed past a few rows): a load that tells the caches so.  Measured on
 // a plain read of 1 GiB whose instructions take whole lines of 128 bytes: 6.8 TB/s with this hint, 4.7 without; with
@@ -228,7 +227,7 @@ __device__ __forceinline__ void stream_body(MfmaGemmArgs g, int tile_n, int tile
       if (on >= g.N || om >= g.M) continue;
       if (g.a_rows && g.a_rows[om] < 0) continue;
       float o = s + bias_at(g, on);
-      if (DUAL) o = silu_f(o) * s2;
+      if (DUAL) o = gate_fn(o, g.gate) * s2;
       store_out<OUT_ACT>(g, om, on, o);
     }
     return;
@@ -246,7 +245,7 @@ __device__ __forceinline__ void stream_body(MfmaGemmArgs g, int tile_n, int tile
         if (m >= g.M) continue;
         if (g.a_rows && g.a_rows[m] < 0) continue;
         float o = acc[t][mt][v] + b;
-        if (DUAL) o = silu_f(o) * acc2[t][mt][v];
+        if (DUAL) o = gate_fn(o, g.gate) * acc2[t][mt][v];
         store_out<OUT_ACT>(g, m, n, o);
       }
   }
@@ -560,7 +559,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g)
         if (m >= g.M) continue;
         if (g.a_rows && g.a_rows[m] < 0) continue;
         float o = acc[mi][ni][v] + b;
-        if (DUAL) o = silu_f(o) * acc2[mi][ni][v];
+        if (DUAL) o = gate_fn(o, g.gate) * acc2[mi][ni][v];
         store_out<OUT_ACT>(g, m, n, o);
       }
   }
@@ -682,16 +681,16 @@ TQ_API int tq_gemm_mfma_splits(int M, int N, int K) {
 TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gather, const void* w, const void* w2,
                         int64_t group_stride, const int* tile_group, const int* n_tiles, const void* bias,
                         int bias_type, void* out, int64_t ldc, int out_is_act, int M, int N, int K, int tile_rows,
-                        int splits, hipStream_t st) {
+                        int splits, int gate, hipStream_t st) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || K % 8 != 0 || lda % 8 != 0) return TQ_ERR_BAD_ARG;
   if (((uintptr_t)a | (uintptr_t)w | (uintptr_t)w2) % 16 != 0 || (group_stride % 8) != 0) return TQ_ERR_BAD_ARG;
   const bool dual = w2 != nullptr, out_act = out_is_act != 0;
-  if (splits < 1 || splits > 64) return TQ_ERR_BAD_ARG;
+  if (splits < 1 || splits > 64 || gate < 0 || gate >= TQ_GATE_COUNT) return TQ_ERR_BAD_ARG;
   if (splits > 1 && (dual || out_act || tile_group || a_rows || splits != tq_gemm_mfma_splits(M, N, K))) return TQ_ERR_BAD_ARG;
   const int k_per = ((K + TBK - 1) / TBK + splits - 1) / splits * TBK;
   MfmaGemmArgs g{(const bf16_t*)a, lda, a_rows, a_gather, (const bf16_t*)w, (const bf16_t*)w2, group_stride,
-                 tile_group, n_tiles, bias, bias_type, out, ldc, M, N, K, splits > 1 ? k_per : K, (int64_t)M * ldc};
+                 tile_group, n_tiles, bias, bias_type, out, ldc, M, N, K, splits > 1 ? k_per : K, (int64_t)M * ldc, gate};
   int rc = 0;
   if (tile_group) {
     if (tile_rows == 16) {
@@ -744,8 +743,8 @@ TQ_API int tq_gemm_mfma_pair_splits(int N1, int K1, int grouped1, int N2, int K2
   return (K2 + k_per - 1) / k_per;
 }
 
-// Two products of few rows in one launch.  d1, d2: 18 numbers each, in the order of tq_gemm_mfma's arguments from
-// `a` to `tile_rows`.  Both must be products that the streaming kernel takes 16 rows at a time (a matrix per
+// Two products of few rows in one launch.  d1, d2: 19 numbers each, in the order of tq_gemm_mfma's arguments from
+// `a` to `tile_rows`, then the gate's activation.  Both must be products that the streaming kernel takes 16 rows at a time (a matrix per
 // expert with tile_rows 16, or one matrix with M <= 16), both gated or both not, both into the same type.  The
 // waves that split k are those of the first product (the larger one by convention).  splits2 > 1 (as
 // tq_gemm_mfma_pair_splits says, for a plain second product into float): run z of its k goes to
@@ -762,7 +761,8 @@ TQ_API int tq_gemm_mfma_pair(const int64_t* d1, const int64_t* d2, int splits2, 
     if (((uintptr_t)p[0] | (uintptr_t)p[4] | (uintptr_t)p[5]) % 16 != 0) return TQ_ERR_BAD_ARG;
     g[i] = MfmaGemmArgs{(const bf16_t*)p[0], p[1], (const int*)p[2], (int)p[3], (const bf16_t*)p[4], (const bf16_t*)p[5],
                         p[6], (const int*)p[7], (const int*)p[8], (const void*)p[9], (int)p[10], (void*)p[11], p[12],
-                        M, N, K, K, 0};
+                        M, N, K, K, 0, (int)p[18]};
+    if (g[i].gate < 0 || g[i].gate >= TQ_GATE_COUNT) return TQ_ERR_BAD_ARG;
     dual[i] = p[5] != 0;
     out_act[i] = p[13] != 0;
     if (g[i].tile_group) {

@@ -21,6 +21,7 @@ class KernelError(RuntimeError):
 
 
 ACT_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+GATES = {"silu": 0, "gelu_tanh": 1, "relu2": 2}      # activations of the gate in a gated pair of products
 _WTYPE = {torch.float32: 0, torch.bfloat16: 1}
 _LIBS: dict[str, ctypes.CDLL] = {}
 
@@ -35,7 +36,7 @@ _SIGNATURES = {
                          _c_ptr],
     "tq_moe_combine": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
     "tq_gemm_generic": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int,
-                        _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+                        _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "tq_attention_generic": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_i64, _c_int, _c_int,
                              _c_int, _c_int, _c_int, _c_f32, _c_ptr, _c_ptr],
     "tq_router_topk": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
@@ -48,10 +49,12 @@ _SIGNATURES = {
     "tq_sample_topp_scratch": [_c_int],
     "tq_sample_topp": [_c_ptr, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
 }
-# entry points that only the bfloat16 library has
+# entry points that only one of the two libraries has
 _OPTIONAL = {
+    "tq_gemm_f32": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int,
+                    _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "tq_gemm_mfma": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int,
-                     _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+                     _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "tq_gemm_mfma_splits": [_c_int, _c_int, _c_int],
     "tq_gemm_mfma_pair_splits": [_c_int, _c_int, _c_int, _c_int, _c_int, _c_int],
     "tq_gemm_mfma_pair": [_c_ptr, _c_ptr, _c_int, _c_ptr],
@@ -366,11 +369,24 @@ def _gemm_problem(k: str, a, w, act, bias, w2, out_act, a_rows, tile_group, n_ti
     return M, N, K, tile_rows, gstride
 
 
+def _gate_code(k: str, activation: str) -> int:
+    _need(activation in GATES, k, f"unknown activation {activation!r}; known: {', '.join(sorted(GATES))}")
+    return GATES[activation]
+
+
+def _use_f32(act, a: torch.Tensor, w: torch.Tensor, K: int, gstride: int) -> bool:
+    """The float matrix-core product takes float operands whose rows start at multiples of 16 bytes."""
+    return (dtype_name(act) == "float32" and w.dtype == torch.float32 and a.dtype == torch.float32 and K % 4 == 0
+            and a.stride(0) % 4 == 0 and gstride % 4 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+            and has_kernel(act, "tq_gemm_f32"))
+
+
 def gemm(a: torch.Tensor, w: torch.Tensor, act, bias: torch.Tensor | None = None, w2: torch.Tensor | None = None,
          out_act: bool = False, a_rows: torch.Tensor | None = None, tile_group: torch.Tensor | None = None,
          n_tiles: torch.Tensor | None = None, tile_rows: int | None = None, gather: bool = True,
-         partial_sums: bool = False) -> torch.Tensor:
-    """out[m, n] = sum_k a[row(m), k] * w[g, n, k]  (+ bias[n]);  with ``w2``: silu(a w^T) * (a w2^T).
+         partial_sums: bool = False, activation: str = "silu") -> torch.Tensor:
+    """out[m, n] = sum_k a[row(m), k] * w[g, n, k]  (+ bias[n]);  with ``w2``: f(a w^T) * (a w2^T), f being the
+    ``activation`` (silu, gelu_tanh or relu2).
 
     ``a`` [M, K] activations.  ``w`` [N, K], or [G, N, K] with ``tile_group`` naming the matrix of each tile of
     ``tile_rows`` output rows and ``a_rows`` [P] the row of ``a`` behind each output row (-1: none; with
@@ -388,6 +404,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, act, bias: torch.Tensor | None = None
         _need(w2 is None and not out_act and not grouped and a_rows is None, k,
               "partial sums are for plain products into float32")
     lib = library(act)
+    gate = _gate_code(k, activation)
     if _use_mfma(act, a, w, K) and (bias is None or bias.dtype in _WTYPE):
         splits = lib.tq_gemm_mfma_splits(M, N, K) if partial_sums else 1
         out = torch.empty((splits, M, N) if partial_sums else (M, N), dtype=adt if out_act else torch.float32,
@@ -395,13 +412,19 @@ def gemm(a: torch.Tensor, w: torch.Tensor, act, bias: torch.Tensor | None = None
         _run("gemm_mfma", lib.tq_gemm_mfma(_ptr(a), a.stride(0), _ptr(a_rows), int(gather), _ptr(w), _ptr(w2), gstride,
                                            _ptr(tile_group), _ptr(n_tiles), _ptr(bias),
                                            _WTYPE[bias.dtype] if bias is not None else 0, _ptr(out), N, int(out_act),
-                                           M, N, K, tile_rows, splits, _stream()))
+                                           M, N, K, tile_rows, splits, gate, _stream()))
         return out
     out = torch.empty((1, M, N) if partial_sums else (M, N), dtype=adt if out_act else torch.float32, device=a.device)
+    if _use_f32(act, a, w, K, gstride) and (w2 is None or w2.data_ptr() % 16 == 0):
+        _run("gemm_f32", lib.tq_gemm_f32(_ptr(a), a.stride(0), _ptr(a_rows), int(gather), _ptr(w), _ptr(w2), gstride,
+                                         _ptr(tile_group), _ptr(n_tiles), _ptr(bias),
+                                         _WTYPE[bias.dtype] if bias is not None else 0, _ptr(out), N, M, N, K, tile_rows,
+                                         gate, _stream()))
+        return out
     _run(k, lib.tq_gemm_generic(_ptr(a), a.stride(0), _ptr(a_rows), int(gather), _ptr(w), _ptr(w2), _WTYPE[w.dtype], gstride,
                                 _ptr(tile_group), _ptr(n_tiles), _ptr(bias),
                                 _WTYPE[bias.dtype] if bias is not None else 0, _ptr(out), N, int(out_act), M, N, K,
-                                tile_rows, _stream()))
+                                tile_rows, gate, _stream()))
     return out
 
 
@@ -411,12 +434,12 @@ def gemm_pair(first: dict, second: dict, act) -> tuple[torch.Tensor, torch.Tenso
     the same type) go out in one launch, so that the smaller one costs no launch of its own; anything else is two
     calls."""
     k = "gemm_pair"
-    keys = ("bias", "w2", "out_act", "a_rows", "tile_group", "n_tiles", "tile_rows", "gather", "partial_sums")
+    keys = ("bias", "w2", "out_act", "a_rows", "tile_group", "n_tiles", "tile_rows", "gather", "partial_sums", "activation")
     probs = []
     _need(not first.get("partial_sums", False), k, "only the second product may leave partial sums")
     for p in (first, second):
         full = {"bias": None, "w2": None, "out_act": False, "a_rows": None, "tile_group": None, "n_tiles": None,
-                "tile_rows": None, "gather": True, "partial_sums": False}
+                "tile_rows": None, "gather": True, "partial_sums": False, "activation": "silu"}
         _need(set(p) <= set(full) | {"a", "w"}, k, f"unknown arguments {sorted(set(p) - set(full) - {'a', 'w'})}")
         full.update(p)
         probs.append(full)
@@ -447,8 +470,9 @@ def gemm_pair(first: dict, second: dict, act) -> tuple[torch.Tensor, torch.Tenso
         outs.append(out)
         vals = [_ptr(p["a"]), p["a"].stride(0), _ptr(p["a_rows"]), int(p["gather"]), _ptr(p["w"]), _ptr(p["w2"]), gstride,
                 _ptr(p["tile_group"]), _ptr(p["n_tiles"]), _ptr(p["bias"]),
-                _WTYPE[p["bias"].dtype] if p["bias"] is not None else 0, _ptr(out), N, int(p["out_act"]), M, N, K, tile_rows]
-        descs.append((ctypes.c_int64 * 18)(*[0 if v is None else int(v) for v in vals]))
+                _WTYPE[p["bias"].dtype] if p["bias"] is not None else 0, _ptr(out), N, int(p["out_act"]), M, N, K, tile_rows,
+                _gate_code(k, p["activation"])]
+        descs.append((ctypes.c_int64 * 19)(*[0 if v is None else int(v) for v in vals]))
     _run(k, lib.tq_gemm_mfma_pair(descs[0], descs[1], splits, _stream()))
     return outs[0], outs[1]
 

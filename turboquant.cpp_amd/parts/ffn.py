@@ -1,6 +1,8 @@
 """Feed-forward parts: a dense gated one and a sparse one with routed experts and a shared expert.
 
-Dense (/root/reference/src/engine/tq_transformer.c:2707-2824): ``down(silu(gate x) * (up x))``, no biases.
+Dense (/root/reference/src/engine/tq_transformer.c:2707-2824): ``down(silu(gate x) * (up x))``, no biases; the
+gate's activation is an argument (``silu``, ``gelu_tanh`` as /root/reference/src/engine/tq_ops.c:1482-1484, ``relu2``)
+that the products' epilogues take.
 Sparse (/root/reference/src/engine/tq_moe.c:600-1059): router logits in float32, top-k with the highest index
 winning ties, weights from a softmax; every chosen expert is the dense formula with its own matrices, summed
 with its weight in the order chosen; the shared expert, scaled by ``sigmoid(x . shared_scale)``, is added
@@ -20,8 +22,10 @@ class DenseSwiGLU(Part):
     graph_safe = True
     wants_f32 = False
 
-    def __init__(self, hidden_size: int, inner_size: int):
-        self.hidden_size, self.inner_size = hidden_size, inner_size
+    def __init__(self, hidden_size: int, inner_size: int, activation: str = "silu"):
+        if activation not in ops.GATES:
+            raise ValueError(f"unknown activation {activation!r}; known: {', '.join(sorted(ops.GATES))}")
+        self.hidden_size, self.inner_size, self.activation = hidden_size, inner_size, activation
         self.gate = self.up = self.down = None
 
     def param_specs(self):
@@ -30,7 +34,7 @@ class DenseSwiGLU(Part):
                 "down": ParamSpec((self.hidden_size, self.inner_size))}
 
     def forward(self, normed, normed32, ctx):
-        h = ops.gemm(normed, self.gate, ctx.act, w2=self.up, out_act=True)
+        h = ops.gemm(normed, self.gate, ctx.act, w2=self.up, out_act=True, activation=self.activation)
         return ops.gemm(h, self.down, ctx.act, partial_sums=True)
 
 
@@ -40,9 +44,12 @@ class SparseMoE(Part):
     wants_f32 = True    # the router reads the normalised activations in float32
 
     def __init__(self, hidden_size: int, num_experts: int, top_k: int, expert_size: int, shared_size: int = 0,
-                 shared_gated: bool = True, renormalize: bool = False):
+                 shared_gated: bool = True, renormalize: bool = False, activation: str = "silu"):
         if not 1 <= top_k <= num_experts:
             raise ValueError(f"top_k {top_k} must be within 1..num_experts {num_experts}")
+        if activation not in ops.GATES:
+            raise ValueError(f"unknown activation {activation!r}; known: {', '.join(sorted(ops.GATES))}")
+        self.activation = activation
         self.hidden_size, self.num_experts, self.top_k = hidden_size, num_experts, top_k
         self.expert_size, self.shared_size = expert_size, shared_size
         self.shared_gated, self.renormalize = shared_gated and shared_size > 0, renormalize
@@ -70,8 +77,10 @@ class SparseMoE(Part):
             # a handful of tokens: the shared expert's two products ride in the launches of the routed experts'
             _, weights, gate, sorted_token, pair_slot, tile_expert, n_tiles = route()
             experts = dict(a_rows=sorted_token, tile_group=tile_expert, n_tiles=n_tiles, tile_rows=unit)
-            h, hs = ops.gemm_pair(dict(a=normed, w=self.expert_gate, w2=self.expert_up, out_act=True, **experts),
-                                  dict(a=normed, w=self.shared_gate, w2=self.shared_up, out_act=True), ctx.act)
+            h, hs = ops.gemm_pair(dict(a=normed, w=self.expert_gate, w2=self.expert_up, out_act=True,
+                                       activation=self.activation, **experts),
+                                  dict(a=normed, w=self.shared_gate, w2=self.shared_up, out_act=True,
+                                       activation=self.activation), ctx.act)
             y, shared = ops.gemm_pair(dict(a=h, w=self.expert_down, gather=False, **experts),
                                       dict(a=hs, w=self.shared_down, partial_sums=True), ctx.act)
             return ops.GatheredSum(y, pair_slot, weights, shared, gate)
@@ -90,7 +99,7 @@ class SparseMoE(Part):
                 shared = self._shared(normed, ctx)
         _, weights, gate, sorted_token, pair_slot, tile_expert, n_tiles = route()
         h = ops.gemm(normed, self.expert_gate, ctx.act, w2=self.expert_up, out_act=True, a_rows=sorted_token,
-                     tile_group=tile_expert, n_tiles=n_tiles, tile_rows=unit)
+                     tile_group=tile_expert, n_tiles=n_tiles, tile_rows=unit, activation=self.activation)
         y = ops.gemm(h, self.expert_down, ctx.act, a_rows=sorted_token, tile_group=tile_expert, n_tiles=n_tiles,
                      tile_rows=unit, gather=False)
         if side is not None:
@@ -99,5 +108,5 @@ class SparseMoE(Part):
         return ops.GatheredSum(y, pair_slot, weights, shared, gate)
 
     def _shared(self, normed, ctx):
-        hs = ops.gemm(normed, self.shared_gate, ctx.act, w2=self.shared_up, out_act=True)
+        hs = ops.gemm(normed, self.shared_gate, ctx.act, w2=self.shared_up, out_act=True, activation=self.activation)
         return ops.gemm(hs, self.shared_down, ctx.act, partial_sums=True)
