@@ -4,6 +4,11 @@
 
 A step is one decode step of the whole batch: the step function, greedy sampling on the GPU and the copy of the
 chosen tokens to the host, exactly what the generation loop runs.  Prints one JSON line.
+
+    python bench.py --sizes a14b --workload unequal         # 8 prompts of 512 to 4,096 tokens, then 256 decode steps
+    python bench.py --dtype float32 --workload unequal      # true 32-bit: 64 prompts of 1 to 2,048 tokens, 64 steps
+
+time the other two workloads: a batch of prompts of unequal lengths in one prompt step, then decode steps.
 """
 from __future__ import annotations
 
@@ -125,6 +130,14 @@ def main() -> int:
                          "each, greedy and with the default sampling (temperature 0.7, top-p 0.9, repetition penalty)")
     ap.add_argument("--probe", action="store_true",
                     help="no model: what this GPU reaches on a plain read of memory and on the matrix instructions alone")
+    ap.add_argument("--workload", default="steps", choices=["steps", "unequal"],
+                    help="unequal: a batch of prompts of unequal lengths in one prompt step, then decode steps "
+                         "(defaults per model: a14b 8 prompts of 512..4096, seed 3, 256 steps; float32 64 prompts of "
+                         "1..2048, seed 4, 64 steps)")
+    ap.add_argument("--prompt-min", type=int, default=None)
+    ap.add_argument("--prompt-max", type=int, default=None)
+    ap.add_argument("--decode-steps", type=int, default=None)
+    ap.add_argument("--seed", type=int, default=None)
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single device)")
@@ -144,12 +157,18 @@ def main() -> int:
     cfg["num_hidden_layers"] = args.layers
     cfg["max_window_layers"] = args.layers
     cfg["max_position_embeddings"] = max(args.context, args.points_context, PREFILL_TOKENS)
+    if args.workload == "unequal":
+        big = args.sizes == "a14b"
+        wl = {"batch": args.batch if args.batch != 8 or big else 64,
+              "lo": args.prompt_min or (512 if big else 1), "hi": args.prompt_max or (4096 if big else 2048),
+              "steps": args.decode_steps or (256 if big else 64), "seed": args.seed if args.seed is not None else (3 if big else 4)}
+        cfg["max_position_embeddings"] = wl["hi"] + wl["steps"] + 64
     act = args.dtype
     short = "bf16" if act == "bfloat16" else "fp32"
     dev = "cuda:0"
     ops.library(act)
     t0 = time.time()
-    model = random_model(cfg, seed=2, act=act, device=dev)
+    model = random_model(cfg, seed=wl["seed"] if args.workload == "unequal" else 2, act=act, device=dev)
     torch.cuda.synchronize()
     print(f"[bench] {args.layers}-layer model with random weights on the device in {time.time() - t0:.1f}s "
           f"({model.weight_bytes / 1e9:.1f} GB)", file=sys.stderr, flush=True)
@@ -173,6 +192,87 @@ def main() -> int:
             n = sum(len(r.tokens) for r in res)
             out[name] = {"value": round(n / dt, 1), "tokens": n, "seconds": round(dt, 3)}
         print(json.dumps(out))
+        return 0
+
+    wbytes = 2 if act == "bfloat16" else 4
+
+    def count_experts(fn):
+        """Runs fn() (an eager decode step) and returns the mean number of distinct experts a layer's router picked."""
+        picked = []
+        route = ops.route
+
+        def counting_route(*a, **k):
+            out = route(*a, **k)
+            picked.append(int(torch.unique(out[0]).numel()))
+            return out
+
+        ops.route = counting_route
+        try:
+            result = fn()
+        finally:
+            ops.route = route
+        return result, sum(picked) / max(len(picked), 1)
+
+    if args.workload == "unequal":
+        B = wl["batch"]
+        g = torch.Generator().manual_seed(wl["seed"])
+        lens = torch.randint(wl["lo"], wl["hi"] + 1, (B,), generator=g).tolist()
+        prompts = [torch.randint(0, V, (n,), generator=g).tolist() for n in lens]
+        page = 64
+        engine = Engine(model, max_tokens=sum(-(-(n + wl["steps"] + 1) // page) * page for n in lens), page_size=page, max_slots=B)
+        fetch = TokenFetch(dev, B)
+        best = None
+        for rep in range(2):                  # the first pass loads kernels and captures the decode graphs
+            slots = engine.open(B)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            logits = engine.step(slots, prompts)
+            torch.cuda.synchronize()
+            t_prompt = time.perf_counter() - t0
+            tokens = ops.argmax(logits, act)
+            used = None
+            t0 = time.perf_counter()
+            for i in range(wl["steps"]):
+                fetch.start(tokens)
+                if rep == 1 and i == 0:       # an eager step of the timed pass also counts the experts that are read
+                    graphs, engine.graphs = engine.graphs, None
+                    lg, used = count_experts(lambda: engine.step_from_device(slots, tokens))
+                    engine.graphs = graphs
+                else:
+                    lg = engine.step_from_device(slots, tokens)
+                fetch.wait()
+                tokens = ops.argmax(lg, act)
+            torch.cuda.synchronize()
+            t_decode = time.perf_counter() - t0
+            engine.close(slots)
+            best = (t_prompt, t_decode, used)
+        t_prompt, t_decode, used = best
+        T = sum(lens)
+        sec = t_decode / wl["steps"]
+        mean_total_ctx = T + B * (wl["steps"] + 1) / 2.0
+        read = decode_bytes(cfg, args.layers, B, mean_total_ctx / B, wbytes, used)
+        flops = sum(prefill_flops(cfg, args.layers, n, 0) for n in lens) + 2.0 * B * cfg["hidden_size"] * V
+        out = {
+            "metric": f"decode tok/s, batch {B} of unequal prompts ({wl['lo']}..{wl['hi']} tokens), {wl['steps']} steps "
+                      f"({model_name} layer sizes, random weights)",
+            "value": round(B / sec, 1), "unit": "tok/s", "n_gpus": 1, "steps": wl["steps"], "warmup": 0,
+            "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": short, "data": "synthetic",
+            "config": {"model": f"{model_name} sizes", "layers": args.layers, "layers_of_full_model": full_layers,
+                       "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
+                       "head_dim": cfg["hidden_size"] // cfg["num_attention_heads"], "vocab": V, "experts": cfg["num_experts"],
+                       "top_k": cfg["num_experts_per_tok"], "expert_inner": cfg["moe_intermediate_size"],
+                       "shared_inner": cfg["shared_expert_intermediate_size"], "global_batch": B,
+                       "prompt_tokens": T, "longest_prompt": max(lens), "shortest_prompt": min(lens),
+                       "weights": f"random N(0,0.02) seed {wl['seed']}", "kv_cache": short,
+                       "experts_read_per_layer": round(used, 1), "parallelism": "single GPU"},
+            "prefill": {"value": round(T / t_prompt, 1), "tokens": T, "ms": round(t_prompt * 1e3, 3),
+                        "frac": round(flops / t_prompt / PEAK_FLOPS[short], 4)},
+            "roofline": {"bound": "hbm", "achieved": round(read / sec / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                         "frac": round(read / sec / 1e9 / PEAK_HBM_GBS, 4)},
+            "decode": {"ms_total": round(t_decode * 1e3, 2), "gb_per_step": round(read / 1e9, 2)},
+        }
+        print(json.dumps(out), flush=True)
         return 0
 
     def run_decode(batch: int, context: int, steps: int, warmup: int):
@@ -203,20 +303,7 @@ def main() -> int:
             return ops.argmax(lg, act)
 
         # the first warm-up step (which runs eagerly) also counts the distinct experts that each layer's router picks
-        picked = []
-        route = ops.route
-
-        def counting_route(*a, **k):
-            out = route(*a, **k)
-            picked.append(int(torch.unique(out[0]).numel()))
-            return out
-
-        ops.route = counting_route
-        try:
-            tokens = one_step(tokens)
-        finally:
-            ops.route = route
-        experts_used = sum(picked) / max(len(picked), 1)
+        tokens, experts_used = count_experts(lambda: one_step(tokens))
         for _ in range(warmup - 1):
             tokens = one_step(tokens)
         torch.cuda.synchronize()
@@ -257,13 +344,25 @@ def main() -> int:
         return 0
     sec, mean_ctx, experts_used = run_decode(args.batch, args.context, args.steps, args.warmup)
     value = args.batch / sec
-    read = decode_bytes(cfg, args.layers, args.batch, mean_ctx, 2 if act == "bfloat16" else 4, experts_used)
+    read = decode_bytes(cfg, args.layers, args.batch, mean_ctx, wbytes, experts_used)
     achieved = read / sec / 1e9
-    points = {}
+
+    def point(b, ctx, s, mean, used):
+        gb = decode_bytes(cfg, args.layers, b, mean, wbytes, used) / 1e9
+        return {"tok_s": round(b / s, 1), "ms_per_step": round(s * 1e3, 4), "gb_per_step": round(gb, 2),
+                "frac": round(gb / s / PEAK_HBM_GBS, 4)}
+
+    # decode at batch 1 and 64 at the headline context, and every batch at the shorter context too
+    points, detail = {}, {f"decode_b{args.batch}_ctx{args.context}": point(args.batch, args.context, sec, mean_ctx, experts_used)}
     if not args.no_points:
         for b in (1, 64):
-            s, _, _ = run_decode(b, args.points_context, 32, 4)
+            s, mean, used = run_decode(b, args.context, 32, 4)
             points[f"decode_b{b}"] = round(b / s, 1)
+            detail[f"decode_b{b}_ctx{args.context}"] = point(b, args.context, s, mean, used)
+        if args.points_context != args.context:
+            for b in sorted({1, args.batch, 64}):
+                s, mean, used = run_decode(b, args.points_context, 32, 4)
+                detail[f"decode_b{b}_ctx{args.points_context}"] = point(b, args.points_context, s, mean, used)
     out = {
         "metric": f"decode tok/s at batch {args.batch}, context {args.context} ({model_name} layer sizes, random weights)",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -284,6 +383,7 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4)},
         "points": points,
+        "points_detail": detail,
     }
     print(json.dumps(out), flush=True)
     return 0

@@ -15,8 +15,12 @@ import torch
 ACT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 
 
-def embed(tokens, table, act):
-    return table[tokens.long()].float()
+def embed(tokens, table, act, scale=1.0):
+    return table[tokens.long()].float() * scale
+
+
+def softcap(logits, cap, act):
+    return logits.copy_(cap * torch.tanh(logits / cap))
 
 
 def add_rmsnorm(x, delta, weight, eps, act, rows=None, want_act=True, want_f32=False):
@@ -226,5 +230,5 @@ def install(monkeypatch):
     """Puts the stand-ins in place of the kernels for one test."""
     from turboquant_cpp_amd.csrc import ops
     for name in ("embed", "add_rmsnorm", "rope_kv_write", "qkv_rope_write", "attention", "gemm", "router_topk", "moe_align", "route", "gemm_pair",
-                 "moe_combine", "argmax", "rep_penalty", "sample_topp"):
+                 "moe_combine", "argmax", "rep_penalty", "sample_topp", "softcap"):
         monkeypatch.setattr(ops, name, globals()[name])

@@ -241,7 +241,7 @@ def test_two_products_in_one_launch(ops, act, gated):
 @pytest.mark.parametrize("act", ACTS)
 def test_second_product_of_a_pair_in_runs_of_k(ops, act):
     """The experts' down products (short k) beside a plain product with a long k whose partial sums are wanted
-    apart: the second one comes in several runs of k (bfloat16: 8 here, and as many whatever the number of rows),
+    apart: the second one comes in several runs of k (as many whatever the number of rows),
     their sum is the product, the bias is counted once, and the first product keeps the bits it has alone."""
     E, I, H, k, S = 5, 512, 264, 2, 4104
     shapes = set()
@@ -265,7 +265,8 @@ def test_second_product_of_a_pair_in_runs_of_k(ops, act):
         scale = ref2.abs().max().item()
         lim = 1e-5 * scale * math.sqrt(S) if act == "float32" else 4e-3 * scale
         assert (y2.cpu().double().sum(0) - ref2).abs().max().item() < lim
-    assert shapes == ({8} if act == "bfloat16" else {1})
+    # as many runs whatever the number of rows: 8 in bfloat16; in float32 what the plain product's own rule gives
+    assert len(shapes) == 1 and (shapes == {8} or act == "float32")
 
 
 @pytest.mark.parametrize("act", ACTS)
@@ -581,14 +582,14 @@ def test_attention_finds_a_far_key(ops, act):
     assert (out_w2.float().view(nh, hd) - v[far].to(adt(act)).float()).abs().max() < 1e-2
 
 
+@pytest.mark.parametrize("act", ACTS)
 @pytest.mark.parametrize("window", [None, 3000])
-def test_decoding_over_long_caches(ops, window):
+def test_decoding_over_long_caches(ops, act, window):
     """One token per sequence at positions on both sides of the length at which the split kernel changes the
     length of its runs (4096), of other multiples of 2048 and well beyond, in one batch: the sequences of 3,500 and
     4,095 tokens have more runs (one per 64 positions) than the longest one (one per 192), after which the grid is
     sized.  In each sequence one far key stands out a little, so that a run that is skipped or joined twice shows.
     Against the plain formula for the last token."""
-    act = "bfloat16"
     nh, nkv, hd, page = 6, 2, 64, 64
     lens = [2047, 2048, 2049, 4095, 4097, 6143, 6145, 9001, 130, 3500]
     table, slots, page_stride, kp, vp = paged_setup(lens, page, nkv, hd, 1, act, 95)
@@ -623,7 +624,7 @@ def test_decoding_over_long_caches(ops, window):
                         torch.tensor(slots, dtype=torch.int32).to(DEV), table.to(DEV), page, page_stride, nh, nkv, hd,
                         window, scale, act, runs=runs).cpu()
     err = (out.double() - torch.stack(want)).abs().max(dim=1).values
-    assert err.max() < 2e-2, err
+    assert err.max() < (2e-5 if act == "float32" else 2e-2), err
     # each sequence alone gives the same bits: what a run is depends on the token's position only
     for i in (1, 3, 4, 7):
         runs1 = {"cu_seqlens": torch.tensor([0, 1], dtype=torch.int32).to(DEV), "slots": torch.tensor([slots[i]], dtype=torch.int32).to(DEV),
@@ -761,11 +762,14 @@ def test_sample_topp_distribution(ops):
                                                      (16, 16, 128, None, 64), (40, 2, 32, 200, 64), (2, 1, 256, None, 64),
                                                      (5, 5, 96, 1, 64), (8, 2, 64, 100, 64),
                                                      # enough heads for two token groups per wave
-                                                     (48, 6, 128, None, 64), (48, 4, 64, 100, 64), (44, 4, 48, 30, 64)])
-def test_attention_tiled(ops, nh, nkv, hd, window, page):
-    """The matrix-core kernels (whole runs of tokens, and one token per sequence split over the cache) against the
-    plain attention: unequal lengths, a sequence that goes on from a cached prefix, groups of more than 16 heads."""
-    act = "bfloat16"
+                                                     (48, 6, 128, None, 64), (48, 4, 64, 100, 64), (44, 4, 48, 30, 64),
+                                                     # head sizes that are a multiple of 4 only (the 32-bit kernels take them)
+                                                     (6, 2, 24, 24, 64), (3, 3, 20, None, 64)])
+@pytest.mark.parametrize("act", ACTS)
+def test_attention_tiled(ops, act, nh, nkv, hd, window, page):
+    """The matrix-core kernels of both types (whole runs of tokens, and one token per sequence split over the cache)
+    against the plain attention: unequal lengths, a sequence that goes on from a cached prefix, groups of more than
+    16 heads."""
     lens = [1, 19, 150, 333]
     layers, layer = 3, 1
     table, slots, page_stride, kp, vp = paged_setup(lens, page, nkv, hd, layers, act, 130)

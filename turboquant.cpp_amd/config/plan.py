@@ -69,9 +69,13 @@ class ModelPlan:
     lm_head: Source | None          # None: tied to the embedding
     max_positions: int
     stop_tokens: tuple[int, ...] = ()
+    embedding_scale: float = 1.0            # the embedding rows are multiplied by it
+    logit_softcap: float | None = None      # logits <- cap * tanh(logits / cap)
 
     def validate(self) -> None:
         n = len(self.layers)
+        if self.logit_softcap is not None and not self.logit_softcap > 0:
+            raise ValueError(f"logit_softcap must be positive, got {self.logit_softcap}")
         for i, e in enumerate(self.schedule):
             if not 0 <= e.layer < n:
                 raise ValueError(f"schedule entry {i} names layer {e.layer}, model has {n}")

@@ -19,7 +19,7 @@ CSRC = os.path.dirname(os.path.abspath(__file__))
 # sources per activation type: each has matrix-core kernels of its own
 COMMON_SOURCES = ["elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "moe.hip", "sampling.hip"]
 SOURCES = {
-    "float32": COMMON_SOURCES + ["gemm_f32.hip"],
+    "float32": COMMON_SOURCES + ["gemm_f32.hip", "attention_f32.hip"],
     "bfloat16": COMMON_SOURCES + ["gemm_mfma.hip", "attention_mfma.hip", "probe.hip"],
 }
 HEADERS = ["common.h", "no_alloc.h"]

@@ -4,20 +4,40 @@
 #include "common.h"
 
 // ---------------------------------------------------------------- embedding
-// x[t, :] = table[tokens[t], :] widened to float, no scaling
-// (/root/reference/src/engine/tq_transformer.c:2297-2329).
+// x[t, :] = table[tokens[t], :] widened to float; no scaling for this architecture
+// (/root/reference/src/engine/tq_transformer.c:2297-2329); `scale` other than 1 multiplies the row, for the
+// architectures that scale their embeddings (tq_transformer.c:2332).
 template <class W>
 __global__ void embed_kernel(const int* __restrict__ tokens, const W* __restrict__ table,
-                             float* __restrict__ x, int H) {
+                             float* __restrict__ x, int H, float scale) {
   const int t = blockIdx.x;
   const W* row = table + (size_t)tokens[t] * H;
   float* out = x + (size_t)t * H;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = to_f32(row[i]);
+  if (scale == 1.0f) {
+    for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = to_f32(row[i]);
+  } else {
+    for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = to_f32(row[i]) * scale;
+  }
 }
 
-TQ_API int tq_embed(const int* tokens, const void* table, int wtype, float* x, int T, int H, hipStream_t st) {
+TQ_API int tq_embed(const int* tokens, const void* table, int wtype, float* x, int T, int H, float scale, hipStream_t st) {
   if (T <= 0) return 0;
-  TQ_DISPATCH_W(wtype, { hipLaunchKernelGGL(embed_kernel<W>, dim3(T), dim3(256), 0, st, tokens, (const W*)table, x, H); });
+  TQ_DISPATCH_W(wtype, { hipLaunchKernelGGL(embed_kernel<W>, dim3(T), dim3(256), 0, st, tokens, (const W*)table, x, H, scale); });
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------- a soft cap on logits
+// x <- cap * tanh(x / cap), in place: what a model plan may ask for between the vocabulary product and sampling.
+__global__ void softcap_kernel(float* __restrict__ x, int64_t n, float cap) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) x[i] = cap * tanhf(x[i] / cap);
+}
+
+TQ_API int tq_softcap(float* x, int64_t n, float cap, hipStream_t st) {
+  if (n <= 0) return 0;
+  if (!(cap > 0.f)) return TQ_ERR_BAD_ARG;
+  hipLaunchKernelGGL(softcap_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, x, n, cap);
   TQ_LAUNCH_CHECK();
   return 0;
 }

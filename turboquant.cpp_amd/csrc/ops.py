@@ -28,7 +28,8 @@ _LIBS: dict[str, ctypes.CDLL] = {}
 _c_int, _c_i64, _c_f32, _c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
 
 _SIGNATURES = {
-    "tq_embed": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr],
+    "tq_embed": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_f32, _c_ptr],
+    "tq_softcap": [_c_ptr, _c_i64, _c_f32, _c_ptr],
     "tq_add_rmsnorm": [_c_ptr, _c_ptr, _c_int, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_f32,
                        _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr],
     "tq_rope_kv_write": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
@@ -52,7 +53,11 @@ _SIGNATURES = {
 # entry points that only one of the two libraries has
 _OPTIONAL = {
     "tq_gemm_f32": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int,
-                    _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+                    _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_ptr],
+    "tq_gemm_f32_runs": [_c_int, _c_int, _c_int, _c_int],
+    "tq_attention_f32_scratch": [_c_int, _c_int, _c_int, _c_int],
+    "tq_attention_f32": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int,
+                         _c_int, _c_int, _c_int, _c_f32, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "tq_gemm_mfma": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int,
                      _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "tq_gemm_mfma_splits": [_c_int, _c_int, _c_int],
@@ -102,8 +107,9 @@ def library(dtype) -> ctypes.CDLL:
             f = getattr(lib, fn)
             f.argtypes, f.restype = sig, _c_int
     lib.tq_sample_topp_scratch.restype = _c_i64
-    if hasattr(lib, "tq_attention_decode_scratch"):
-        lib.tq_attention_decode_scratch.restype = _c_i64
+    for fn in ("tq_attention_decode_scratch", "tq_attention_f32_scratch"):
+        if hasattr(lib, fn):
+            getattr(lib, fn).restype = _c_i64
     _LIBS[name] = lib
     return lib
 
@@ -146,16 +152,25 @@ def _run(kernel: str, code: int) -> None:
 
 
 # ------------------------------------------------------------------ row-wise kernels
-def embed(tokens: torch.Tensor, table: torch.Tensor, act) -> torch.Tensor:
-    """x[t] = table[tokens[t]] as float32 [T, H]."""
+def embed(tokens: torch.Tensor, table: torch.Tensor, act, scale: float = 1.0) -> torch.Tensor:
+    """x[t] = table[tokens[t]] (times ``scale``) as float32 [T, H]."""
     k = "embed"
     _check(tokens, k, "tokens", torch.int32)
     _need(tokens.dim() == 1 and table.dim() == 2, k, "tokens [T], table [V, H]")
     _check(table, k, "table", tuple(_WTYPE))
     T, (V, H) = tokens.numel(), table.shape
     x = torch.empty((T, H), dtype=torch.float32, device=table.device)
-    _run(k, library(act).tq_embed(_ptr(tokens), _ptr(table), _WTYPE[table.dtype], _ptr(x), T, H, _stream()))
+    _run(k, library(act).tq_embed(_ptr(tokens), _ptr(table), _WTYPE[table.dtype], _ptr(x), T, H, float(scale), _stream()))
     return x
+
+
+def softcap(logits: torch.Tensor, cap: float, act) -> torch.Tensor:
+    """logits <- cap * tanh(logits / cap), in place."""
+    k = "softcap"
+    _check(logits, k, "logits", torch.float32)
+    _need(cap > 0, k, "the cap must be positive")
+    _run(k, library(act).tq_softcap(_ptr(logits), logits.numel(), float(cap), _stream()))
+    return logits
 
 
 @dataclasses.dataclass
@@ -414,13 +429,20 @@ def gemm(a: torch.Tensor, w: torch.Tensor, act, bias: torch.Tensor | None = None
                                            _WTYPE[bias.dtype] if bias is not None else 0, _ptr(out), N, int(out_act),
                                            M, N, K, tile_rows, splits, gate, _stream()))
         return out
-    out = torch.empty((1, M, N) if partial_sums else (M, N), dtype=adt if out_act else torch.float32, device=a.device)
     if _use_f32(act, a, w, K, gstride) and (w2 is None or w2.data_ptr() % 16 == 0):
+        # a narrow matrix times few rows is cut into runs of k: they come back apart if the caller adds them up
+        # anyway, else they pass through scratch memory and a second kernel
+        runs = lib.tq_gemm_f32_runs(M, N, K, int(grouped or a_rows is not None))
+        out = torch.empty((runs, M, N) if partial_sums else (M, N), dtype=torch.float32, device=a.device)
+        scratch = None
+        if runs > 1 and not partial_sums:
+            scratch = torch.empty((runs * (2 if w2 is not None else 1), M, N), dtype=torch.float32, device=a.device)
         _run("gemm_f32", lib.tq_gemm_f32(_ptr(a), a.stride(0), _ptr(a_rows), int(gather), _ptr(w), _ptr(w2), gstride,
                                          _ptr(tile_group), _ptr(n_tiles), _ptr(bias),
                                          _WTYPE[bias.dtype] if bias is not None else 0, _ptr(out), N, M, N, K, tile_rows,
-                                         gate, _stream()))
+                                         gate, _ptr(scratch), int(partial_sums and runs > 1), _stream()))
         return out
+    out = torch.empty((1, M, N) if partial_sums else (M, N), dtype=adt if out_act else torch.float32, device=a.device)
     _run(k, lib.tq_gemm_generic(_ptr(a), a.stride(0), _ptr(a_rows), int(gather), _ptr(w), _ptr(w2), _WTYPE[w.dtype], gstride,
                                 _ptr(tile_group), _ptr(n_tiles), _ptr(bias),
                                 _WTYPE[bias.dtype] if bias is not None else 0, _ptr(out), N, int(out_act), M, N, K,
@@ -517,6 +539,24 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, lay
             partial = torch.empty((lib.tq_attention_decode_scratch(B, num_heads, head_dim, int(runs["max_end"])),),
                                   dtype=torch.float32, device=q.device)
         _run("attention_mfma", lib.tq_attention_mfma(
+            _ptr(q), k_pages.data_ptr() + layer_offset * esz, v_pages.data_ptr() + layer_offset * esz,
+            _ptr(block_table), block_table.shape[1], _ptr(runs["cu_seqlens"]), _ptr(runs["slots"]), _ptr(runs["start"]),
+            page_size, page_stride, B, num_heads, num_kv_heads, head_dim, int(window or 0), float(scale), _ptr(out),
+            _ptr(partial), int(bool(runs["decode"])), int(runs["max_new"]), int(runs["max_end"]), _stream()))
+        return out
+    if (runs is not None and dtype_name(act) == "float32" and hasattr(lib, "tq_attention_f32") and head_dim % 4 == 0
+            and head_dim <= 256 and page_size % 64 == 0 and page_stride % 4 == 0 and layer_offset % 4 == 0):
+        B = runs["slots"].numel()
+        _check(runs["cu_seqlens"], k, "cu_seqlens", torch.int32, (B + 1,))
+        _check(runs["slots"], k, "slots", torch.int32, (B,))
+        _check(runs["start"], k, "start", torch.int32, (B,))
+        _need(runs["max_end"] <= block_table.shape[1] * page_size, k, "positions reach beyond the page table")
+        partial = None
+        if runs["decode"]:
+            _need(T == B, k, "decoding brings one token per sequence")
+            partial = torch.empty((lib.tq_attention_f32_scratch(B, num_heads, head_dim, int(runs["max_end"])),),
+                                  dtype=torch.float32, device=q.device)
+        _run("attention_f32", lib.tq_attention_f32(
             _ptr(q), k_pages.data_ptr() + layer_offset * esz, v_pages.data_ptr() + layer_offset * esz,
             _ptr(block_table), block_table.shape[1], _ptr(runs["cu_seqlens"]), _ptr(runs["slots"]), _ptr(runs["start"]),
             page_size, page_stride, B, num_heads, num_kv_heads, head_dim, int(window or 0), float(scale), _ptr(out),

@@ -112,14 +112,17 @@ class CausalLM:
     def forward(self, ctx: StepContext) -> torch.Tensor:
         """Runs the step's tokens through the schedule; returns float32 logits [wanted rows, vocab]."""
         b = ctx.batch
-        x = ops.embed(b.tokens, self.embedding, self.act)
+        x = ops.embed(b.tokens, self.embedding, self.act, scale=self.plan.embedding_scale)
         pending = None
         for entry, e in enumerate(self.schedule):
             pending = self.blocks[e.layer].forward(x, pending, ctx, entry)
         if b.n_want == 0:
             return torch.empty((0, self.plan.vocab_size), dtype=torch.float32, device=x.device)
         normed, _ = self.final_norm.forward(x, pending, ctx, rows=b.want_rows)
-        return ops.gemm(normed, self.lm_head, self.act)
+        logits = ops.gemm(normed, self.lm_head, self.act)
+        if self.plan.logit_softcap is not None:
+            ops.softcap(logits, self.plan.logit_softcap, self.act)
+        return logits
 
 
 # ---------------------------------------------------------------- construction

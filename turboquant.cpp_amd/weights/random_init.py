@@ -27,7 +27,7 @@ from .safetensors_io import SafetensorsWriter
 
 _FILE_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32, "float16": torch.float16}
 _GAMMA = 0x9E3779B97F4A7C15
-_CHUNK = 1 << 24          # elements drawn at a time: bounds the 64-bit temporaries
+_CHUNK = {"cpu": 1 << 22, "cuda": 1 << 27}      # elements drawn at a time: bounds the 64-bit temporaries
 
 
 def _signed(v: int) -> int:
@@ -82,8 +82,9 @@ def random_tensor(index: int, shape, role: str, seed: int, std: float, norm_std:
         out.fill_(shift)
         return out.view(tuple(shape))
     key = tensor_key(seed, index)
-    for first in range(0, numel, _CHUNK):
-        n = min(_CHUNK, numel - first)
+    chunk = _CHUNK[torch.device(device).type]
+    for first in range(0, numel, chunk):
+        n = min(chunk, numel - first)
         v = standard_normal(key, first, n, device) * scale
         if shift:
             v += shift
