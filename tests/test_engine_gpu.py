@@ -555,6 +555,8 @@ def test_a_mixer_with_state_of_its_own_is_registered_built_and_stepped():
     H, V, INNER, L = 48, 90, 64, 2
 
     class ToyDecayMixer(Part):
+        graph_safe = True          # its decode steps reach the state through the slots on the device
+
         def __init__(self, hidden_size, decay):
             self.hidden_size, self.decay = hidden_size, decay
             self.w_in = self.w_out = None
@@ -569,10 +571,14 @@ def test_a_mixer_with_state_of_its_own_is_registered_built_and_stepped():
             return StateNeed((self.hidden_size,), torch.float32)
 
         def forward(self, normed, ctx, entry):
-            state = ctx.state(entry)                               # [slots, H]; zero for a new sequence
             u = normed.float() @ self.w_in.float().T
-            out = torch.empty_like(u)
             b = ctx.batch
+            if b.is_decode:                                        # one token per sequence: advance every state by one
+                s = self.decay * ctx.state_rows(entry) + u
+                ctx.store_state_rows(entry, s)
+                return (s @ self.w_out.float().T).unsqueeze(0)
+            state = ctx.state(entry)                               # [slots, H]; zero for a new sequence
+            out = torch.empty_like(u)
             o = 0
             for slot, n in zip(b.slots, b.n_new):                  # a scan over each sequence's new tokens
                 s = state[slot]
@@ -602,6 +608,7 @@ def test_a_mixer_with_state_of_its_own_is_registered_built_and_stepped():
         model.load(TensorDict(tensors), DEV)
         eng = Engine(model, max_tokens=64 * 4, max_slots=3)
         assert eng.cache.groups == [] and sorted(eng.cache.states) == [0, 1]
+        assert eng.graphs.replayable(2)
 
         def plain(tokens):
             import plain_qwen2moe as P
@@ -638,6 +645,18 @@ def test_a_mixer_with_state_of_its_own_is_registered_built_and_stepped():
                 eng.close([slots[i]])
                 live.remove(i)
         assert eng.cache.n_live == 0
+        assert len(eng.graphs.graphs) >= 1, "the decode steps of the stateful mixer were not replayed"
+        # replayed steps give the bits of eager ones, with other slots behind the same graph
+        slow = Engine(model, max_tokens=64 * 4, max_slots=3, use_graphs=False)
+        for order in ([0, 2], [2, 0]):
+            sf, ss = eng.open(3), slow.open(3)
+            for e, sl in ((eng, sf), (slow, ss)):
+                e.step([sl[i] for i in order], [prompts[i][:4] for i in order], [[], []])
+            for t in range(4, 9):
+                a = eng.step([sf[i] for i in order], [[prompts[i][t]] for i in order])
+                b_ = slow.step([ss[i] for i in order], [[prompts[i][t]] for i in order])
+                assert torch.equal(a, b_), f"replayed step {t} differs from the eager one"
+            eng.close(sf), slow.close(ss)
     finally:
         unregister_part("mixer", "toy_decay")
 
@@ -709,7 +728,7 @@ def test_a_feed_forward_with_routing_and_another_position_encoding_defined_here(
                    for n, (s, role) in model.tensor_table().items()}
         model.load(TensorDict(tensors), DEV)
         eng = Engine(model, max_tokens=64 * 6, max_slots=3)
-        assert eng.graphs is None          # parts that do not declare themselves safe for replay switch it off
+        assert not eng.graphs.replayable(2) and not eng.graphs.graphs   # parts that do not say they are safe for replay keep their model's steps eager
         assert len(eng.cache.groups) == 2  # the windowed layer has storage of its own
 
         def turn(x, angles_per_step, pairing, rot):      # x [T, heads, hd]
@@ -760,6 +779,112 @@ def test_a_feed_forward_with_routing_and_another_position_encoding_defined_here(
     finally:
         unregister_part("position", "toy_linear")
         unregister_part("ffn", "toy_one_of_four")
+
+
+def test_a_mixer_that_keeps_one_row_per_position_and_a_scaled_embedding_with_capped_logits():
+    """A toy mixer defined here that keeps a single latent row per position (keys only, no value pool: ``value_dim``
+    0) and attends over those rows, in a model whose plan scales the embedding and soft-caps the logits; the dense
+    feed-forward takes another activation than silu.  None of this touches the framework's files."""
+    import plain_qwen2moe as P
+    from turboquant_cpp_amd.config import LayerSpec, ModelPlan, PartSpec, ScheduleEntry, Source
+    from turboquant_cpp_amd.engine.model import CausalLM
+    from turboquant_cpp_amd.engine.step import Engine
+    from turboquant_cpp_amd.parts import CacheNeed, ParamSpec, Part, register_part, unregister_part
+    from turboquant_cpp_amd.weights import TensorDict
+
+    H, V, LAT, INNER, L = 40, 60, 24, 56, 2
+    SCALE, CAP = 3.0, 2.5
+
+    class ToyLatentMixer(Part):
+        def __init__(self, hidden_size, latent):
+            self.hidden_size, self.latent = hidden_size, latent
+            self.w_q = self.w_c = self.w_o = None
+
+        def param_specs(self):
+            return {"w_q": ParamSpec((self.latent, self.hidden_size)), "w_c": ParamSpec((self.latent, self.hidden_size)),
+                    "w_o": ParamSpec((self.hidden_size, self.latent))}
+
+        def cache_need(self):
+            return CacheNeed(1, self.latent, None, value_dim=0)
+
+        def state_need(self):
+            return None
+
+        def forward(self, normed, ctx, entry):
+            kv, b = ctx.kv(entry), ctx.batch
+            assert kv.v_pages is None and kv.value_dim == 0
+            x = normed.float()
+            q, c = x @ self.w_q.float().T, x @ self.w_c.float().T
+            table = kv.table.cpu()
+            pages = kv.k_pages.view(-1, kv.page_stride)
+            out, o = torch.empty_like(q), 0
+            for slot, start, n in zip(b.slots, b.start, b.n_new):
+                for j in range(n):                     # the new rows go into the sequence's pages
+                    pos = start + j
+                    off = kv.layer_offset + (pos % kv.page_size) * self.latent
+                    pages[int(table[slot, pos // kv.page_size]), off:off + self.latent] = c[o + j].to(pages.dtype)
+                rows = torch.stack([pages[int(table[slot, p // kv.page_size]),
+                                          kv.layer_offset + (p % kv.page_size) * self.latent:][:self.latent]
+                                    for p in range(start + n)]).float()
+                for j in range(n):
+                    seen = rows[:start + j + 1]
+                    out[o + j] = torch.softmax(seen @ q[o + j] / self.latent ** 0.5, dim=0) @ seen
+                o += n
+            return (out @ self.w_o.float().T).unsqueeze(0)
+
+    register_part("mixer", "toy_latent")(ToyLatentMixer)
+    try:
+        def norm(name):
+            return PartSpec("rmsnorm", dict(size=H, eps=1e-6), {"weight": Source.single(name)})
+        layers = [LayerSpec("prenorm", {
+            "mixer_norm": norm(f"l{l}.n1"), "ffn_norm": norm(f"l{l}.n2"),
+            "mixer": PartSpec("toy_latent", dict(hidden_size=H, latent=LAT),
+                              {n: Source.single(f"l{l}.{n}") for n in ("w_q", "w_c", "w_o")}),
+            "ffn": PartSpec("dense_swiglu", dict(hidden_size=H, inner_size=INNER, activation="gelu_tanh"),
+                            {n: Source.single(f"l{l}.{n}") for n in ("gate", "up", "down")})}) for l in range(L)]
+        plan = ModelPlan("ToyLatentLM", V, H, layers, [ScheduleEntry(l) for l in range(L)], norm("final"),
+                         Source.single("embed"), None, max_positions=256, embedding_scale=SCALE, logit_softcap=CAP)
+        model = CausalLM(plan, "float32")
+        g = torch.Generator().manual_seed(90)
+        tensors = {n: (torch.ones(s) if role == "scale" else 0.3 * torch.randn(s, generator=g))
+                   for n, (s, role) in model.tensor_table().items()}
+        model.load(TensorDict(tensors), DEV)
+        eng = Engine(model, max_tokens=64 * 6, max_slots=3)
+        (group,) = eng.cache.groups
+        assert group.v_pages is None and group.key.value_dim == 0 and group.page_stride == L * 64 * LAT
+        assert eng.cache.bytes() == group.k_pages.numel() * 4
+
+        def plain(tokens):
+            t = {n: v.double() for n, v in tensors.items()}
+            x = SCALE * t["embed"][tokens]
+            T = len(tokens)
+            for l in range(L):
+                xb = P.rmsnorm(x, t[f"l{l}.n1"], 1e-6)
+                q, c = xb @ t[f"l{l}.w_q"].T, xb @ t[f"l{l}.w_c"].T
+                att = torch.stack([torch.softmax(c[:i + 1] @ q[i] / LAT ** 0.5, dim=0) @ c[:i + 1] for i in range(T)])
+                x = x + att @ t[f"l{l}.w_o"].T
+                xb = P.rmsnorm(x, t[f"l{l}.n2"], 1e-6)
+                gate = torch.nn.functional.gelu(xb @ t[f"l{l}.gate"].T, approximate="tanh")
+                x = x + (gate * (xb @ t[f"l{l}.up"].T)) @ t[f"l{l}.down"].T
+            logits = P.rmsnorm(x, t["final"], 1e-6) @ t["embed"].T
+            return CAP * torch.tanh(logits / CAP)
+
+        prompts = [torch.randint(0, V, (n,), generator=g).tolist() for n in (70, 3, 21)]
+        refs = [plain(p) for p in prompts]
+        assert max(r.abs().max() for r in refs) > 0.8 * CAP          # the cap bites
+        slots = eng.open(3)
+        lg = eng.step(slots, prompts, [list(range(len(p))) for p in prompts]).cpu().double()
+        assert (lg - torch.cat(refs)).abs().max() < 2e-4
+        eng.close(slots)
+        slots = eng.open(2)                    # a prefix, then token by token, in slots and pages that were used before
+        eng.step(slots, [prompts[0][:60], prompts[2][:9]], [[], []])
+        for i in range(8):
+            lg = eng.step(slots, [[prompts[0][60 + i]], [prompts[2][9 + i]]]).cpu().double()
+            assert (lg[0] - refs[0][60 + i]).abs().max() < 2e-4 and (lg[1] - refs[2][9 + i]).abs().max() < 2e-4
+        eng.close(slots)
+        assert eng.cache.n_live == 0 and group.pool.n_free == group.pool.n_pages
+    finally:
+        unregister_part("mixer", "toy_latent")
 
 
 def test_a_capture_is_not_disturbed_by_garbage_of_earlier_engines(engines, sharp_dirs):

@@ -103,13 +103,23 @@ class DecodeGraphs:
         self.graphs: dict[tuple[int, int], DecodeGraph] = {}
         self.seen: set[tuple[int, int]] = set()
         self.pool = None
+        self._replayable: dict[int, bool] = {}
+
+    def replayable(self, n_seqs: int) -> bool:
+        """Whether every part of the model lets a decode step of ``n_seqs`` sequences be captured."""
+        if n_seqs not in self._replayable:
+            self._replayable[n_seqs] = all(p.replayable(n_seqs) for p in self.engine.model.parts())
+        return self._replayable[n_seqs]
 
     def key(self, n_seqs: int, max_end: int) -> tuple[int, int]:
         cap = self.engine.cache.max_positions
         return n_seqs, min(cap, -(-max_end // RUN_BUCKET) * RUN_BUCKET)
 
     def run(self, slots, starts, tokens):
-        """Logits [B, vocab] of one decode step, or None if this shape has not been seen before."""
+        """Logits [B, vocab] of one decode step, or None if this shape has not been seen before or a part of the
+        model does not let it be replayed."""
+        if not self.replayable(len(slots)):
+            return None
         key = self.key(len(slots), max(starts) + 1)
         g = self.graphs.get(key)
         if g is not None:

@@ -36,7 +36,8 @@ class Engine:
         # decode steps are replayed as HIP graphs where a GPU runs them
         on_gpu = self.device is not None and self.device.type == "cuda"
         self.side_stream = torch.cuda.Stream(device=self.device) if on_gpu else None     # default priority
-        self.graphs = DecodeGraphs(self) if use_graphs and on_gpu and all(p.graph_safe for p in model.parts()) else None
+        # (which shapes of step are replayed is the parts' word, asked shape by shape: Part.replayable)
+        self.graphs = DecodeGraphs(self) if use_graphs and on_gpu else None
 
     # ------------------------------------------------------------ sequences
     def open(self, n: int = 1) -> list[int]:

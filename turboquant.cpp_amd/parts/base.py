@@ -12,7 +12,9 @@ Interfaces (``ctx`` is the :class:`~..engine.context.StepContext` of the running
             rows in the activation type (and in float32 if asked).
 * mixer     ``forward(normed, ctx, entry) -> delta``: mixes tokens of each sequence; ``entry`` is the index of
             the schedule entry that runs, by which it finds its cache (``ctx.kv(entry)``) or its fixed-size
-            state (``ctx.state(entry)``).  ``cache_need()`` / ``state_need()`` say what storage each run wants.
+            state (``ctx.state(entry)``; ``ctx.state_rows(entry)`` / ``ctx.store_state_rows(entry, rows)`` read and
+            write the rows of the step's sequences through the slots on the device, which a decode step that is to
+            be replayed must use).  ``cache_need()`` / ``state_need()`` say what storage each run wants.
 * ffn       ``forward(normed, normed32, ctx) -> delta``; ``wants_f32`` says whether it reads the float32 copy.
 * position  ``table(device)``, ``pairing``, ``rotary_dim``: the rotation a mixer applies to queries and keys.
 * block     ``forward(x, pending, ctx, entry) -> pending``: the arrangement of norms, mixer and ffn around
@@ -66,10 +68,16 @@ class StateNeed:
 class Part:
     category: str = ""
     kind: str = ""
-    # True if forward() reads what changes from step to step (tokens, positions, slots, lengths) from the
-    # batch's device arrays only, so that a captured launch sequence can be replayed for other sequences.
-    # Decode steps of a model are replayed as graphs only if all its parts say so.
+    # True if forward(), in a decode step (one token per sequence), reads what changes from step to step (tokens,
+    # positions, slots, lengths) from the batch's device arrays only and launches nothing that a stream capture
+    # cannot record, so that a captured launch sequence can be replayed for other sequences.
     graph_safe: bool = False
+
+    def replayable(self, n_seqs: int) -> bool:
+        """Whether a decode step of ``n_seqs`` sequences may be captured and replayed as far as this part goes.  The
+        engine asks every part before it captures a step of a shape; one that says no makes steps of that shape run
+        eagerly, others are still replayed."""
+        return self.graph_safe
 
     def param_specs(self) -> dict[str, ParamSpec]:
         return {}
