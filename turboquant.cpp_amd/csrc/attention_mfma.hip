@@ -513,7 +513,7 @@ template <int DT, int QG, bool EXACT>
 static int launch_prefill(const AttnArgs& a, int B, int max_new, hipStream_t st) {
   const size_t shmem = 2 * (EXACT ? (size_t)2 * TILE * a.hd : (size_t)TILE * (a.hd + KPAD) + (size_t)a.hd * VSTR) * sizeof(bf16_t);
   if (shmem > 48 * 1024)
-    hipFuncSetAttribute((const void*)attn_prefill_kernel<DT, QG, EXACT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+    (void)hipFuncSetAttribute((const void*)attn_prefill_kernel<DT, QG, EXACT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
   const int n_blocks = (max_new + 64 * QG - 1) / (64 * QG);
   if ((int64_t)n_blocks * a.nh * B > 0x7fffffff) return TQ_ERR_UNSUPPORTED;
   hipLaunchKernelGGL((attn_prefill_kernel<DT, QG, EXACT>), dim3(n_blocks * a.nh * B), dim3(256), shmem, st, a, n_blocks, B);

@@ -22,7 +22,7 @@ SOURCES = {
     "float32": COMMON_SOURCES + ["gemm_f32.hip", "attention_f32.hip"],
     "bfloat16": COMMON_SOURCES + ["gemm_mfma.hip", "attention_mfma.hip", "probe.hip"],
 }
-HEADERS = ["common.h", "no_alloc.h"]
+HEADERS = ["common.h", "no_alloc.h", "gemm_mfma.h"]
 DEFINES = {"float32": "-DTQ_ACT_F32", "bfloat16": "-DTQ_ACT_BF16"}
 FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-fno-gpu-rdc",
          # keep the compiler from forming packed 32-bit float instructions
@@ -108,19 +108,24 @@ def build(dtype: str, force: bool = False, verbose: bool = True) -> str:
     for src in sources:
         obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
         cmd = [hipcc, *FLAGS, DEFINES[dtype], "-c", os.path.join(CSRC, src), "-o", obj]
-        procs.append((src, obj, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        # what the compiler prints goes to a file: a pipe that nobody reads while the compilers run together
+        # would block the one that fills it
+        log = open(obj + ".log", "w+")
+        procs.append((src, obj, subprocess.Popen(cmd, stdout=log, stderr=subprocess.STDOUT), log))
     objs = []
     pending = list(procs)
     last = time.time()
     while pending:
         for item in list(pending):
-            src, obj, p = item
+            src, obj, p, log = item
             if p.poll() is None:
                 continue
-            out = p.stdout.read()
+            log.seek(0)
+            out = log.read()
+            log.close()
             pending.remove(item)
             if p.returncode != 0:
-                for _, _, q in pending:
+                for _, _, q, _ in pending:
                     q.kill()
                 raise BuildError(f"hipcc failed on {src}:\n{out}")
             say(f"  compiled {src} ({time.time() - t0:.0f}s)")
@@ -128,7 +133,7 @@ def build(dtype: str, force: bool = False, verbose: bool = True) -> str:
         if pending:
             time.sleep(0.2)
             if time.time() - last > 10:
-                say(f"  still compiling: {', '.join(s for s, _, _ in pending)} ({time.time() - t0:.0f}s)")
+                say(f"  still compiling: {', '.join(s for s, _, _, _ in pending)} ({time.time() - t0:.0f}s)")
                 last = time.time()
     tmp = target + f".tmp{os.getpid()}"
     link = subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *sorted(objs), "-o", tmp],

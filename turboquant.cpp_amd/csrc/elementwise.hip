@@ -196,7 +196,7 @@ TQ_API int tq_add_rmsnorm(float* x, const float* delta, int S, int64_t delta_str
   if (shmem > 150 * 1024) return TQ_ERR_UNSUPPORTED;
   TQ_DISPATCH_W(wtype, {
     if (shmem > 48 * 1024)
-      hipFuncSetAttribute((const void*)add_rmsnorm_kernel<W>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+      (void)hipFuncSetAttribute((const void*)add_rmsnorm_kernel<W>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
     hipLaunchKernelGGL(add_rmsnorm_kernel<W>, dim3(R), dim3(threads), shmem, st, x, delta, S, (size_t)delta_stride, y,
                        pair_slot, weights, topk, gate, (const W*)w, eps, rows, (act_t*)out, out32, H);
   });
@@ -352,7 +352,7 @@ TQ_API int tq_rope_kv_write(const float* qkv, const int* positions, const int* s
   TQ_LAUNCH_CHECK();
   if (tiles) {
     if (vt_shmem > 48 * 1024)
-      hipFuncSetAttribute((const void*)v_write_tile_kernel<VEC>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)vt_shmem);
+      (void)hipFuncSetAttribute((const void*)v_write_tile_kernel<VEC>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)vt_shmem);
     hipLaunchKernelGGL(v_write_tile_kernel<VEC>, dim3((max_new + VT_POS - 1) / VT_POS + 1, nkv, B), dim3(256), vt_shmem,
                        st, qkv, cu_seqlens, slots, start, block_table, bt_stride, (act_t*)v_pool, page_size,
                        page_stride, nh, nkv, hd);

@@ -224,7 +224,7 @@ static int launch_router_logits(const float* x, const void* wr, const void* shar
 #define TQ_ROUTER(TGV, RWV)                                                                                         \
   do {                                                                                                              \
     if (shmem > 48 * 1024)                                                                                          \
-      hipFuncSetAttribute((const void*)router_logits_kernel<W, TGV, RWV>,                                           \
+      (void)hipFuncSetAttribute((const void*)router_logits_kernel<W, TGV, RWV>,                                           \
                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);                                  \
     hipLaunchKernelGGL((router_logits_kernel<W, TGV, RWV>), dim3(groups, row_groups), dim3(256), shmem, st, x,      \
                        (const W*)wr, (const W*)shared_w, rows, E, logits, T, H);                                    \
@@ -410,7 +410,7 @@ TQ_API int tq_moe_align(const int* ids, int n_pairs, int E, int topk, int unit, 
   const size_t shmem = (size_t)(AW + 1) * E * sizeof(int);
   if (shmem > 160 * 1024) return TQ_ERR_UNSUPPORTED;
   if (shmem > 48 * 1024)
-    hipFuncSetAttribute((const void*)moe_align_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+    (void)hipFuncSetAttribute((const void*)moe_align_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
   hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(64 * AW), shmem, st, ids, n_pairs, E, topk, unit, cap,
                      sorted_token, pair_slot, tile_expert, n_tiles);
   TQ_LAUNCH_CHECK();
@@ -440,7 +440,7 @@ TQ_API int tq_route(const float* x, const void* wr, const void* shared_w, int wt
     return 0;
   }
   if (shmem > 48 * 1024)
-    hipFuncSetAttribute((const void*)select_align_kernel<AW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+    (void)hipFuncSetAttribute((const void*)select_align_kernel<AW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
   hipLaunchKernelGGL(select_align_kernel<AW>, dim3(1), dim3(64 * AW), shmem, st, logits, E + (shared_w ? 1 : 0), E, topk,
                      renorm, ids, weights, shared_gate, T, unit, cap, sorted_token, pair_slot, tile_expert, n_tiles);
   TQ_LAUNCH_CHECK();
