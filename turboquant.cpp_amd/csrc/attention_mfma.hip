@@ -412,8 +412,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 // writes their unnormalised sums with maximum and denominator.  The grid has the runs of the step's longest
 // sequence, so that no wave is started for nothing where all sequences are about as long (a wave that finds no run
 // costs as much to start as one that does: a third more of them made the kernel a fifth slower).  A shorter
-// sequence of the same step may still have more runs than that, positions below 4096 being cut finer: the wave of
-// the grid's last run then takes all of the sequence's further runs, one after the other, each into its own place.
+// sequence of the same step may still have more runs than that, positions below 4096 being cut finer: its waves
+// then take the further runs in turn (wave x the runs x, x + the grid's runs, ...), each into its own place, so
+// that no wave has more than one or two of them (left to the last wave alone, 30 runs in a row made a step with
+// one sequence beyond position 4096 and seven shorter ones a third slower).
 template <int DT, bool EXACT>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DT > 8 ? 2 : 3))) void attn_decode_kernel(AttnArgs a) {
   const int b = blockIdx.z;
@@ -433,8 +435,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DT > 8 ? 2 :
 
   bf16x8 qf[1][(DT + 1) / 2];
   load_query<DT>(qf[0], a.q + ((size_t)t * a.nh + h) * a.hd, a.hd, valid);
-  const int run_end = blockIdx.x + 1 == gridDim.x ? n_runs : (int)blockIdx.x + 1;
-  for (int run = blockIdx.x; run < run_end; ++run) {
+  for (int run = blockIdx.x; run < n_runs; run += gridDim.x) {
     const int tile_beg = max(run * S, lo / TILE), tile_end = min((run + 1) * S, p / TILE + 1);
     if (tile_beg >= tile_end) continue;       // all of the run lies before the window
     f32x4 o[1][DT];
