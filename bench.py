@@ -277,7 +277,7 @@ def main() -> int:
 
     def run_decode(batch: int, context: int, steps: int, warmup: int):
         """Prefills `batch` prompts so that the timed steps end at `context`, then times `steps` decode steps."""
-        prompt_len = context - steps - warmup - 1
+        prompt_len = context - steps - warmup
         page = 64
         per_seq = -(-context // page) * page
         engine = Engine(model, max_tokens=per_seq * batch, page_size=page, max_slots=batch)
@@ -307,12 +307,18 @@ def main() -> int:
         for _ in range(warmup - 1):
             tokens = one_step(tokens)
         torch.cuda.synchronize()
+        held = lambda: sum(engine.cache.length(s) for s in slots) / batch
+        before = held()
         t = time.perf_counter()
         for _ in range(steps):
             tokens = one_step(tokens)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
-        mean_ctx = prompt_len + warmup + steps / 2.0
+        # what a timed step read on average, from the cache's own count of positions: a step that finds L positions
+        # writes one and reads L + 1; the first timed step finds `before`, the last one leaves `context`
+        mean_ctx = (before + 1 + held()) / 2.0
+        if held() != context or before != context - steps:
+            raise RuntimeError(f"the timed steps ran from {before} to {held()} positions, not up to {context}")
         engine.close(slots)
         del engine
         torch.cuda.empty_cache()

@@ -39,3 +39,37 @@ def test_operations_of_a_prompt_step_at_the_headline_sizes():
     assert abs(total - 8.87e12) < 0.03e12
     one_more_row = bench.prefill_flops(c, 24, 2048, rows_out=2) - total
     assert one_more_row == 2 * 2048 * 151936
+
+
+import json  # noqa: E402
+
+import pytest  # noqa: E402
+
+
+@pytest.mark.gpu
+def test_the_line_of_a_short_run_on_the_gpu():
+    """One layer, a few steps: the line has the contract's keys, a flat configuration of at most 20 keys, and figures
+    that fit each other (tokens a second and milliseconds a step; bytes a step, time and rate; a context that the
+    timed steps really ended at, which bench.py checks against the cache and refuses to print otherwise)."""
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--layers", "1", "--steps", "6", "--warmup", "2",
+                        "--batch", "3", "--context", "330", "--points-context", "330", "--no-points"],
+                       capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    line = json.loads(r.stdout.strip().splitlines()[-1])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "prefill", "roofline", "points"):
+        assert key in line, key
+    assert line["n_gpus"] == 1 and line["steps"] == 6 and line["warmup"] == 2 and line["dtype"] == "bf16"
+    cfg = line["config"]
+    assert len(cfg) <= 20 and all(not isinstance(v, (dict, list)) for v in cfg.values())
+    assert cfg["layers"] == 1 and cfg["layers_of_full_model"] == 24 and cfg["global_batch"] == 3 and cfg["seq_len"] == 330
+    assert abs(line["value"] - 3 / (line["ms_per_step"] * 1e-3)) < 0.01 * line["value"]
+    roof = line["roofline"]
+    assert roof["bound"] == "hbm" and roof["peak"] == 8000.0 and abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-3
+    detail = line["points_detail"]["decode_b3_ctx330"]
+    # the bytes of a step at the mean context of the timed steps: they find 324 .. 329 positions and read one more
+    want = bench.decode_bytes(bench.SIZES["a27b"][0], 1, 3, (324 + 1 + 330) / 2.0, 2, cfg["experts_read_per_layer"]) / 1e9
+    assert abs(detail["gb_per_step"] - want) < 0.01 * want
+    assert abs(roof["achieved"] - detail["gb_per_step"] / (line["ms_per_step"] * 1e-3)) < 0.01 * roof["achieved"]
+    pre = line["prefill"]
+    assert pre["tokens"] == 2048 and abs(pre["value"] - 2048 / (pre["ms"] * 1e-3)) < 0.01 * pre["value"] and 0 < pre["frac"] < 1

@@ -811,11 +811,34 @@ def test_attention_tiled(ops, act, nh, nkv, hd, window, page):
 
 
 def test_probes_run(ops):
-    """The two kernels behind `bench.py --probe` (a plain read, the matrix instructions alone) launch and finish;
-    the second reports how many operations it did."""
-    buf = torch.arange(1 << 20, dtype=torch.int32, device=DEV)
+    """The two kernels behind `bench.py --probe` (a plain read, the matrix instructions alone) do the work they are
+    timed for: the read of 256 MiB takes at least as long as the memory's published rate allows and no longer
+    than a tenth of it would, and the matrix loop stays below the published peak and above a tenth of it.  A
+    kernel whose loop the compiler had emptied, or that read a fraction of the buffer, would be too fast."""
+    def seconds(fn):
+        fn()
+        torch.cuda.synchronize()
+        best = 1e9
+        for _ in range(3):
+            t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            t0.record()
+            fn()
+            t1.record()
+            torch.cuda.synchronize()
+            best = min(best, t0.elapsed_time(t1) * 1e-3)
+        return best
+
+    buf = torch.arange(1 << 26, dtype=torch.int32, device=DEV)
+    nbytes = buf.numel() * 4
     for once in (False, True):
-        ops.probe_stream(buf, once)
+        rate = nbytes / seconds(lambda: ops.probe_stream(buf, once))
+        assert 0.8e12 < rate < 8.0e12 * 1.05, (once, rate)
     assert ops.probe_mfma(32, 4, 10, 1, DEV) == 4 * 8 * 10 * 196608.0
-    assert ops.probe_mfma(16, 4, 10, 0, DEV) == 4 * 8 * 10 * 196608.0
-    torch.cuda.synchronize()
+    for shape in (32, 16):
+        flop = [0.0]
+
+        def run():
+            flop[0] = ops.probe_mfma(shape, 512, 2000, 12345, DEV)
+        t = seconds(run)
+        rate = flop[0] / t
+        assert 0.25e15 < rate < 2.5e15 * 1.02, (shape, rate)
