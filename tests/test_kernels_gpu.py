@@ -637,6 +637,21 @@ def test_decoding_over_long_caches(ops, act, window):
 
 # ------------------------------------------------------------------------------------------------ sampling
 @pytest.mark.parametrize("V", [10, 1000, 151937])
+def test_negative_log_likelihood(ops, V):
+    """-log softmax at a given token, per row, against float64; a row with one towering logit (no overflow), and a
+    target that is no token (NaN, for the caller to leave out)."""
+    logits = rnd((5, V), torch.float32, 98, 3.0)
+    logits[1, V // 2] = 300.0
+    logits[2] = -1000.0
+    targets = torch.tensor([0, V // 2, V - 1, V, -1], dtype=torch.int32)
+    out = ops.nll(logits.to(DEV), targets.to(DEV), "float32").cpu().double()
+    ref = -torch.log_softmax(logits.double(), dim=-1)
+    for r in range(3):
+        assert abs(out[r] - ref[r, int(targets[r])]) < 1e-5 * max(1.0, float(ref[r, int(targets[r])])), r
+    assert torch.isnan(out[3]) and torch.isnan(out[4])
+
+
+@pytest.mark.parametrize("V", [10, 1000, 151937])
 def test_argmax_first_maximum(ops, V):
     logits = rnd((3, V), torch.float32, 100)
     logits[1, V // 3] = logits[1, V - 1] = 50.0          # equal maxima: the first wins

@@ -178,6 +178,39 @@ def test_the_command_line_generates(act, sharp):
     assert info.returncode == 0 and "Qwen2MoeForCausalLM" in info.stdout
 
 
+@pytest.mark.parametrize("act", ACTS)
+def test_the_command_line_scores_a_file_of_tokens(act, sharp, tmp_path):
+    """``bin/quant DIR --ppl FILE --json`` (the reference's teacher-forced perplexity, /root/reference/tools/quant.c:430-720):
+    700 tokens in steps of 512, one of them outside the vocabulary and so never a target; against the plain model's
+    mean negative log-likelihood over the same targets.  ``--tokens-file`` gives the prompts of ``-p``."""
+    d, plain, _ = sharp("B", act)
+    (ids,) = prompts_for("B", [700], seed=28)
+    ids[300] = 10 ** 6
+    f = tmp_path / "tokens.txt"
+    f.write_text(" ".join(str(t) for t in ids[:350]) + "\n" + ",".join(str(t) for t in ids[350:]) + "\n")
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "quant"), d, "--ppl", str(f), "--json", "--dtype", act, "--ctx", "1024"]
+    run = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr[-2000:]
+    res = json.loads(run.stdout)
+    fed = [t if t < 10 ** 6 else 0 for t in ids]
+    logp = torch.log_softmax(plain.logits(fed).double(), dim=-1)
+    targets = [(i, ids[i + 1]) for i in range(len(ids) - 1) if ids[i + 1] < 10 ** 6]
+    want = -sum(float(logp[i, t]) for i, t in targets) / len(targets)
+    assert res["tokens"] == 700 and res["tokens_evaluated"] == 698 == len(targets)
+    assert abs(res["avg_nll"] - want) < (1e-4 if act == "float32" else 0.02), (res["avg_nll"], want)
+    assert abs(res["perplexity"] - torch.exp(torch.tensor(res["avg_nll"])).item()) < 1e-2 * res["perplexity"]
+    assert f"PPL_CSV:698,{res['avg_nll']:.6f}" in run.stderr and "=== Perplexity Results ===" in run.stderr
+    # the same file as prompts: two lines, two sequences
+    short = tmp_path / "prompts.txt"
+    short.write_text("5, 17, 3\n\n9 8\n")
+    gen = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "quant"), d, "--tokens-file", str(short), "-n", "4", "-T", "0",
+                          "--json", "--dtype", act], capture_output=True, text=True, timeout=300)
+    direct = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "quant"), d, "-p", "5,17,3;9,8", "-n", "4", "-T", "0",
+                             "--json", "--dtype", act], capture_output=True, text=True, timeout=300)
+    assert gen.returncode == 0 and direct.returncode == 0, gen.stderr[-1000:] + direct.stderr[-1000:]
+    assert json.loads(gen.stdout.strip().splitlines()[-1]) == json.loads(direct.stdout.strip().splitlines()[-1])
+
+
 def test_a_context_length_binds_and_a_full_cache_ends_sequences(sharp):
     from turboquant_cpp_amd import Model
     d, plain, _ = sharp("A", "float32")

@@ -6,9 +6,13 @@ part of the library).
 """
 from __future__ import annotations
 
+import math
 import os
 from typing import Iterator, Sequence
 
+import torch
+
+from .csrc import ops
 from .engine.generate import GenerationOptions, GenerationResult, generate
 from .engine.model import load_model, random_model
 from .engine.step import Engine
@@ -75,6 +79,37 @@ class Model:
     def stream(self, prompt: Sequence[int], **overrides) -> Iterator[int]:
         """Yields the tokens of one continuation (the reference's ``generate`` yields text pieces)."""
         yield from self.generate(list(prompt), **overrides)
+
+    def perplexity(self, tokens: Sequence[int], chunk: int = 512) -> dict:
+        """Teacher-forced evaluation of a token sequence as the reference's ``--ppl`` does it
+        (/root/reference/tools/quant.c:430-720): the sequence, cut to the context length, goes through the model once
+        (here ``chunk`` tokens a step), and every token but the first is scored by the logits of the position
+        before it.  Returns ``tokens``, ``tokens_evaluated`` (targets outside the vocabulary are left out, :575),
+        ``avg_nll`` and ``perplexity`` = exp(avg_nll)."""
+        self._ensure_open()
+        tokens = [int(t) for t in tokens][:self.context_length]
+        if len(tokens) < 2:
+            raise ValueError("need at least 2 tokens for perplexity")
+        eng, act = self._engine, self._model.act
+        V = eng.vocab_size
+        feed = [t if 0 <= t < V else 0 for t in tokens]      # a token outside the vocabulary is fed as token 0, never scored
+        slot = eng.open(1)
+        total, n_eval = 0.0, 0
+        try:
+            for lo in range(0, len(tokens) - 1, chunk):
+                hi = min(lo + chunk, len(tokens) - 1)           # positions lo .. hi - 1 predict tokens lo + 1 .. hi
+                logits = eng.step(slot, [feed[lo:hi]], [list(range(hi - lo))])
+                targets = torch.tensor(tokens[lo + 1:hi + 1], dtype=torch.int32).to(logits.device)
+                nll = ops.nll(logits, targets, act).double().cpu()
+                scored = ~torch.isnan(nll)
+                total += float(nll[scored].sum())
+                n_eval += int(scored.sum())
+        finally:
+            eng.close(slot)
+        if n_eval == 0:
+            raise ValueError("no token of the sequence is a token of the vocabulary")
+        avg = total / n_eval
+        return {"tokens": len(tokens), "tokens_evaluated": n_eval, "avg_nll": avg, "perplexity": math.exp(avg)}
 
     # ------------------------------------------------------------ lower level, for tests and tools
     @property

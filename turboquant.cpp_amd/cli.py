@@ -3,7 +3,9 @@ defaults :196-239): the model path first, then ``-p`` prompt, ``-n`` max tokens 
 ``-P`` top-p (0.9), ``-s`` seed (42), ``--ctx`` context length, ``--info``, ``--profile``, ``--version``.  There is no
 tokenizer in this library, so a prompt is a list of token ids (``-p "5,17,3"``; several prompts are separated by
 ``;`` and run as one batch), or ``--random-prompt LEN[,LEN...]`` draws them.  ``--random-weights CONFIG.json --save
-DIR`` is the random-weights mode: it writes a model folder for a configuration and a seed and exits.
+DIR`` is the random-weights mode: it writes a model folder for a configuration and a seed and exits.  ``--ppl FILE``
+is the reference's teacher-forced perplexity (/root/reference/tools/quant.c:430-720) over a file of token ids, with its
+report and, with ``--json``, its JSON.
 """
 from __future__ import annotations
 
@@ -28,6 +30,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap = argparse.ArgumentParser(prog="turboquant_cpp_amd", description="Qwen2-MoE generation on one MI355X.")
     ap.add_argument("model", nargs="?", help="folder with config.json and model.safetensors")
     ap.add_argument("-p", dest="prompt", default=None, help='token ids of the prompt, e.g. "5,17,3"; ";" separates prompts')
+    ap.add_argument("--tokens-file", default=None, metavar="FILE", help="prompts from a file: one prompt of token ids a line")
+    ap.add_argument("--ppl", default=None, metavar="FILE", help="compute perplexity on a file of token ids (teacher-forced)")
     ap.add_argument("-n", dest="max_tokens", type=int, default=256, help="max tokens to generate (default: 256)")
     ap.add_argument("-T", dest="temperature", type=float, default=0.7, help="sampling temperature (default: 0.7)")
     ap.add_argument("-P", dest="top_p", type=float, default=0.9, help="top-p sampling (default: 0.9)")
@@ -85,7 +89,37 @@ def main(argv=None) -> int:
                   context_length=args.ctx, dtype=args.dtype, seed=args.seed, rep_penalty=args.rep_penalty,
                   max_batch=args.max_batch, stop_tokens=args.stop_id)
     print(f"loaded {args.model} in {time.time() - t0:.1f}s ({args.dtype}, context {model.context_length})", file=sys.stderr)
-    if args.random_prompt:
+    if args.ppl:
+        with open(args.ppl) as f:
+            ids = [int(t) for t in f.read().replace(",", " ").split()]
+        print(f"PPL evaluation: {min(len(ids), model.context_length)} tokens from {args.ppl}", file=sys.stderr)
+        torch.cuda.synchronize()
+        t1 = time.time()
+        res = model.perplexity(ids)
+        elapsed = time.time() - t1
+        rate = res["tokens_evaluated"] / elapsed if elapsed > 0 else 0.0
+        print("\n=== Perplexity Results ===", file=sys.stderr)
+        print(f"File:         {args.ppl}", file=sys.stderr)
+        print(f"Tokens:       {res['tokens']} (evaluated {res['tokens_evaluated']})", file=sys.stderr)
+        print(f"KV type:      {args.dtype}", file=sys.stderr)
+        print(f"Avg NLL:      {res['avg_nll']:.6f}", file=sys.stderr)
+        print(f"Perplexity:   {res['perplexity']:.4f}", file=sys.stderr)
+        print(f"Time:         {elapsed:.1f}s ({rate:.1f} tok/s)", file=sys.stderr)
+        print("==========================", file=sys.stderr)
+        print(f"PPL_CSV:{res['tokens_evaluated']},{res['avg_nll']:.6f},{res['perplexity']:.4f}", file=sys.stderr)
+        if args.json:
+            print(json.dumps({"model": args.model, "benchmark": args.ppl, "tokens": res["tokens"],
+                              "tokens_evaluated": res["tokens_evaluated"], "kv_type": args.dtype,
+                              "perplexity": round(res["perplexity"], 4), "avg_nll": round(res["avg_nll"], 6),
+                              "elapsed_s": round(elapsed, 2), "tok_per_s": round(rate, 1)}, indent=2))
+        model.close()
+        return 0
+    if args.tokens_file:
+        with open(args.tokens_file) as f:
+            prompts = [p for line in f if line.strip() for p in parse_prompts(line)]
+        if not prompts:
+            raise ValueError(f"{args.tokens_file} holds no token id")
+    elif args.random_prompt:
         g = torch.Generator().manual_seed(args.seed)
         V = model.engine.vocab_size
         prompts = [torch.randint(0, V, (int(n),), generator=g).tolist() for n in args.random_prompt.split(",")]

@@ -46,6 +46,7 @@ _SIGNATURES = {
     "tq_route": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
                  _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
     "tq_argmax": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr],
+    "tq_nll": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr],
     "tq_rep_penalty": [_c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_ptr, _c_f32, _c_ptr],
     "tq_sample_topp_scratch": [_c_int],
     "tq_sample_topp": [_c_ptr, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
@@ -646,6 +647,17 @@ def argmax(logits: torch.Tensor, act) -> torch.Tensor:
     R, V = logits.shape
     out = torch.empty((R,), dtype=torch.int32, device=logits.device)
     _run(k, library(act).tq_argmax(_ptr(logits), R, V, _ptr(out), _stream()))
+    return out
+
+
+def nll(logits: torch.Tensor, targets: torch.Tensor, act) -> torch.Tensor:
+    """-log softmax(logits[r])[targets[r]] per row, float32 [R] (NaN where the target is no token of the vocabulary)."""
+    k = "nll"
+    _check(logits, k, "logits", torch.float32)
+    R, V = logits.shape
+    _check(targets, k, "targets", torch.int32, (R,))
+    out = torch.empty((R,), dtype=torch.float32, device=logits.device)
+    _run(k, library(act).tq_nll(_ptr(logits), R, V, _ptr(targets), _ptr(out), _stream()))
     return out
 
 

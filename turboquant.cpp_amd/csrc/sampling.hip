@@ -63,6 +63,39 @@ TQ_API int tq_argmax(const float* logits, int R, int V, int* out, hipStream_t st
   return 0;
 }
 
+// ---------------------------------------------------------------- negative log-likelihood of a given next token
+// out[r] = -(logits[r][target[r]] - max_j logits[r][j] - log sum_j exp(logits[r][j] - max)), the sum in double as
+// /root/reference/tools/quant.c:577-592 takes it (a target outside the vocabulary gives NaN: the caller leaves it out, :575).
+// One workgroup per row; threads and then waves are added up in a fixed order.
+__global__ __launch_bounds__(ST) void nll_kernel(const float* __restrict__ logits, int V, const int* __restrict__ target,
+                                                 float* __restrict__ out) {
+  __shared__ float red[ST / TQ_WAVE];
+  __shared__ double dred[ST / TQ_WAVE];
+  const float* row = logits + (size_t)blockIdx.x * V;
+  float mx = -INFINITY;
+  for (int i = threadIdx.x; i < V; i += ST) mx = fmaxf(mx, row[i]);
+  mx = block_max(mx, red);
+  double sum = 0.0;
+  for (int i = threadIdx.x; i < V; i += ST) sum += exp((double)(row[i] - mx));
+#pragma unroll
+  for (int o = TQ_WAVE / 2; o > 0; o >>= 1) sum += __shfl_xor(sum, o, TQ_WAVE);
+  if (threadIdx.x % TQ_WAVE == 0) dred[threadIdx.x / TQ_WAVE] = sum;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    double total = 0.0;
+    for (int w = 0; w < ST / TQ_WAVE; ++w) total += dred[w];
+    const int t = target[blockIdx.x];
+    out[blockIdx.x] = t < 0 || t >= V ? NAN : (float)(log(total) - (double)(row[t] - mx));
+  }
+}
+
+TQ_API int tq_nll(const float* logits, int R, int V, const int* target, float* out, hipStream_t st) {
+  if (R <= 0) return 0;
+  hipLaunchKernelGGL(nll_kernel, dim3(R), dim3(ST), 0, st, logits, V, target, out);
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
 // ---------------------------------------------------------------- repetition penalty
 // For each of the last `count` tokens of a row's history, once per occurrence: a positive logit is
 // divided by the penalty, any other multiplied (/root/reference/src/engine/tq_generate.c:387-400).
