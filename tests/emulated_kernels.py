@@ -219,6 +219,15 @@ def route(x32, router, shared_scale, top_k, renormalize, unit, act):
     return (ids, weights, gate) + tuple(moe_align(ids, router.shape[0], unit, act))
 
 
+def head_rmsnorm(qkv, q_weight, k_weight, eps, num_heads, num_kv_heads, head_dim, act):
+    x = qkv.view(qkv.shape[0], num_heads + 2 * num_kv_heads, head_dim)
+    for lo, hi, w in ((0, num_heads, q_weight), (num_heads, num_heads + num_kv_heads, k_weight)):
+        if w is not None:
+            h = x[:, lo:hi].float()
+            x[:, lo:hi] = h * torch.rsqrt((h * h).mean(-1, keepdim=True) + eps) * w.float()
+    return qkv
+
+
 def qkv_rope_write(a, qkv_weight, qkv_bias, positions, seq_of_token, block_table, inv_freq, pairing, rotary_dim, k_pages,
                    v_pages, layer_offset, page_size, page_stride, num_heads, num_kv_heads, head_dim, act, runs=None):
     qkv = gemm(a, qkv_weight, act, bias=qkv_bias)
@@ -230,5 +239,5 @@ def install(monkeypatch):
     """Puts the stand-ins in place of the kernels for one test."""
     from turboquant_cpp_amd.csrc import ops
     for name in ("embed", "add_rmsnorm", "rope_kv_write", "qkv_rope_write", "attention", "gemm", "router_topk", "moe_align", "route", "gemm_pair",
-                 "moe_combine", "argmax", "rep_penalty", "sample_topp", "softcap"):
+                 "head_rmsnorm", "moe_combine", "argmax", "rep_penalty", "sample_topp", "softcap"):
         monkeypatch.setattr(ops, name, globals()[name])

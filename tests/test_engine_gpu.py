@@ -446,32 +446,40 @@ def rnd(shape, act, seed, scale=1.0):
 
 
 @pytest.mark.parametrize("act", ACTS)
-def test_attention_part_alone(act):
+@pytest.mark.parametrize("out_bias,qk_norm", [(False, False), (True, False), (True, True)])
+def test_attention_part_alone(act, out_bias, qk_norm):
     import plain_qwen2moe as P
     from turboquant_cpp_amd.config import PartSpec
     from turboquant_cpp_amd.parts import build_part
     H, nh, nkv, hd, window = 80, 6, 3, 16, 20
     spec = PartSpec("gqa_attention", dict(hidden_size=H, num_heads=nh, num_kv_heads=nkv, head_dim=hd, qkv_bias=True,
-                                          window=window, position=PartSpec("rope", dict(head_dim=hd, rotary_dim=hd,
+                                          out_bias=out_bias, qk_norm_eps=1e-3 if qk_norm else None, window=window, position=PartSpec("rope", dict(head_dim=hd, rotary_dim=hd,
                                                                                         theta=5000.0, pairing="interleaved"))))
     part = build_part("mixer", spec)
     specs = part.param_specs()
     assert specs["qkv_weight"].shape == ((nh + 2 * nkv) * hd, H) and specs["qkv_weight"].splits == (96, 48, 48)
+    assert ("out_bias" in specs) == out_bias and ("q_norm" in specs) == qk_norm == ("k_norm" in specs)
     w = {n: rnd(s.shape, act, 20 + i, 0.3) for i, (n, s) in enumerate(specs.items())}
     part.set_params({n: t.to(DEV) for n, t in w.items()})
     lens = [50, 1, 27]
     ctx, cache, slots = part_context([(part.cache_need(), None, None)], lens, act)
     x = rnd((sum(lens), H), act, 30)
     y = part.forward(x.to(DEV), ctx, 0)
-    assert y.shape == (1, sum(lens), H) and y.dtype == torch.float32
+    assert y.shape[1:] == (sum(lens), H) and y.dtype == torch.float32
+    y = y.double().sum(dim=0, keepdim=True)         # the partial sums that the next norm would add up
     o = 0
     for n in lens:
         xs = x[o:o + n].double()
         qkv = xs @ w["qkv_weight"].double().T + w["qkv_bias"].double()
         q, k, v = qkv[:, :96].view(n, nh, hd), qkv[:, 96:144].view(n, nkv, hd), qkv[:, 144:].view(n, nkv, hd)
+        if qk_norm:         # every head by itself, before the rotation
+            q = q / torch.sqrt((q * q).mean(-1, keepdim=True) + 1e-3) * w["q_norm"].double()
+            k = k / torch.sqrt((k * k).mean(-1, keepdim=True) + 1e-3) * w["k_norm"].double()
         pos = list(range(n))
         att = P.attention(P.rope(q, pos, 5000.0, "interleaved"), P.rope(k, pos, 5000.0, "interleaved"), v, window=window)
         ref = att.reshape(n, nh * hd) @ w["out_weight"].double().T
+        if out_bias:
+            ref = ref + w["out_bias"].double()
         err = (y[0, o:o + n].cpu().double() - ref).abs().max() / ref.abs().max()
         assert err < (1e-5 if act == "float32" else 3e-2)
         o += n

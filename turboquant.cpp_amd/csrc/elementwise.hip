@@ -204,6 +204,39 @@ TQ_API int tq_add_rmsnorm(float* x, const float* delta, int S, int64_t delta_str
   return 0;
 }
 
+// ---------------------------------------------------------------- RMS norm of every head of q and k
+// qkv[t] holds, in float, nh query heads, then nkv key heads, then nkv value heads of hd each.  Every query head is
+// normed over its hd values with the weights wq[hd], every key head with wk[hd] (a null pointer leaves those heads
+// as they are), in place: the per-head norm between the product and the rotation of
+// /root/reference/src/engine/tq_transformer.c:1111-1124, with the formula of tq_ops.c:1373-1410.  A wave per head.
+template <class W>
+__global__ __launch_bounds__(256) void head_rmsnorm_kernel(float* __restrict__ qkv, const W* __restrict__ wq,
+                                                           const W* __restrict__ wk, float eps, int nh, int nkv, int hd) {
+  const int wave = threadIdx.x / TQ_WAVE, lane = threadIdx.x % TQ_WAVE;
+  const int head = blockIdx.y * 4 + wave;
+  if (head >= nh + nkv) return;
+  const W* w = head < nh ? wq : wk;
+  if (!w) return;
+  float* x = qkv + ((size_t)blockIdx.x * (nh + 2 * nkv) + head) * hd;
+  float ss = 0.f;
+  for (int i = lane; i < hd; i += TQ_WAVE) ss = fmaf(x[i], x[i], ss);
+  ss = wave_sum(ss) / (float)hd + eps;
+  const float rs = 1.0f / sqrtf(ss);
+  for (int i = lane; i < hd; i += TQ_WAVE) x[i] = x[i] * rs * to_f32(w[i]);
+}
+
+TQ_API int tq_head_rmsnorm(float* qkv, const void* wq, const void* wk, int wtype, float eps, int T, int nh, int nkv,
+                           int hd, hipStream_t st) {
+  if (T <= 0 || (!wq && !wk)) return 0;
+  if (nh < 0 || nkv < 0 || hd < 1 || (nh + nkv + 3) / 4 > 65535) return TQ_ERR_BAD_ARG;
+  TQ_DISPATCH_W(wtype, {
+    hipLaunchKernelGGL(head_rmsnorm_kernel<W>, dim3(T, (nh + nkv + 3) / 4), dim3(256), 0, st, qkv, (const W*)wq,
+                       (const W*)wk, eps, nh, nkv, hd);
+  });
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
 // ---------------------------------------------------------------- rotary encoding + cache write
 // qkv[t] holds, in float, nh query heads, then nkv key heads, then nkv value heads of hd each.
 // Queries and keys are rotated by angle pos * inv_freq[i] (float) on the pair

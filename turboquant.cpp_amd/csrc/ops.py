@@ -30,6 +30,7 @@ _c_int, _c_i64, _c_f32, _c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, c
 _SIGNATURES = {
     "tq_embed": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_f32, _c_ptr],
     "tq_softcap": [_c_ptr, _c_i64, _c_f32, _c_ptr],
+    "tq_head_rmsnorm": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_f32, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "tq_add_rmsnorm": [_c_ptr, _c_ptr, _c_int, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_f32,
                        _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr],
     "tq_rope_kv_write": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
@@ -230,6 +231,26 @@ def add_rmsnorm(x: torch.Tensor, delta, weight: torch.Tensor, eps: float, act,
                                         _ptr(gate), _ptr(weight), _WTYPE[weight.dtype], float(eps), _ptr(rows), R,
                                         _ptr(out), _ptr(out32), H, _stream()))
     return out, out32
+
+
+def head_rmsnorm(qkv: torch.Tensor, q_weight: torch.Tensor | None, k_weight: torch.Tensor | None, eps: float,
+                 num_heads: int, num_kv_heads: int, head_dim: int, act) -> torch.Tensor:
+    """RMS norm of every query head (weights ``q_weight`` [hd]) and key head (``k_weight``) of the float32 rows
+    ``qkv`` [T, (nh + 2 nkv) * hd], in place; None leaves those heads alone.  Returns ``qkv``."""
+    k = "head_rmsnorm"
+    _check(qkv, k, "qkv", torch.float32)
+    _need(qkv.dim() == 2 and qkv.shape[1] == (num_heads + 2 * num_kv_heads) * head_dim, k,
+          f"qkv must be [T, {(num_heads + 2 * num_kv_heads) * head_dim}]")
+    wtype = None
+    for name, w in (("q_weight", q_weight), ("k_weight", k_weight)):
+        if w is not None:
+            _check(w, k, name, tuple(_WTYPE), (head_dim,))
+            _need(wtype in (None, w.dtype), k, "q_weight and k_weight must have one type")
+            wtype = w.dtype
+    if wtype is not None:
+        _run(k, library(act).tq_head_rmsnorm(_ptr(qkv), _ptr(q_weight), _ptr(k_weight), _WTYPE[wtype], float(eps),
+                                             qkv.shape[0], num_heads, num_kv_heads, head_dim, _stream()))
+    return qkv
 
 
 def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor,
