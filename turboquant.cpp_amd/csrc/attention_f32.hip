@@ -45,6 +45,21 @@ struct AttnF32Args {
   int tiles_max;           // decode: tiles per sequence in `partial`
 };
 
+// Lanes l and l ^ 8 (the same quarter g = l / 16, rows r and r ^ 8 of 16) fetched whole lines: lane (r, g) chunk
+// g + 4 (r / 8) of row r % 8 into t0 and of row 8 + r % 8 into t1.  Afterwards t0 is chunk g and t1 chunk g + 4 of
+// the lane's own row r.
+__device__ __forceinline__ void to_own_row(f32x4& t0, f32x4& t1) {
+  f32x4 s0, s1;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    // row_ror:8 reads lane l ^ 8 of each row of 16 lanes; the bank mask says which lanes take it (0xc: 8..15, 0x3: 0..7)
+    s0[i] = __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(t0[i]), __float_as_int(t1[i]), 0x128, 0xf, 0xc, false));
+    s1[i] = __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(t1[i]), __float_as_int(t0[i]), 0x128, 0xf, 0x3, false));
+  }
+  t0 = s0;
+  t1 = s1;
+}
+
 __device__ __forceinline__ float group_max(float v) {       // over the four lanes l, l^16, l^32, l^48
   v = fmaxf(v, __shfl_xor(v, 16, 64));
   return fmaxf(v, __shfl_xor(v, 32, 64));
@@ -187,23 +202,26 @@ __global__ __launch_bounds__(256) void attn_f32_prefill_kernel(AttnF32Args p, in
 }
 
 // ------------------------------------------------------------------------------------------ one token per sequence
-// grid (B, nkv * passes, tiles / 4): wave w of workgroup z takes tile 4 z + w of its sequence for up to 16 heads of
-// one kv group; what it finds goes to partial[b][head][tile] = (maximum, sum, weighted values[hd]).  Keys and values
-// go from the pages straight into the operand registers as the products come to them; five waves share a SIMD, and
-// while some wait for memory others multiply.  (Measured at 64 sequences of 1,071 positions on average, 16 heads of
-// 128: 398 us a layer.  Asking for a whole tile before the first product, by whole lines of 128 bytes, leaves one or
-// two waves to a SIMD, whose loads and products then take turns instead of overlapping: 474 to 512 us.)
-template <int ND>
-__global__ __launch_bounds__(256) void attn_f32_decode_kernel(AttnF32Args p, int passes) {
+// grid (B, nkv * passes, tiles), one wave each: wave z of a sequence takes the z-th tile of its reach for up to 16
+// heads of one kv group; what it finds goes to partial[b][head][tile] = (maximum, sum, weighted values[hd]).
+// Keys and values go from the pages straight into the operand registers as the products come to them, by whole
+// lines of 128 bytes where the head size allows (a multiple of 32): lanes l and l ^ 8 fetch for each other and
+// exchange (to_own_row).  Four or five waves share a SIMD, and while some wait for memory others multiply.
+// Measured at 64 sequences of 1,071 positions on average, 16 heads of 128, a layer: 414 us with half lines per
+// instruction, a tile per wave and four waves to a workgroup; 286 with whole lines; 277 with one wave to a
+// workgroup.  Asking for a whole tile before the first product leaves one or two waves to a SIMD, whose loads and
+// products then take turns instead of overlapping: 474 to 512 us.  A wave that takes two or three tiles in turn
+// (half or a third as many waves, fewer of them empty) needs 118 registers instead of 90 and gains nothing: 302 to 306 us.
+template <int ND, bool LINES>
+__global__ __launch_bounds__(64) void attn_f32_decode_kernel(AttnF32Args p, int passes) {
   const int b = blockIdx.x, kvh = blockIdx.y / passes, pass = blockIdx.y % passes;
-  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, r = lane % 16, g = lane / 16;
-  const int tile = blockIdx.z * 4 + wave;
+  const int lane = threadIdx.x, r = lane % 16, g = lane / 16;
   const int pos = p.start[b];                       // the token's position: it attends to lo..pos
   const int lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
-  const int key0 = tile * AT;
-  if (key0 > pos || key0 + AT <= lo) return;
+  const int first = lo / AT, last = pos / AT;
+  const int tile = first + blockIdx.z;
+  if (tile > last) return;
   const int* table = p.block_table + (size_t)p.slots[b] * p.bt_stride;
-  const int page = table[key0 / p.page_size];
   const int hd = p.hd, group = p.nh / p.nkv;
   const int hq = pass * 16 + r;                     // this lane's query: head hq of the group
   const bool q_ok = hq < group;
@@ -218,40 +236,70 @@ __global__ __launch_bounds__(256) void attn_f32_decode_kernel(AttnF32Args p, int
     qf[u] = *reinterpret_cast<const f32x4*>(d < hd ? qrow + d : qrow);
     qf[u] = q_ok && d < hd ? qf[u] : zero;
   }
-  f32x4 acc[ND];
+  {
+    const int key0 = tile * AT;
+    const int page = table[key0 / p.page_size];
+    f32x4 acc[ND];
 #pragma unroll
-  for (int dt = 0; dt < ND; ++dt) acc[dt] = zero;
-  float m_run = -INFINITY, l_run = 0.f;
-  const float* kp = p.k_pool + (size_t)page * p.page_stride + ((size_t)kvh * p.page_size + key0 % p.page_size) * hd;
-  const float* vp = p.v_pool + (size_t)page * p.page_stride + (size_t)kvh * p.page_size * hd + key0 % p.page_size;
-  // (what lies beyond the head size is asked for at the tile's first address instead and replaced by zeros: every
-  // lane loads, so that no load waits behind a branch)
-  attend_tile<ND>(
-      qf,
-      [&](int kt, int u) {
-        const int d = 16 * u + 4 * g;
-        const f32x4 x = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(d < hd ? kp + (size_t)(16 * kt + r) * hd + d : kp));
-        return d < hd ? x : zero;
-      },
-      [&](int dt, int kt) {
-        const int d = 16 * dt + r;
-        const f32x4 x = __builtin_nontemporal_load(
-            reinterpret_cast<const f32x4*>(d < hd ? vp + (size_t)d * p.page_size + 16 * kt + 4 * g : vp));
-        return d < hd ? x : zero;
-      },
-      key0, q_ok ? pos : -1, lo, p.scale, m_run, l_run, acc);
-  if (!q_ok) return;
-  float* out = p.partial + (((size_t)b * p.nh + h) * p.tiles_max + tile) * (hd + 2);
-  if (g == 0) {
-    out[0] = m_run;
-    out[1] = l_run;
-  }
+    for (int dt = 0; dt < ND; ++dt) acc[dt] = zero;
+    float m_run = -INFINITY, l_run = 0.f;
+    const float* kp = p.k_pool + (size_t)page * p.page_stride + ((size_t)kvh * p.page_size + key0 % p.page_size) * hd;
+    const float* vp = p.v_pool + (size_t)page * p.page_stride + (size_t)kvh * p.page_size * hd + key0 % p.page_size;
+    if (LINES) {
+      const int r8 = r % 8, ch = 4 * (g + 4 * (r / 8));
+      f32x4 k_next, v_next;
+      attend_tile<ND>(
+          qf,
+          [&](int kt, int u) {
+            if (u % 2) return k_next;
+            const float* base = kp + (size_t)(16 * kt + r8) * hd + 16 * u + ch;
+            f32x4 t0 = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(base));
+            f32x4 t1 = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(base + (size_t)8 * hd));
+            to_own_row(t0, t1);
+            k_next = t1;
+            return t0;
+          },
+          [&](int dt, int kt) {
+            if (kt % 2) return v_next;
+            const float* base = vp + (size_t)(16 * dt + r8) * p.page_size + 16 * kt + ch;
+            f32x4 t0 = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(base));
+            f32x4 t1 = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(base + (size_t)8 * p.page_size));
+            to_own_row(t0, t1);
+            v_next = t1;
+            return t0;
+          },
+          key0, q_ok ? pos : -1, lo, p.scale, m_run, l_run, acc);
+    } else {
+      // (what lies beyond the head size is asked for at the tile's first address instead and replaced by zeros:
+      // every lane loads, so that no load waits behind a branch)
+      attend_tile<ND>(
+          qf,
+          [&](int kt, int u) {
+            const int d = 16 * u + 4 * g;
+            const f32x4 x = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(d < hd ? kp + (size_t)(16 * kt + r) * hd + d : kp));
+            return d < hd ? x : zero;
+          },
+          [&](int dt, int kt) {
+            const int d = 16 * dt + r;
+            const f32x4 x = __builtin_nontemporal_load(
+                reinterpret_cast<const f32x4*>(d < hd ? vp + (size_t)d * p.page_size + 16 * kt + 4 * g : vp));
+            return d < hd ? x : zero;
+          },
+          key0, q_ok ? pos : -1, lo, p.scale, m_run, l_run, acc);
+    }
+    if (!q_ok) return;
+    float* out = p.partial + (((size_t)b * p.nh + h) * p.tiles_max + tile) * (hd + 2);
+    if (g == 0) {
+      out[0] = m_run;
+      out[1] = l_run;
+    }
 #pragma unroll
-  for (int dt = 0; dt < ND; ++dt) {
-    const int d = 16 * dt + 4 * g;
-    if (d < hd) {
+    for (int dt = 0; dt < ND; ++dt) {
+      const int d = 16 * dt + 4 * g;
+      if (d < hd) {
 #pragma unroll
-      for (int v = 0; v < 4; ++v) out[2 + d + v] = acc[dt][v];
+        for (int v = 0; v < 4; ++v) out[2 + d + v] = acc[dt][v];
+      }
     }
   }
 }
@@ -292,8 +340,12 @@ static int launch_attention_f32(const AttnF32Args& p, int B, int decode, int max
   if (decode) {
     const int tiles = (max_end + AT - 1) / AT;
     const int group = p.nh / p.nkv, passes = (group + 15) / 16;
-    if (p.nkv * passes > 65535 || (tiles + 3) / 4 > 65535) return TQ_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL(attn_f32_decode_kernel<ND>, dim3(B, p.nkv * passes, (tiles + 3) / 4), dim3(256), 0, st, p, passes);
+    const int waves = tiles;
+    if (p.nkv * passes > 65535 || waves > 65535) return TQ_ERR_UNSUPPORTED;
+    if (p.hd % 32 == 0 && p.page_size % 32 == 0)
+      hipLaunchKernelGGL((attn_f32_decode_kernel<ND, true>), dim3(B, p.nkv * passes, waves), dim3(64), 0, st, p, passes);
+    else
+      hipLaunchKernelGGL((attn_f32_decode_kernel<ND, false>), dim3(B, p.nkv * passes, waves), dim3(64), 0, st, p, passes);
     hipLaunchKernelGGL(attn_f32_join_kernel, dim3(B, p.nh), dim3(128), 0, st, p);
     return 0;
   }
