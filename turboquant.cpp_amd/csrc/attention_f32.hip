@@ -304,28 +304,40 @@ __global__ __launch_bounds__(64) void attn_f32_decode_kernel(AttnF32Args p, int 
   }
 }
 
-// out[b][h] = sum over the tiles in reach, in ascending order, of exp(m_tile - m) * values / sum of exp(m_tile - m) * sums
-__global__ __launch_bounds__(128) void attn_f32_join_kernel(AttnF32Args p) {
-  const int b = blockIdx.x, h = blockIdx.y;
+// out[b][h] = sum over the tiles in reach, in ascending order, of exp(m_tile - m) * values / sum of exp(m_tile - m) * sums.
+// grid (B, nh), one wave: the tiles' weights exp(m_tile - m) are worked out once, a lane per tile, and kept in LDS;
+// the denominators are added 64 tiles at a time in tile order; then every lane sums its dimensions over the tiles in order.
+#define F32_JOIN_TILES 4096
+__global__ __launch_bounds__(64) void attn_f32_join_kernel(AttnF32Args p) {
+  __shared__ float wgt[F32_JOIN_TILES];
+  const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int pos = p.start[b];
   const int lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
   const int first = lo / AT, last = pos / AT;
-  const float* part = p.partial + ((size_t)b * p.nh + h) * p.tiles_max * (p.hd + 2);
+  const int stride = p.hd + 2;
+  const float* part = p.partial + ((size_t)b * p.nh + h) * p.tiles_max * stride;
   float m = -INFINITY;
-  for (int tile = first; tile <= last; ++tile) m = fmaxf(m, part[(size_t)tile * (p.hd + 2)]);
+  for (int tile = first + lane; tile <= last; tile += 64) m = fmaxf(m, part[(size_t)tile * stride]);
+  m = wave_max(m);
   float l = 0.f;
-  for (int tile = first; tile <= last; ++tile) {
-    const float* q = part + (size_t)tile * (p.hd + 2);
-    l += expf(q[0] - m) * q[1];
+  for (int t0 = first; t0 <= last; t0 += 64) {
+    const int tile = t0 + lane;
+    float w = 0.f, wl = 0.f;
+    if (tile <= last) {
+      const float* q = part + (size_t)tile * stride;
+      w = expf(q[0] - m);
+      wl = w * q[1];
+      wgt[tile - first] = w;
+    }
+    l += wave_sum(wl);
   }
+  __builtin_amdgcn_wave_barrier();
   const float inv = 1.0f / l;
   float* orow = p.out + ((size_t)p.cu_seqlens[b] * p.nh + h) * p.hd;
-  for (int d = threadIdx.x; d < p.hd; d += blockDim.x) {
+  for (int d = lane; d < p.hd; d += 64) {
     float a = 0.f;
-    for (int tile = first; tile <= last; ++tile) {
-      const float* q = part + (size_t)tile * (p.hd + 2);
-      a += expf(q[0] - m) * q[2 + d];
-    }
+#pragma unroll 8
+    for (int tile = first; tile <= last; ++tile) a = fmaf(wgt[tile - first], part[(size_t)tile * stride + 2 + d], a);
     orow[d] = a * inv;
   }
 }
@@ -341,12 +353,12 @@ static int launch_attention_f32(const AttnF32Args& p, int B, int decode, int max
     const int tiles = (max_end + AT - 1) / AT;
     const int group = p.nh / p.nkv, passes = (group + 15) / 16;
     const int waves = tiles;
-    if (p.nkv * passes > 65535 || waves > 65535) return TQ_ERR_UNSUPPORTED;
+    if (p.nkv * passes > 65535 || waves > 65535 || tiles > F32_JOIN_TILES) return TQ_ERR_UNSUPPORTED;
     if (p.hd % 32 == 0 && p.page_size % 32 == 0)
       hipLaunchKernelGGL((attn_f32_decode_kernel<ND, true>), dim3(B, p.nkv * passes, waves), dim3(64), 0, st, p, passes);
     else
       hipLaunchKernelGGL((attn_f32_decode_kernel<ND, false>), dim3(B, p.nkv * passes, waves), dim3(64), 0, st, p, passes);
-    hipLaunchKernelGGL(attn_f32_join_kernel, dim3(B, p.nh), dim3(128), 0, st, p);
+    hipLaunchKernelGGL(attn_f32_join_kernel, dim3(B, p.nh), dim3(64), 0, st, p);
     return 0;
   }
   constexpr int HDP = 16 * ND;
