@@ -228,6 +228,10 @@ def head_rmsnorm(qkv, q_weight, k_weight, eps, num_heads, num_kv_heads, head_dim
     return qkv
 
 
+def expert_tile_rows(n_pairs, num_experts, act, a, w):
+    return 16 if n_pairs <= 16 * num_experts else 64
+
+
 def qkv_rope_write(a, qkv_weight, qkv_bias, positions, seq_of_token, block_table, inv_freq, pairing, rotary_dim, k_pages,
                    v_pages, layer_offset, page_size, page_stride, num_heads, num_kv_heads, head_dim, act, runs=None):
     qkv = gemm(a, qkv_weight, act, bias=qkv_bias)
@@ -239,5 +243,5 @@ def install(monkeypatch):
     """Puts the stand-ins in place of the kernels for one test."""
     from turboquant_cpp_amd.csrc import ops
     for name in ("embed", "add_rmsnorm", "rope_kv_write", "qkv_rope_write", "attention", "gemm", "router_topk", "moe_align", "route", "gemm_pair",
-                 "head_rmsnorm", "moe_combine", "argmax", "rep_penalty", "sample_topp", "softcap"):
+                 "head_rmsnorm", "expert_tile_rows", "moe_combine", "argmax", "rep_penalty", "sample_topp", "softcap"):
         monkeypatch.setattr(ops, name, globals()[name])

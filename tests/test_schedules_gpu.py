@@ -145,6 +145,33 @@ def test_sequences_cross_the_positions_where_steps_change_shape(act, sharp):
     check_logits(out[True][1], torch.cat([ref_s[20:36]] * 2), torch.cat([margins_s[20:36]] * 2), act, f"A {act} the short one beside it")
 
 
+# ------------------------------------------------------------------------------------------------ a long prompt's experts
+def test_a_long_prompt_takes_the_taller_expert_tiles(sharp, monkeypatch):
+    """From 256 rows per expert on, the bfloat16 products over experts take tiles of 128 rows: a prompt of 1,400 tokens
+    with one expert of five per token goes that way through the engine (and one of 700 does not), and every
+    position agrees with the plain model."""
+    from turboquant_cpp_amd.csrc import ops
+    from turboquant_cpp_amd.engine.step import Engine
+    d, plain, model = sharp("C", "bfloat16")
+    units = []
+    route = ops.route
+
+    def spy(x32, router, shared_scale, top_k, renormalize, unit, act):
+        units.append(unit)
+        return route(x32, router, shared_scale, top_k, renormalize, unit, act)
+
+    monkeypatch.setattr(ops, "route", spy)
+    eng = Engine(model, max_tokens=64 * 40, page_size=64)
+    for n, unit in ((1400, 128), (700, 64)):
+        (prompt,) = prompts_for("C", [n], seed=29)
+        del units[:]
+        slots = eng.open(1)
+        got = eng.step(slots, [prompt], [list(range(n))])
+        eng.close(slots)
+        assert units and all(u == unit for u in units), (n, units)
+        check_sequence(got, plain, prompt, "bfloat16", f"C bfloat16 {n} tokens at once")
+
+
 # ------------------------------------------------------------------------------------------------ entry points
 @pytest.mark.parametrize("act", ACTS)
 def test_the_command_line_generates(act, sharp):

@@ -625,7 +625,7 @@ TQ_API int tq_gemm_mfma_splits(int M, int N, int K) {
 }
 
 // a: bfloat16 [.., K] with row stride lda (a multiple of 8, as K must be); w, w2: bfloat16.
-// tile_rows: with tile_group set, the padding unit of the row order (16 or 64); else a hint that is ignored.
+// tile_rows: with tile_group set, the padding unit of the row order (16, 64 or 128); else a hint that is ignored.
 // splits > 1 (as tq_gemm_mfma_splits says, for a plain product into float): run z of k goes to out + z * M * ldc,
 // the bias to run 0; the sum over the runs is the caller's.
 TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gather, const void* w, const void* w2,
@@ -649,6 +649,9 @@ TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gat
     } else if (tile_rows == 64) {
       if ((N + TBN - 1) / TBN > 65535) return TQ_ERR_UNSUPPORTED;
       rc = launch_tile<64, 2, 4>(g, dual, out_act, 1, st);
+    } else if (tile_rows == 128) {     // experts with hundreds of rows each: the taller tile's rate for little padding
+      if ((N + TBN - 1) / TBN > 65535 || M % 128) return TQ_ERR_UNSUPPORTED;
+      rc = launch_tile<128, 4, 2>(g, dual, out_act, 1, st);
     } else {
       return TQ_ERR_BAD_ARG;
     }

@@ -70,7 +70,7 @@ class SparseMoE(Part):
 
     def forward(self, normed, normed32, ctx):
         T = normed.shape[0]
-        unit = 16 if T * self.top_k <= 16 * self.num_experts else 64
+        unit = ops.expert_tile_rows(T * self.top_k, self.num_experts, ctx.act, normed, self.expert_gate)
         route = lambda: ops.route(normed32, self.router, self.shared_scale if self.shared_gated else None,
                                   self.top_k, self.renormalize, unit, ctx.act)
         if self.shared_size > 0 and T <= 16 and unit == 16:
