@@ -145,6 +145,74 @@ def test_sequences_cross_the_positions_where_steps_change_shape(act, sharp):
     check_logits(out[True][1], torch.cat([ref_s[20:36]] * 2), torch.cat([margins_s[20:36]] * 2), act, f"A {act} the short one beside it")
 
 
+# ------------------------------------------------------------------------------------------------ sizes drawn at random
+def random_configuration(rnd):
+    nkv = rnd.choice([1, 2, 3, 4])
+    nh = nkv * rnd.choice([1, 1, 2, 3, 5, 7])
+    E = rnd.choice([2, 5, 8, 17, 64])
+    window = rnd.choice([None, None, 3, 17, 70])
+    return {"architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe", "vocab_size": rnd.choice([50, 257, 1000]),
+            "hidden_size": rnd.choice([40, 64, 72, 136, 200, 256]), "num_hidden_layers": rnd.choice([1, 2, 3]),
+            "num_attention_heads": nh, "num_key_value_heads": nkv, "head_dim": rnd.choice([16, 24, 32, 48, 64, 80, 128]),
+            "intermediate_size": rnd.choice([24, 96, 104]), "moe_intermediate_size": rnd.choice([8, 24, 40]),
+            "shared_expert_intermediate_size": rnd.choice([0, 16, 56]), "num_experts": E,
+            "num_experts_per_tok": rnd.randint(1, min(E, 8)), "norm_topk_prob": rnd.choice([True, False]),
+            "decoder_sparse_step": rnd.choice([1, 1, 2]), "mlp_only_layers": rnd.choice([[], [0]]),
+            "rope_theta": rnd.choice([1e4, 1e6]), "rms_norm_eps": rnd.choice([1e-6, 1e-5]),
+            "use_sliding_window": window is not None, "sliding_window": window or 4096,
+            "max_window_layers": rnd.choice([0, 1]), "max_position_embeddings": 512,
+            "tie_word_embeddings": rnd.choice([True, False]), "torch_dtype": "float32"}
+
+
+@pytest.mark.parametrize("seed", [3, 8, 11, 17, 24, 30, 36, 41])
+def test_configurations_drawn_at_random(seed, tmp_path):
+    """Head counts, groups, head sizes in steps of 8, widths, vocabularies, expert counts, windows and layer kinds drawn
+    at random, in 32-bit: three sequences whole in one batch, then their first halves as prompts and the rest token
+    by token in slots that were used before, every position against the plain model."""
+    import random
+    from turboquant_cpp_amd.engine.model import load_model, write_random_model_dir
+    from turboquant_cpp_amd.engine.step import Engine
+    rnd = random.Random(seed)
+    cfg = random_configuration(rnd)
+    what = " ".join(f"{k}={cfg[k]}" for k in ("num_attention_heads", "num_key_value_heads", "head_dim", "hidden_size",
+                                             "num_experts", "num_experts_per_tok", "sliding_window", "vocab_size"))
+    act = "float32"
+    d = str(tmp_path / "model")
+    write_random_model_dir(d, cfg, seed, 0.1, 0.02, act)
+    plain = PlainQwen2Moe(d)
+    eng = Engine(load_model(d, act=act, device=DEV), max_tokens=64 * 12)
+    lens = [rnd.randint(1, 90), rnd.randint(1, 40), rnd.randint(60, 150)]
+    g = torch.Generator().manual_seed(seed)
+    prompts = [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in lens]
+    slots = eng.open(3)
+    whole = eng.step(slots, prompts, [list(range(n)) for n in lens])
+    eng.close(slots)
+    o = 0
+    for i, p in enumerate(prompts):
+        check_sequence(whole[o:o + len(p)], plain, p, act, f"{what}: sequence {i} whole")
+        o += len(p)
+    slots = eng.open(3)
+    cut = [max(1, n // 2) for n in lens]
+    first = eng.step(slots, [p[:c] for p, c in zip(prompts, cut)], [list(range(c)) for c in cut])
+    rows, o = [], 0
+    for c in cut:
+        rows.append([first[o:o + c]])
+        o += c
+    pos = list(cut)
+    live = [i for i in range(3) if cut[i] < lens[i]]
+    eng.close([slots[i] for i in range(3) if i not in live])
+    while live:
+        lg = eng.step([slots[i] for i in live], [[prompts[i][pos[i]]] for i in live])
+        for j, i in enumerate(live):
+            rows[i].append(lg[j:j + 1])
+            pos[i] += 1
+        done = [i for i in live if pos[i] == lens[i]]
+        eng.close([slots[i] for i in done])
+        live = [i for i in live if i not in done]
+    for i, p in enumerate(prompts):
+        check_sequence(torch.cat(rows[i]), plain, p, act, f"{what}: sequence {i}, second half token by token")
+
+
 # ------------------------------------------------------------------------------------------------ a long prompt's experts
 def test_a_long_prompt_takes_the_taller_expert_tiles(sharp, monkeypatch):
     """From 256 rows per expert on, the bfloat16 products over experts take tiles of 128 rows: a prompt of 1,400 tokens
