@@ -106,7 +106,13 @@ def check_sequence(got, plain, prompt, act, what):
     tie = F32_TIE if act == "float32" else BF16_TIE
     plain.other_side = {}
     try:
-        ref = plain.logits(prompt)
+        # the plain model's logits with no decision turned are kept per sequence: several cuts of a sequence share them
+        kept = plain.__dict__.setdefault("_undecided", {})
+        key = tuple(prompt)
+        at_hand = key not in kept          # whether the plain model's record of margins is that of `ref`
+        if at_hand:
+            kept[key] = plain.logits(prompt)
+        ref = kept[key]
         scale = ref.abs().max().item()
         tol = 1e-4 if act == "float32" else 0.04 * scale
         for _ in range(len(prompt)):
@@ -115,6 +121,9 @@ def check_sequence(got, plain, prompt, act, what):
             if bad.numel() == 0:
                 break
             p = int(bad[0])
+            if not at_hand:
+                plain.logits(prompt)
+                at_hand = True
             swaps = [(l, i, j) for _gap, l, _p, i, j in plain.near_ties(tie, p) if (l, p) not in plain.other_side]
             tries = [(s,) for s in swaps] + [c for c in itertools.combinations(swaps[:6], 2) if c[0][0] != c[1][0]]
             settled = False
@@ -270,10 +279,13 @@ def test_first_tokens_and_long_decoding(name, act, engines):
 
 def test_the_layer_sizes_of_a_real_checkpoint(tmp_path):
     """Two layers with the sizes of Qwen1.5-MoE-A2.7B (width 2,048, 16 heads of 128, 60 experts of 1,408, top 4, a
-    shared expert of 5,632; a small vocabulary) with random weights, against the plain implementation: three
-    prompts of unequal length in one step (one long enough for the tiled products), then steps of one token.
-    The tiny configurations of the other tests never reach the kernel variants of these sizes (rows of whole cache
-    lines, waves that split k, two products in one launch, head size 128, the product that rotates and stores)."""
+    shared expert of 5,632; a small vocabulary) with random weights, against the plain implementation, cut three
+    ways: the prompts whole in one step (one long enough for the tiled products) and then steps of one token; the
+    first tokens as prompts and the last 32 of each sequence token by token, shorter sequences ending earlier; and
+    the sequences in another order over two batches in slots used before, their prompts cut elsewhere and continued
+    by a second chunk.  The tiny configurations of the other tests never reach the kernel variants of these sizes
+    (rows of whole cache lines, waves that split k, two products in one launch, head size 128, the product that
+    rotates and stores)."""
     from turboquant_cpp_amd.engine.model import load_model, write_random_model_dir
     from turboquant_cpp_amd.engine.step import Engine
     cfg = {"architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe", "vocab_size": 8000, "hidden_size": 2048,
@@ -285,24 +297,61 @@ def test_the_layer_sizes_of_a_real_checkpoint(tmp_path):
     g = torch.Generator().manual_seed(41)
     n_fed = 4
     seqs = [torch.randint(0, 8000, (n + n_fed,), generator=g).tolist() for n in (200, 70, 9)]
+
+    def run(eng, order, cuts):
+        """The sequences `order` as one batch: tokens up to cuts[i][0] as prompts, then chunks up to each further
+        cut, then token by token; returns every sequence's logits at all of its positions."""
+        slots = eng.open(len(order))
+        rows = {i: [] for i in order}
+        pos = {i: 0 for i in order}
+        depth = max(len(cuts[i]) for i in order)
+        for c in range(depth):
+            live = [i for i in order if c < len(cuts[i])]
+            lg = eng.step([slots[order.index(i)] for i in live], [seqs[i][pos[i]:cuts[i][c]] for i in live],
+                          [list(range(cuts[i][c] - pos[i])) for i in live]).cpu()
+            o = 0
+            for i in live:
+                n = cuts[i][c] - pos[i]
+                rows[i].append(lg[o:o + n])
+                o += n
+                pos[i] = cuts[i][c]
+        live = [i for i in order if pos[i] < len(seqs[i])]
+        for i in order:
+            if i not in live:
+                eng.close([slots[order.index(i)]])
+        while live:
+            lg = eng.step([slots[order.index(i)] for i in live], [[seqs[i][pos[i]]] for i in live]).cpu()
+            for j, i in enumerate(live):
+                rows[i].append(lg[j:j + 1])
+                pos[i] += 1
+            for i in [i for i in live if pos[i] == len(seqs[i])]:
+                eng.close([slots[order.index(i)]])
+                live.remove(i)
+        return {i: torch.cat(rows[i]) for i in order}
+
     for act in ACTS:
         d = write_random_model_dir(str(tmp_path / f"a27b_two_layers_{act}"), cfg, 3, 0.02, 0.02, act)
         plain = PlainQwen2Moe(d)
         eng = Engine(load_model(d, act=act, device=DEV), max_tokens=64 * 8)
-        slots = eng.open(3)
-        prompts = [s[:-n_fed] for s in seqs]
-        first = eng.step(slots, prompts, [list(range(len(p))) for p in prompts]).cpu()
-        fed = [eng.step(slots, [[s[len(s) - n_fed + t]] for s in seqs]).cpu() for t in range(n_fed)]
-        eng.close(slots)
+        L = [len(s) for s in seqs]
+        splits = {
+            "whole prompts, then four steps": run(eng, [0, 1, 2], {i: [L[i] - n_fed] for i in range(3)}),
+            "the last 32 token by token": run(eng, [0, 1, 2], {i: [max(1, L[i] - 32)] for i in range(3)}),
+        }
+        other = run(eng, [2, 0], {2: [5], 0: [37, 150]})
+        other.update(run(eng, [1], {1: [64, 65]}))
+        splits["another order, two batches, prompts in chunks"] = other
         del eng
         torch.cuda.empty_cache()
         shutil.rmtree(d)              # gigabytes of weights: not kept for the next test session to find
-        off = 0
         for i, s in enumerate(seqs):
-            n = len(s) - n_fed
-            got = torch.cat([first[off:off + n]] + [f[i:i + 1] for f in fed])
-            off += n
-            check_sequence(got, plain, s, act, f"real layer sizes, {act}, sequence of {len(s)}")
+            first = None
+            for how, got in splits.items():
+                # a cut that agrees with one already checked to a tenth of the bound needs no second run of the plain model
+                if first is not None and act == "float32" and (got[i] - first).abs().max() < 1e-5:
+                    continue
+                check_sequence(got[i], plain, s, act, f"real layer sizes, {act}, sequence of {len(s)}, {how}")
+                first = got[i] if first is None else first
         del plain
 
 
