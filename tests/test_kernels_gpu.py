@@ -116,9 +116,9 @@ def test_gemm_partial_sums(ops, act, M, N, K, bias):
     if act == "bfloat16":
         if M <= 16:
             runs = 1
-        elif M <= 64:       # few rows of a narrow matrix: runs of at least 256 of k for each of 8 waves, up to 2048 waves
+        elif M <= 64:       # few rows of a narrow matrix: runs of at least 128 of k for each of 8 waves, up to 4096 waves
             runs, waves = 1, -(-N // 32) * 8
-            while runs < 8 and waves * runs < 2048 and K // (16 * runs) >= 256:
+            while runs < 8 and waves * runs < 4096 and K // (16 * runs) >= 128:
                 runs *= 2
         else:
             runs = 1 if K < 2048 else (2 if K < 4096 else 4)

@@ -608,14 +608,15 @@ static int plain_tile_choice(int M, int N, int splits) {
 // Into how many runs of k a plain product of M rows may be split when its partial sums are wanted apart.  Many
 // rows: a product whose tiles do not fill the chip twice, and that has k enough, goes faster in 2 to 4 runs, each
 // at least 1024 long.  17 to 64 rows of a narrow matrix with a long k (the streaming kernel with at most 8 waves
-// over k): as many runs as bring about 2048 waves, each wave keeping 256 of k.  1 for up to 16 rows.
+// over k): as many runs as bring about 4096 waves, each wave keeping 128 of k (64 rows by 2,048 x 2,048: 13.4 us in
+// two runs against 15.2 in one; by 2,048 x 5,632: 17.3 in four against 20.7 in two).  1 for up to 16 rows.
 TQ_API int tq_gemm_mfma_splits(int M, int N, int K) {
   if (M <= 16) return 1;
   if (M <= 64) {
     if (wide_enough_for_tiles(N)) return 1;
     const int64_t waves = (int64_t)((N + 31) / 32) * 8;
     int s = 1;
-    while (s < 8 && waves * s < 2048 && K / (16 * s) >= 256) s *= 2;
+    while (s < 8 && waves * s < 4096 && K / (16 * s) >= 128) s *= 2;
     return s;
   }
   const int64_t tiles = (int64_t)((M + 127) / 128) * ((N + TBN - 1) / TBN);
