@@ -281,6 +281,8 @@ def main() -> int:
         page = 64
         per_seq = -(-context // page) * page
         engine = Engine(model, max_tokens=per_seq * batch, page_size=page, max_slots=batch)
+        if args.one_stream:
+            engine.side_stream = None
         slots = engine.open(batch)
         prompts = [torch.randint(0, V, (prompt_len,), generator=gen).tolist() for _ in range(batch)]
         tp = time.time()

@@ -116,31 +116,38 @@ def library(dtype) -> ctypes.CDLL:
     return lib
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None) or (lambda dev: torch.cuda.current_stream(dev).cuda_stream)
+
+
 def has_kernel(dtype, name: str) -> bool:
     return hasattr(library(dtype), name)
 
 
 def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    """The current stream's handle (the raw call: building a stream object for every launch cost 5 us of the host's
+    time, a fifth of what a launch took)."""
+    return _raw_stream(torch.cuda.current_device())
 
 
 def _ptr(t: torch.Tensor | None) -> int | None:
     return None if t is None else t.data_ptr()
 
 
-def _need(cond: bool, kernel: str, what: str) -> None:
+def _need(cond: bool, kernel: str, what) -> None:
+    """``what``: the message, or a function that makes it (so that a check that holds formats nothing)."""
     if not cond:
-        raise KernelError(f"{kernel}: {what}")
+        raise KernelError(f"{kernel}: {what() if callable(what) else what}")
 
 
 def _check(t: torch.Tensor, kernel: str, name: str, dtype=None, shape=None) -> None:
-    _need(isinstance(t, torch.Tensor) and t.is_cuda, kernel, f"{name} must be a GPU tensor")
-    _need(t.is_contiguous(), kernel, f"{name} must be contiguous, has strides {t.stride()}")
-    if dtype is not None:
-        ok = t.dtype in dtype if isinstance(dtype, (tuple, list)) else t.dtype == dtype
-        _need(ok, kernel, f"{name} must be {dtype}, is {t.dtype}")
-    if shape is not None:
-        _need(tuple(t.shape) == tuple(shape), kernel, f"{name} must have shape {tuple(shape)}, has {tuple(t.shape)}")
+    if not (isinstance(t, torch.Tensor) and t.is_cuda):
+        raise KernelError(f"{kernel}: {name} must be a GPU tensor")
+    if not t.is_contiguous():
+        raise KernelError(f"{kernel}: {name} must be contiguous, has strides {t.stride()}")
+    if dtype is not None and not (t.dtype in dtype if type(dtype) in (tuple, list) else t.dtype == dtype):
+        raise KernelError(f"{kernel}: {name} must be {dtype}, is {t.dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise KernelError(f"{kernel}: {name} must have shape {tuple(shape)}, has {tuple(t.shape)}")
 
 
 def _run(kernel: str, code: int) -> None:
@@ -206,18 +213,18 @@ def add_rmsnorm(x: torch.Tensor, delta, weight: torch.Tensor, eps: float, act,
     if isinstance(delta, GatheredSum):
         y, pair_slot, weights, gate, delta = delta.y, delta.pair_slot, delta.weights, delta.gate, delta.dense
         _check(y, k, "y", torch.float32)
-        _need(y.dim() == 2 and y.shape[1] == H, k, f"y must be [rows, {H}]")
+        _need(y.dim() == 2 and y.shape[1] == H, k, lambda: f"y must be [rows, {H}]")
         _check(pair_slot, k, "pair_slot", torch.int32)
-        _need(pair_slot.dim() == 2 and pair_slot.shape[0] == T, k, f"pair_slot must be [{T}, k]")
+        _need(pair_slot.dim() == 2 and pair_slot.shape[0] == T, k, lambda: f"pair_slot must be [{T}, k]")
         topk = pair_slot.shape[1]
-        _need(1 <= topk <= 64, k, f"{topk} experts per token is beyond the 64 this kernel takes")
+        _need(1 <= topk <= 64, k, lambda: f"{topk} experts per token is beyond the 64 this kernel takes")
         _check(weights, k, "weights", torch.float32, (T, topk))
         if gate is not None:
             _check(gate, k, "gate", torch.float32, (T,))
     S, stride = 0, 0
     if delta is not None:
         _check(delta, k, "delta", torch.float32)
-        _need(delta.dim() == 3 and tuple(delta.shape[1:]) == (T, H), k, f"delta must be [S, {T}, {H}], is {tuple(delta.shape)}")
+        _need(delta.dim() == 3 and tuple(delta.shape[1:]) == (T, H), k, lambda: f"delta must be [S, {T}, {H}], is {tuple(delta.shape)}")
         S, stride = delta.shape[0], T * H
     R = T
     if rows is not None:
@@ -240,7 +247,7 @@ def head_rmsnorm(qkv: torch.Tensor, q_weight: torch.Tensor | None, k_weight: tor
     k = "head_rmsnorm"
     _check(qkv, k, "qkv", torch.float32)
     _need(qkv.dim() == 2 and qkv.shape[1] == (num_heads + 2 * num_kv_heads) * head_dim, k,
-          f"qkv must be [T, {(num_heads + 2 * num_kv_heads) * head_dim}]")
+          lambda: f"qkv must be [T, {(num_heads + 2 * num_kv_heads) * head_dim}]")
     wtype = None
     for name, w in (("q_weight", q_weight), ("k_weight", k_weight)):
         if w is not None:
@@ -271,7 +278,7 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torc
     _check(block_table, k, "block_table", torch.int32)
     _need(block_table.dim() == 2, k, "block_table must be [B, pages]")
     _check(inv_freq, k, "inv_freq", torch.float32)
-    _need(inv_freq.numel() * 2 == rotary_dim or rotary_dim == 0, k, f"inv_freq must hold rotary_dim/2 = {rotary_dim // 2} entries")
+    _need(inv_freq.numel() * 2 == rotary_dim or rotary_dim == 0, k, lambda: f"inv_freq must hold rotary_dim/2 = {rotary_dim // 2} entries")
     adt = ACT_DTYPES[dtype_name(act)]
     q = torch.empty((T, num_heads * head_dim), dtype=adt, device=qkv.device)
     write = k_pages is not None
@@ -355,7 +362,7 @@ def moe_combine(y: torch.Tensor, pair_slot: torch.Tensor, weights: torch.Tensor,
     S, stride = 0, 0
     if shared is not None:
         _check(shared, k, "shared", torch.float32)
-        _need(shared.dim() == 3 and tuple(shared.shape[1:]) == (T, H), k, f"shared must be [S, {T}, {H}]")
+        _need(shared.dim() == 3 and tuple(shared.shape[1:]) == (T, H), k, lambda: f"shared must be [S, {T}, {H}]")
         S, stride = shared.shape[0], T * H
     if shared_gate is not None:
         _check(shared_gate, k, "shared_gate", torch.float32, (T,))
@@ -392,7 +399,7 @@ def _gemm_problem(k: str, a, w, act, bias, w2, out_act, a_rows, tile_group, n_ti
     _check(w, k, "w", tuple(_WTYPE))
     grouped = tile_group is not None
     if grouped:
-        _need(w.dim() == 3 and w.shape[2] == K, k, f"grouped w must be [G, N, {K}], is {tuple(w.shape)}")
+        _need(w.dim() == 3 and w.shape[2] == K, k, lambda: f"grouped w must be [G, N, {K}], is {tuple(w.shape)}")
         _need(a_rows is not None and n_tiles is not None and tile_rows in (16, 64, 128), k,
               "grouped product needs a_rows, n_tiles and tile_rows of 16, 64 or 128")
         _need(tile_rows != 128 or _use_mfma(act, a, w, a.shape[1]), k,
@@ -405,7 +412,7 @@ def _gemm_problem(k: str, a, w, act, bias, w2, out_act, a_rows, tile_group, n_ti
         N = w.shape[1]
         gstride = N * K
     else:
-        _need(w.dim() == 2 and w.shape[1] == K, k, f"w must be [N, {K}], is {tuple(w.shape)}")
+        _need(w.dim() == 2 and w.shape[1] == K, k, lambda: f"w must be [N, {K}], is {tuple(w.shape)}")
         N = w.shape[0]
         M = a.shape[0] if a_rows is None else a_rows.numel()
         if a_rows is not None:
@@ -421,7 +428,7 @@ def _gemm_problem(k: str, a, w, act, bias, w2, out_act, a_rows, tile_group, n_ti
 
 
 def _gate_code(k: str, activation: str) -> int:
-    _need(activation in GATES, k, f"unknown activation {activation!r}; known: {', '.join(sorted(GATES))}")
+    _need(activation in GATES, k, lambda: f"unknown activation {activation!r}; known: {', '.join(sorted(GATES))}")
     return GATES[activation]
 
 
@@ -498,7 +505,7 @@ def gemm_pair(first: dict, second: dict, act) -> tuple[torch.Tensor, torch.Tenso
     for p in (first, second):
         full = {"bias": None, "w2": None, "out_act": False, "a_rows": None, "tile_group": None, "n_tiles": None,
                 "tile_rows": None, "gather": True, "partial_sums": False, "activation": "silu"}
-        _need(set(p) <= set(full) | {"a", "w"}, k, f"unknown arguments {sorted(set(p) - set(full) - {'a', 'w'})}")
+        _need(set(p) <= set(full) | {"a", "w"}, k, lambda: f"unknown arguments {sorted(set(p) - set(full) - {'a', 'w'})}")
         full.update(p)
         probs.append(full)
     lib = library(act) if dtype_name(act) == "bfloat16" else None
@@ -557,7 +564,7 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, lay
     _check(block_table, k, "block_table", torch.int32)
     _need(block_table.dim() == 2, k, "block_table must be [B, pages]")
     _need(num_heads % num_kv_heads == 0, k, "heads must be a multiple of kv heads")
-    _need(head_dim <= 512, k, f"head size {head_dim} is beyond the 512 this kernel takes")
+    _need(head_dim <= 512, k, lambda: f"head size {head_dim} is beyond the 512 this kernel takes")
     _need(layer_offset + num_kv_heads * page_size * head_dim <= page_stride, k, "layer does not fit in a page")
     out = torch.empty_like(q)
     esz = k_pages.element_size()
@@ -623,12 +630,12 @@ def _router_outputs(k: str, x32: torch.Tensor, router: torch.Tensor, shared_scal
     _need(x32.dim() == 2, k, "x must be [T, H]")
     T, H = x32.shape
     _check(router, k, "router", tuple(_WTYPE))
-    _need(router.dim() == 2 and router.shape[1] == H, k, f"router must be [E, {H}]")
+    _need(router.dim() == 2 and router.shape[1] == H, k, lambda: f"router must be [E, {H}]")
     E = router.shape[0]
-    _need(1 <= top_k <= min(E, 64), k, f"top_k {top_k} must be within 1..min(E, 64)")
+    _need(1 <= top_k <= min(E, 64), k, lambda: f"top_k {top_k} must be within 1..min(E, 64)")
     if shared_scale is not None:
         _check(shared_scale, k, "shared_scale", router.dtype)
-        _need(shared_scale.numel() == H, k, f"shared_scale must hold {H} values")
+        _need(shared_scale.numel() == H, k, lambda: f"shared_scale must hold {H} values")
     ids = torch.empty((T, top_k), dtype=torch.int32, device=x32.device)
     weights = torch.empty((T, top_k), dtype=torch.float32, device=x32.device)
     gate = torch.empty((T,), dtype=torch.float32, device=x32.device) if shared_scale is not None else None
@@ -701,7 +708,7 @@ def rep_penalty(logits: torch.Tensor, recent: torch.Tensor, counts: torch.Tensor
     _check(logits, k, "logits", torch.float32)
     R, V = logits.shape
     _check(recent, k, "recent", torch.int32)
-    _need(recent.dim() == 2 and recent.shape[0] == R, k, f"recent must be [{R}, window]")
+    _need(recent.dim() == 2 and recent.shape[0] == R, k, lambda: f"recent must be [{R}, window]")
     _check(counts, k, "counts", torch.int32, (R,))
     _run(k, library(act).tq_rep_penalty(_ptr(logits), R, V, _ptr(recent), recent.shape[1], _ptr(counts),
                                         float(penalty), _stream()))

@@ -16,6 +16,7 @@ class StepContext:
     act: str                          # "float32" or "bfloat16": the type of activations and cache
     device: torch.device
     side_stream: "torch.cuda.Stream | None" = None   # a second stream for work that does not depend on the main line
+    capturing: bool = False      # the step is being recorded for replay: what the host pays now it pays once
 
     def kv(self, entry: int) -> KVView:
         """Keys and values of the schedule entry (or of the entry whose cache it reads)."""
