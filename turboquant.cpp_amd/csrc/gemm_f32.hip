@@ -12,8 +12,7 @@
 //    17 to 64 rows (a decode step of many sequences) are one row of tiles, at which multiply-adds and bytes of w
 //    are in balance; a narrow matrix is cut into runs of k so that the chip has enough workgroups.
 //  * gemm_f32_stream_kernel, for few rows (decoding; experts that few tokens chose): the work is reading w once.
-//    A workgroup owns 64 rows of w (every row of `a` that a wave fetches multiplies all of them: fetched for 16
-//    rows of w only, the rows of `a` came to four times the bytes of w and bound the kernel), its four waves split k
+//    A workgroup owns 32 rows of w (every row of `a` that a wave fetches multiplies all of them), its four waves split k
 //    and add their sums in wave order through LDS; the rows of w go from memory straight into the operand
 //    registers, by whole lines of 128 bytes and with the hint that they are read once.
 //  Runs of k of a narrow matrix leave their sums apart; a second kernel adds them up in order and finishes them.
@@ -407,9 +406,11 @@ __global__ void gemm_f32_bias_kernel(F32GemmArgs g) {
 }
 
 // Into how many runs k is cut for a plain product (one matrix, up to 64 rows): enough that a narrow matrix still
-// gives every compute unit two workgroups (of 128 columns for 17 to 64 rows, of 64 for fewer), each run keeping at
+// gives every compute unit two workgroups (of 128 columns for 17 to 64 rows, of 32 for fewer), each run keeping at
 // least 256 of k.  A function of N and K alone, so that a row's sums do not depend on how many rows there are.
-#define SNT 4            // tiles of 16 rows of w per workgroup of the few-row kernel
+// Tiles of 16 rows of w per workgroup of the few-row kernel.  Measured on the experts' gated product at 64, 128 and 240
+// tokens (60 experts of 1,408 x 2,048, 4 per token): 290, 299 and 412 us with 2; 315, 317 and 436 with 4; 272, 289 and 423 with 1.
+#define SNT 2
 static int f32_runs_of_k(int N, int K, int* k_per_split) {
   const int groups = (N + 127) / 128;
   int runs = 1;
