@@ -718,6 +718,84 @@ def test_a_mixer_with_state_of_its_own_is_registered_built_and_stepped():
         unregister_part("mixer", "toy_decay")
 
 
+@pytest.mark.parametrize("act", ACTS)
+def test_the_order_of_layers_is_a_list(act):
+    """A plan of the library's own parts whose schedule names layers twice: layer 0, layer 1, layer 0 again with keys
+    and values of its own for that run, and layer 1 again reading the keys and values that its first run wrote
+    (it writes none).  Whole prompts in an unequal batch and token by token in slots used before, against a plain
+    loop over the same list; the cache holds three runs' worth of keys and values, not four."""
+    import plain_qwen2moe as P
+    from turboquant_cpp_amd.config import LayerSpec, ModelPlan, PartSpec, ScheduleEntry, Source
+    from turboquant_cpp_amd.engine.model import CausalLM
+    from turboquant_cpp_amd.engine.step import Engine
+    from turboquant_cpp_amd.weights import TensorDict
+    H, V, INNER, nh, nkv, hd, theta = 64, 120, 96, 4, 2, 16, 10000.0
+    windows = [None, 12]
+
+    def norm(name):
+        return PartSpec("rmsnorm", dict(size=H, eps=1e-5), {"weight": Source.single(name)})
+    layers = [LayerSpec("prenorm", {
+        "mixer_norm": norm(f"l{l}.n1"), "ffn_norm": norm(f"l{l}.n2"),
+        "mixer": PartSpec("gqa_attention", dict(hidden_size=H, num_heads=nh, num_kv_heads=nkv, head_dim=hd, qkv_bias=True,
+                                                window=windows[l],
+                                                position=PartSpec("rope", dict(head_dim=hd, rotary_dim=hd, theta=theta, pairing="half"))),
+                          {"qkv_weight": Source.concat([f"l{l}.q", f"l{l}.k", f"l{l}.v"]),
+                           "qkv_bias": Source.concat([f"l{l}.qb", f"l{l}.kb", f"l{l}.vb"]), "out_weight": Source.single(f"l{l}.o")}),
+        "ffn": PartSpec("dense_swiglu", dict(hidden_size=H, inner_size=INNER),
+                        {n: Source.single(f"l{l}.{n}") for n in ("gate", "up", "down")})}) for l in range(2)]
+    schedule = [ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0), ScheduleEntry(1, cache_of=1)]
+    plan = ModelPlan("ToyLoopedLM", V, H, layers, schedule, norm("final"), Source.single("embed"), None, max_positions=512)
+    model = CausalLM(plan, act)
+    g = torch.Generator().manual_seed(81)
+    dt = torch.float32 if act == "float32" else torch.bfloat16
+    tensors = {n: ((1 + 0.1 * torch.randn(sh, generator=g)) if role == "scale" else 0.12 * torch.randn(sh, generator=g)).to(dt)
+               for n, (sh, role) in model.tensor_table().items()}
+    model.load(TensorDict(tensors), DEV)
+    eng = Engine(model, max_tokens=64 * 6, max_slots=3)
+    # runs 0, 1 and 2 keep keys and values (run 1 with a window), run 3 keeps none
+    assert sum(len(grp.entries) for grp in eng.cache.groups) == 3
+
+    def plain(tokens):
+        t = {n: v.double() for n, v in tensors.items()}
+        n, pos = len(tokens), list(range(len(tokens)))
+        x = t["embed"][tokens]
+        kept = {}
+        for run, e in enumerate(schedule):
+            l = e.layer
+            h = P.rmsnorm(x, t[f"l{l}.n1"], 1e-5)
+            q = (h @ t[f"l{l}.q"].T + t[f"l{l}.qb"]).view(n, nh, hd)
+            if e.cache_of is None:
+                k = (h @ t[f"l{l}.k"].T + t[f"l{l}.kb"]).view(n, nkv, hd)
+                v = (h @ t[f"l{l}.v"].T + t[f"l{l}.vb"]).view(n, nkv, hd)
+                kept[run] = (P.rope(k, pos, theta, "half"), v)
+            k, v = kept[run if e.cache_of is None else e.cache_of]
+            att = P.attention(P.rope(q, pos, theta, "half"), k, v, window=windows[l])
+            x = x + att.reshape(n, nh * hd) @ t[f"l{l}.o"].T
+            x = x + P.swiglu_mlp(P.rmsnorm(x, t[f"l{l}.n2"], 1e-5), t[f"l{l}.gate"], t[f"l{l}.up"], t[f"l{l}.down"])
+        return P.rmsnorm(x, t["final"], 1e-5) @ t["embed"].T
+
+    prompts = [torch.randint(0, V, (n,), generator=g).tolist() for n in (70, 3, 31)]
+    refs = [plain(p) for p in prompts]
+    bound = 1e-4 if act == "float32" else 0.04 * max(r.abs().max().item() for r in refs)
+    slots = eng.open(3)
+    lg = eng.step(slots, prompts, [list(range(len(p))) for p in prompts]).cpu().double()
+    assert (lg - torch.cat(refs)).abs().max() < bound
+    eng.close(slots)
+    slots = eng.open(3)
+    cut = [40, 1, 9]
+    eng.step(slots, [p[:c] for p, c in zip(prompts, cut)], [[] for _ in prompts])
+    pos, live = list(cut), [0, 1, 2]
+    while live:
+        lg = eng.step([slots[i] for i in live], [[prompts[i][pos[i]]] for i in live]).cpu().double()
+        for j, i in enumerate(live):
+            assert (lg[j] - refs[i][pos[i]]).abs().max() < bound, (i, pos[i])
+            pos[i] += 1
+        for i in [i for i in live if pos[i] == len(prompts[i])]:
+            eng.close([slots[i]])
+            live.remove(i)
+    assert eng.cache.n_live == 0
+
+
 def test_a_feed_forward_with_routing_and_another_position_encoding_defined_here():
     """Two more parts defined in the test and registered from here: a feed-forward that sends each token to one of
     four small experts (chosen by the largest of four router scores, relu inside), and a position encoding whose
