@@ -142,6 +142,10 @@ def build(dtype: str, force: bool = False, verbose: bool = True) -> str:
         raise BuildError(f"hipcc failed to link {target}:\n{link.stdout}")
     os.replace(tmp, target)
     shutil.rmtree(obj_dir, ignore_errors=True)
+    for old in os.listdir(out_dir):     # what a build that was killed left behind
+        pid = old.rsplit("_", 1)[-1]
+        if old.startswith("obj_") and pid.isdigit() and not os.path.exists(f"/proc/{pid}"):
+            shutil.rmtree(os.path.join(out_dir, old), ignore_errors=True)
     for old in os.listdir(out_dir):     # libraries of earlier sources
         if old.startswith(f"libtq_{dtype}-") and old.endswith(".so") and old != os.path.basename(target):
             try:
