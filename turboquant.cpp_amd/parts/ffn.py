@@ -91,10 +91,10 @@ class SparseMoE(Part):
         shared, side = None, None
         if self.shared_size > 0:
             tiles = -(-T // 128) * -(-self.shared_size // 128)
-            # (up to 64 tokens the host's part of forking and joining, 1.7 ms of a step of 24 layers, is more than the
-            # second stream gains: a prompt step of 17 tokens took 6.0 ms with it and 4.2 without, one of 128 6.7 and 7.5)
-            # A step that is being captured pays the host once and is replayed with the two streams (64 sequences: 10.8
-            # ms a step with them, 11.15 without).
+            # Up to 64 tokens the host's part of forking and joining (1.7 ms of a step of 24 layers) is more than the
+            # second stream gains: a prompt step of 17 tokens took 6.0 ms with it and 4.2 without, one of 128 tokens 6.7
+            # and 7.5.  A step that is being captured pays the host once and is replayed with the two streams (64
+            # sequences: 10.8 ms a step with them, 11.15 without).
             worth = T > 64 or getattr(ctx, "capturing", False)
             side = ctx.fork() if hasattr(ctx, "fork") and worth and tiles < 8 * 256 else None
             if side is not None:
