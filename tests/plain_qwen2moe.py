@@ -148,12 +148,13 @@ def swiglu_mlp(x: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torc
     return matvec_rows(down, silu(matvec_rows(gate, x)) * matvec_rows(up, x))
 
 
-def near_swaps(x: torch.Tensor, router: torch.Tensor, top_k: int, reach: int = 3) -> list:
+def near_swaps(x: torch.Tensor, router: torch.Tensor, top_k: int, reach: int = 3, spread: float | None = None) -> list:
     """(gap, i, j) for every chosen rank i and every rank j among the ``reach`` best left out, the gap being the
-    difference of their logits in units of the logits' spread, smallest first."""
+    difference of their logits in units of the logits' spread (the token's own, unless one is given), smallest
+    first."""
     logits = matvec_rows(router, x)
     top = torch.sort(logits, descending=True).values
-    spread = float(logits.std()) + 1e-30
+    spread = (float(logits.std()) if spread is None else spread) + 1e-30
     out = [(float(top[i] - top[j]) / spread, i, j) for i in range(top_k) for j in range(top_k, min(top_k + reach, len(top)))]
     return sorted(out)
 
@@ -164,10 +165,14 @@ def moe(x: torch.Tensor, w: dict, top_k: int, renormalize: bool, margins: list |
     (/root/reference/src/engine/tq_moe.c:720,864-999); then + sigmoid(x . shared_scale) * shared(x)
     (tq_moe.c:1005-1058)."""
     out = torch.zeros_like(x)
+    # with two experts a token's own spread is the gap itself: there the unit is the spread over all the step's tokens
+    spread = None
+    if swaps is not None and w["router"].shape[0] == 2 and x.shape[0] > 1:
+        spread = float(torch.stack([matvec_rows(w["router"], x[t]) for t in range(x.shape[0])]).std())
     for t in range(x.shape[0]):
         ids, wts = route(x[t], w["router"], top_k, renormalize, other_side=(other_side or {}).get(t))
         if swaps is not None:
-            swaps.append(near_swaps(x[t], w["router"], top_k))
+            swaps.append(near_swaps(x[t], w["router"], top_k, spread=spread))
         if margins is not None:
             margins.append(route_margin(x[t], w["router"], top_k))
         acc = torch.zeros_like(x[t])
