@@ -278,3 +278,34 @@ def test_random_weights_are_a_function_of_seed_tensor_and_element(tmp_path):
             loaded.load(f, "cpu")
         for a, b in zip(drawn.bindings, loaded.bindings):
             assert torch.equal(getattr(a.owner, a.attr), getattr(b.owner, b.attr)), a.path
+
+
+def test_the_header_the_sources_and_the_python_face_name_the_same_entry_points():
+    """Every exported function of the kernel sources is declared in `csrc/turboquant_kernels.h` (or `no_alloc.h`) with
+    as many arguments as its definition has, and `ops.py` gives ctypes that many argument types."""
+    import glob
+    import os
+    import re
+    from turboquant_cpp_amd.csrc import ops
+    csrc = os.path.dirname(ops.__file__)
+
+    def declared(text, pattern):
+        found = {}
+        for m in re.finditer(pattern, text):
+            args = " ".join(m.group(2).split())
+            found[m.group(1)] = 0 if args in ("", "void") else args.count(",") + 1
+        return found
+
+    defined = {}
+    for f in glob.glob(os.path.join(csrc, "*.hip")):
+        defined.update(declared(open(f).read(), r"TQ_API\s+[\w\s\*]+?\s+(tq_\w+)\s*\(([^)]*)\)\s*\{"))
+    header = {}
+    for name in ("turboquant_kernels.h", "no_alloc.h"):
+        header.update(declared(open(os.path.join(csrc, name)).read(), r"\b(tq_\w+)\s*\(([^)]*)\)\s*;"))
+    assert defined == header, {k: (defined.get(k), header.get(k)) for k in set(defined) | set(header)
+                               if defined.get(k) != header.get(k)}
+    python = {**ops._SIGNATURES, **ops._OPTIONAL}
+    for name, n_args in defined.items():
+        if name in python:
+            assert len(python[name]) == n_args, (name, len(python[name]), n_args)
+    assert set(python) <= set(defined), set(python) - set(defined)
