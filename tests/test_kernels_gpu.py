@@ -87,19 +87,94 @@ def ref_gemm(a, w, bias=None, w2=None):
 @pytest.mark.parametrize("M,N,K", [(5, 33, 50), (1, 50, 72), (5, 130, 200), (16, 64, 64), (17, 33, 136), (40, 257, 264),
                                    (64, 96, 1000), (65, 130, 72), (200, 300, 520), (300, 129, 64), (1130, 7400, 136), (2048, 4096, 72)])
 @pytest.mark.parametrize("mode", ["plain", "bias", "gated"])
-def test_gemm_dense(ops, act, M, N, K, mode):
+def test_gemm_dense(ops, act, M, N, K, mode, monkeypatch):
     a = rnd((M, K), adt(act), 10)
     w = rnd((N, K), adt(act), 11, 0.2)
     bias = rnd((N,), adt(act), 12) if mode == "bias" else None
     w2 = rnd((N, K), adt(act), 13, 0.2) if mode == "gated" else None
-    for out_act in (False, True):
-        y = ops.gemm(a.to(DEV), w.to(DEV), act, bias=None if bias is None else bias.to(DEV),
-                     w2=None if w2 is None else w2.to(DEV), out_act=out_act).cpu()
-        ref = ref_gemm(a, w, bias, w2)
-        scale = ref.abs().max().item()
-        err = (y.double() - ref).abs().max().item()
-        limit = 1e-5 * scale * math.sqrt(K) if act == "float32" else (2e-2 if out_act else 4e-3) * scale
-        assert err < limit, (err, scale)
+    # where the vendor library would take the product, this library's own kernel is held to the same bound
+    for vendor in (True, False) if ops._vendor_product(act, a.to(DEV), w.to(DEV), M, K) and mode == "plain" else (True,):
+        monkeypatch.setattr(ops, "_VENDOR", vendor)
+        for out_act in (False, True):
+            y = ops.gemm(a.to(DEV), w.to(DEV), act, bias=None if bias is None else bias.to(DEV),
+                         w2=None if w2 is None else w2.to(DEV), out_act=out_act).cpu()
+            ref = ref_gemm(a, w, bias, w2)
+            scale = ref.abs().max().item()
+            err = (y.double() - ref).abs().max().item()
+            limit = 1e-5 * scale * math.sqrt(K) if act == "float32" else (2e-2 if out_act else 4e-3) * scale
+            assert err < limit, (err, scale, vendor)
+
+
+@pytest.mark.parametrize("M,N,K", [(512, 130, 264), (700, 6144, 2048), (2048, 257, 1000), (8192, 96, 16384), (600, 96, 16384)])
+def test_plain_products_of_many_rows(ops, M, N, K, monkeypatch):
+    """From 512 rows on a plain bfloat16 product without bias goes to the vendor's library unless k is long and the
+    rows are not many; its result and the own kernel's are the same product in another order of sums.  Gated
+    products, products with a bias and the 32-bit path stay; TQ_PLAIN_PRODUCTS=own (read at import) keeps all."""
+    act = "bfloat16"
+    a, w = rnd((M, K), adt(act), 14).to(DEV), rnd((N, K), adt(act), 15, 0.2).to(DEV)
+    calls = []
+    real = torch.mm
+    monkeypatch.setattr(torch, "mm", lambda *x, **kw: (calls.append(1), real(*x, **kw))[1])
+    taken = ops._vendor_product(act, a, w, M, K)
+    assert taken == (K < 16384 or M >= 8192)
+    got = ops.gemm(a, w, act, partial_sums=True)
+    assert len(calls) == (1 if taken else 0) and got.shape[1:] == (M, N) and got.dtype == torch.float32
+    ref = ref_gemm(a.cpu(), w.cpu())
+    scale = ref.abs().max().item()
+    assert (got.sum(0).cpu().double() - ref).abs().max().item() < 4e-3 * scale
+    assert ops.gemm(a, w, act, out_act=True).dtype == torch.bfloat16
+    n = len(calls)
+    ops.gemm(a, w, act, bias=w[:, 0].contiguous())
+    ops.gemm(a, w, act, w2=w, out_act=True)
+    ops.gemm(a.float(), w.float(), "float32")
+    assert len(calls) == n
+    monkeypatch.setattr(ops, "_VENDOR", False)
+    own = ops.gemm(a, w, act)
+    assert len(calls) == n and (own.cpu().double() - ref).abs().max().item() < 4e-3 * scale
+
+
+@pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("activation", ["silu", "gelu_tanh", "relu2"])
+@pytest.mark.parametrize("M,N,ld", [(3, 40, 80), (70, 33, 70), (5, 1028, 2056), (9, 10, 21)])
+def test_the_gate_applied_afterwards(ops, act, activation, M, N, ld):
+    gu = rnd((M, ld), torch.float32, 16, 2.0).to(DEV)
+    out = torch.empty((M, N), dtype=adt(act), device=DEV)
+    ops._run("gated_act", ops.library(act).tq_gated_act(gu.data_ptr(), ld, out.data_ptr(), M, N, ops.GATES[activation],
+                                                        ops._stream()))
+    g, u = gu[:, :N].cpu().double(), gu[:, N:2 * N].cpu().double()
+    f = {"silu": torch.nn.functional.silu, "relu2": lambda v: torch.relu(v) ** 2,
+         "gelu_tanh": lambda v: torch.nn.functional.gelu(v, approximate="tanh")}[activation]
+    ref = f(g) * u
+    assert (out.cpu().double() - ref).abs().max().item() < (1e-5 if act == "float32" else 8e-3) * ref.abs().max().item()
+    assert ops.library(act).tq_gated_act(gu.data_ptr(), 2 * N - 1, out.data_ptr(), M, N, 0, ops._stream()) != 0
+
+
+@pytest.mark.parametrize("activation", ["silu", "gelu_tanh"])
+@pytest.mark.parametrize("M,N,K", [(512, 130, 264), (5000, 96, 72), (700, 1408, 2048)])
+def test_gated_pairs_of_many_rows(ops, activation, M, N, K, monkeypatch):
+    """A gated pair whose second matrix lies right behind the first goes, from 512 rows on, to the vendor's library
+    as one product over both, a few thousand rows at a time, with the gate in a pass of its own; matrices that lie
+    apart stay in this library's kernel.  Both are the same function."""
+    act = "bfloat16"
+    a = rnd((M, K), adt(act), 17).to(DEV)
+    w, w2 = rnd((N, K), adt(act), 18, 0.2).to(DEV), rnd((N, K), adt(act), 19, 0.2).to(DEV)
+    g, u = ops.side_by_side(w, w2)
+    assert torch.equal(g, w) and torch.equal(u, w2) and ops._behind(g, u) and not ops._behind(w, w2) and not ops._behind(u, g)
+    calls = []
+    real = torch.mm
+    monkeypatch.setattr(torch, "mm", lambda *x, **kw: (calls.append(x[0].shape[0]), real(*x, **kw))[1])
+    monkeypatch.setattr(ops, "VENDOR_GATED_ROWS", 2048)
+    got = ops.gemm(a, g, act, w2=u, out_act=True, activation=activation)
+    assert calls == [min(2048, M - r) for r in range(0, M, 2048)]
+    own = ops.gemm(a, w, act, w2=w2, out_act=True, activation=activation)
+    assert len(calls) == -(-M // 2048)
+    f = torch.nn.functional.silu if activation == "silu" else lambda v: torch.nn.functional.gelu(v, approximate="tanh")
+    ref = f(a.cpu().double() @ w.cpu().double().T) * (a.cpu().double() @ w2.cpu().double().T)
+    scale = ref.abs().max().item()
+    for y in (got, own):
+        assert y.dtype == torch.bfloat16 and (y.cpu().double() - ref).abs().max().item() < 2e-2 * scale
+    ops.gemm(a, g, act, w2=u)          # into float32: this library's kernel
+    assert len(calls) == -(-M // 2048)
 
 
 @pytest.mark.parametrize("act", ACTS)
@@ -434,6 +509,73 @@ def test_rope_kv_write(ops, act, pairing, rot):
         assert (vc[vbase:vbase + hd * page:page].double() - x[t, nh + nkv]).abs().max() < tol(act, 4)
     # nothing outside the written rows was touched
     assert int((kc != 0).sum()) <= T * nkv * hd and int((vc != 0).sum()) <= T * nkv * hd
+
+
+@pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("bias_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,hd,page", [(3, 1, 48, 64), (2, 2, 18, 64)])
+def test_rotation_adds_a_bias_that_the_product_left_out(ops, act, bias_dtype, nh, nkv, hd, page):
+    """Given the bias, the rotation kernel reads qkv + bias: queries and pages hold the bits they hold when the
+    bias was added beforehand, token by token and by tiles of a run's values."""
+    from plain_qwen2moe import rope_frequencies
+    starts, news = [0, 37, 5], [150, 100, 9]
+    lens = [a + b for a, b in zip(starts, news)]
+    table, slots, page_stride, kp, vp = paged_setup(lens, page, nkv, hd, 2, act, 112)
+    off = nkv * page * hd
+    T = sum(news)
+    width = (nh + 2 * nkv) * hd
+    qkv = rnd((T, width), torch.float32, 113).to(DEV)
+    bias = rnd((width,), bias_dtype, 114).to(DEV)
+    positions = torch.cat([torch.arange(a, a + b) for a, b in zip(starts, news)]).to(torch.int32)
+    slot_of = torch.cat([torch.full((b,), s) for s, b in zip(slots, news)]).to(torch.int32)
+    freqs = torch.from_numpy(rope_frequencies(hd, 1e4))
+    cu = torch.tensor([0] + list(torch.tensor(news).cumsum(0)), dtype=torch.int32)
+    runs = {"cu_seqlens": cu.to(DEV), "slots": torch.tensor(slots, dtype=torch.int32).to(DEV),
+            "start": torch.tensor(starts, dtype=torch.int32).to(DEV), "max_new": max(news), "max_end": max(lens), "decode": False}
+    for r in (None, runs):
+        got = []
+        for late in (True, False):
+            kd, vd = kp.to(DEV).clone(), vp.to(DEV).clone()
+            q = ops.rope_kv_write(qkv if late else qkv + bias.float(), positions.to(DEV), slot_of.to(DEV), table.to(DEV),
+                                  freqs.to(DEV), 0, hd, kd, vd, off, page, page_stride, nh, nkv, hd, act, runs=r,
+                                  bias=bias if late else None)
+            got.append((q.cpu(), kd.cpu(), vd.cpu()))
+        for x, y in zip(*got):
+            assert torch.equal(x, y)
+        assert not torch.equal(got[0][0], ops.rope_kv_write(qkv, positions.to(DEV), slot_of.to(DEV), table.to(DEV),
+                                                            freqs.to(DEV), 0, hd, None, None, off, page, page_stride, nh,
+                                                            nkv, hd, act).cpu())
+    with pytest.raises(ops.KernelError, match="bias"):
+        ops.rope_kv_write(qkv, positions.to(DEV), slot_of.to(DEV), table.to(DEV), freqs.to(DEV), 0, hd, None, None, off, page,
+                          page_stride, nh, nkv, hd, act, bias=bias[:-1])
+
+
+@pytest.mark.parametrize("T", [700])
+def test_queries_keys_values_of_a_long_prompt(ops, T, monkeypatch):
+    """A long prompt's product of q, k and v goes to the vendor's library without its bias, which the rotation adds:
+    queries and pages are those of this library's own product with the bias in it, up to the order of sums."""
+    from plain_qwen2moe import rope_frequencies
+    act, nh, nkv, hd, H, page = "bfloat16", 6, 2, 64, 264, 64
+    table, slots, page_stride, kp, vp = paged_setup([T], page, nkv, hd, 1, act, 174)
+    a = rnd((T, H), adt(act), 175).to(DEV)
+    w = rnd(((nh + 2 * nkv) * hd, H), adt(act), 176, 0.2).to(DEV)
+    b = rnd(((nh + 2 * nkv) * hd,), adt(act), 177).to(DEV)
+    positions = torch.arange(T, dtype=torch.int32).to(DEV)
+    slot_of = torch.full((T,), slots[0], dtype=torch.int32).to(DEV)
+    freqs = torch.from_numpy(rope_frequencies(hd, 1e6)).to(DEV)
+    out = []
+    for vendor in (True, False):
+        monkeypatch.setattr(ops, "_VENDOR", vendor)
+        kd, vd = kp.to(DEV).clone(), vp.to(DEV).clone()
+        q = ops.qkv_rope_write(a, w, b, positions, slot_of, table.to(DEV), freqs, 0, hd, kd, vd, 0, page, page_stride, nh, nkv,
+                               hd, act)
+        out.append((q.cpu().float(), kd.cpu().float(), vd.cpu().float()))
+    scale = out[1][0].abs().max().item()
+    for x, y in zip(*out):
+        assert (x - y).abs().max().item() <= 1.6e-2 * scale
+    nobias = ops.qkv_rope_write(a, w, None, positions, slot_of, table.to(DEV), freqs, 0, hd, None, None, 0, page, page_stride,
+                                nh, nkv, hd, act).cpu().float()
+    assert (nobias - out[0][0]).abs().max().item() > 0.1 * scale
 
 
 @pytest.mark.parametrize("act", ACTS)

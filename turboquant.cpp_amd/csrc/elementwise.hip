@@ -204,6 +204,39 @@ TQ_API int tq_add_rmsnorm(float* x, const float* delta, int S, int64_t delta_str
   return 0;
 }
 
+// ---------------------------------------------------------------- the gate of a gated pair, applied afterwards
+// out[m][n] = f(gu[m][n]) * gu[m][N + n]: for a pair of products that came out of one plain product over the two
+// matrices laid one behind the other (a library's, which has no such epilogue).  gu is float32 with row stride ld.
+template <bool VEC>
+__global__ __launch_bounds__(256) void gated_act_kernel(const float* __restrict__ gu, int64_t ld, act_t* __restrict__ out,
+                                                        int N, int gate) {
+  const float* row = gu + (size_t)blockIdx.y * ld;
+  act_t* dst = out + (size_t)blockIdx.y * N;
+  if (VEC) {
+    const int n = (blockIdx.x * 256 + threadIdx.x) * 4;
+    if (n >= N) return;
+    const f32x4 g = load4f(row + n), u = load4f(row + N + n);
+    store4(dst + n, f32x4{gate_fn(g.x, gate) * u.x, gate_fn(g.y, gate) * u.y, gate_fn(g.z, gate) * u.z,
+                          gate_fn(g.w, gate) * u.w});
+  } else {
+    const int n = blockIdx.x * 256 + threadIdx.x;
+    if (n < N) dst[n] = from_f32<act_t>(gate_fn(row[n], gate) * row[N + n]);
+  }
+}
+
+TQ_API int tq_gated_act(const float* gu, int64_t ld, void* out, int M, int N, int gate, hipStream_t st) {
+  if (M <= 0 || N <= 0) return 0;
+  if (gate < 0 || gate >= TQ_GATE_COUNT || ld < 2 * (int64_t)N) return TQ_ERR_BAD_ARG;
+  if (M > 65535) return TQ_ERR_UNSUPPORTED;
+  const bool vec = N % 4 == 0 && ld % 4 == 0 && ((uintptr_t)gu % 16) == 0 && ((uintptr_t)out % 16) == 0;
+  if (vec)
+    hipLaunchKernelGGL(gated_act_kernel<true>, dim3((N / 4 + 255) / 256, M), dim3(256), 0, st, gu, ld, (act_t*)out, N, gate);
+  else
+    hipLaunchKernelGGL(gated_act_kernel<false>, dim3((N + 255) / 256, M), dim3(256), 0, st, gu, ld, (act_t*)out, N, gate);
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
 // ---------------------------------------------------------------- RMS norm of every head of q and k
 // qkv[t] holds, in float, nh query heads, then nkv key heads, then nkv value heads of hd each.  Every query head is
 // normed over its hd values with the weights wq[hd], every key head with wk[hd] (a null pointer leaves those heads
@@ -250,7 +283,14 @@ TQ_API int tq_head_rmsnorm(float* qkv, const void* wq, const void* wk, int wtype
 // A workgroup of four waves takes `spb` heads of one token (grid (T, ceil(heads / spb))); a wave takes every
 // fourth of them and turns pair i of all its heads with one sine and cosine.  write_kv: 0 queries only, 1 keys
 // and values, 2 keys only (the values of whole runs of tokens go through v_write_tile_kernel below).
-__global__ __launch_bounds__(256) void rope_kv_write_kernel(const float* __restrict__ qkv, const int* __restrict__ positions,
+// element i of a bias that the product before did not add (null: none); float32 or bfloat16 as bias_type says
+__device__ __forceinline__ float bias_elem(const void* bias, int bias_type, size_t i) {
+  if (!bias) return 0.f;
+  return bias_type == TQ_F32 ? ((const float*)bias)[i] : to_f32(((const bf16_t*)bias)[i]);
+}
+
+__global__ __launch_bounds__(256) void rope_kv_write_kernel(const float* __restrict__ qkv, const void* __restrict__ bias,
+                                     int bias_type, const int* __restrict__ positions,
                                      const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
                                      int bt_stride, const float* __restrict__ inv_freq, int pairing, int rot,
                                      act_t* __restrict__ q_out, act_t* __restrict__ k_pool,
@@ -283,7 +323,8 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(const float* __restr
     for (int s = s0; s < rot_end; s += 4) {
       const float* src = src_t + (size_t)s * hd;
       act_t* dst = s < nh ? q_t + (size_t)s * hd : k_t + (size_t)(s - nh) * kv_head_stride;
-      const float a = src[ia], b = src[ib];
+      const float a = src[ia] + bias_elem(bias, bias_type, (size_t)s * hd + ia);
+      const float b = src[ib] + bias_elem(bias, bias_type, (size_t)s * hd + ib);
       dst[ia] = from_f32<act_t>(a * cs - b * sn);
       dst[ib] = from_f32<act_t>(a * sn + b * cs);
     }
@@ -291,14 +332,16 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(const float* __restr
   for (int s = s0; s < rot_end; s += 4) {      // dimensions from rot on pass through
     const float* src = src_t + (size_t)s * hd;
     act_t* dst = s < nh ? q_t + (size_t)s * hd : k_t + (size_t)(s - nh) * kv_head_stride;
-    for (int i = rot + lane; i < hd; i += TQ_WAVE) dst[i] = from_f32<act_t>(src[i]);
+    for (int i = rot + lane; i < hd; i += TQ_WAVE)
+      dst[i] = from_f32<act_t>(src[i] + bias_elem(bias, bias_type, (size_t)s * hd + i));
   }
   if (write_kv != 1) return;
   for (int s = s0; s < s1; s += 4) {           // values lie transposed, [hd][row]
     if (s < nh + nkv) continue;
     const float* src = src_t + (size_t)s * hd;
     act_t* col = v_t + (size_t)(s - nh - nkv) * kv_head_stride;
-    for (int i = lane; i < hd; i += TQ_WAVE) col[(size_t)i * page_size] = from_f32<act_t>(src[i]);
+    for (int i = lane; i < hd; i += TQ_WAVE)
+      col[(size_t)i * page_size] = from_f32<act_t>(src[i] + bias_elem(bias, bias_type, (size_t)s * hd + i));
   }
 }
 
@@ -309,6 +352,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(const float* __restr
 #define VT_POS 64
 template <int VEC>      // positions per 16-byte store
 __global__ __launch_bounds__(256) void v_write_tile_kernel(const float* __restrict__ qkv,
+                                                           const void* __restrict__ bias, int bias_type,
                                                            const int* __restrict__ cu_seqlens,
                                                            const int* __restrict__ slots,
                                                            const int* __restrict__ start,
@@ -327,6 +371,7 @@ __global__ __launch_bounds__(256) void v_write_tile_kernel(const float* __restri
   const int heads = nh + 2 * nkv;
   const float* src0 = qkv + ((size_t)(t0 + lo - st) * heads + nh + nkv + h) * hd;      // value row of position lo
   const size_t row_stride = (size_t)heads * hd;
+  const size_t bias0 = (size_t)(nh + nkv + h) * hd;      // the bias of this value head
   if (hd % 4 == 0) {        // 16 bytes of a row per thread and turn, all of a thread's loads on their way at once
     const int q4 = hd / 4, total = (hi - lo) * q4;
 #pragma unroll 8
@@ -334,14 +379,15 @@ __global__ __launch_bounds__(256) void v_write_tile_kernel(const float* __restri
       const int r = idx / q4, d = (idx % q4) * 4;
       const f32x4 v = load4f(src0 + r * row_stride + d);
       act_t* to = ts + d * TS + (lo + r - P0);
-      to[0] = from_f32<act_t>(v.x);
-      to[TS] = from_f32<act_t>(v.y);
-      to[2 * TS] = from_f32<act_t>(v.z);
-      to[3 * TS] = from_f32<act_t>(v.w);
+      to[0] = from_f32<act_t>(v.x + bias_elem(bias, bias_type, bias0 + d));
+      to[TS] = from_f32<act_t>(v.y + bias_elem(bias, bias_type, bias0 + d + 1));
+      to[2 * TS] = from_f32<act_t>(v.z + bias_elem(bias, bias_type, bias0 + d + 2));
+      to[3 * TS] = from_f32<act_t>(v.w + bias_elem(bias, bias_type, bias0 + d + 3));
     }
   } else {
     for (int r = wave; r < hi - lo; r += 4)
-      for (int d = lane; d < hd; d += TQ_WAVE) ts[d * TS + (lo + r - P0)] = from_f32<act_t>(src0[r * row_stride + d]);
+      for (int d = lane; d < hd; d += TQ_WAVE)
+        ts[d * TS + (lo + r - P0)] = from_f32<act_t>(src0[r * row_stride + d] + bias_elem(bias, bias_type, bias0 + d));
   }
   __syncthreads();
   const int page = block_table[(size_t)slots[b] * bt_stride + P0 / page_size];
@@ -362,13 +408,15 @@ __global__ __launch_bounds__(256) void v_write_tile_kernel(const float* __restri
 
 // cu_seqlens, slots, start (null, or [B + 1], [B], [B] with max_new the longest run): the tokens as runs of
 // consecutive positions, one per sequence; given for whole prompts, they let the values go by tiles.
-TQ_API int tq_rope_kv_write(const float* qkv, const int* positions, const int* seq_of_token,
+// bias (null, or [(nh + 2 nkv) * hd] of bias_type): added to qkv as it is read, for a product that left it out.
+TQ_API int tq_rope_kv_write(const float* qkv, const void* bias, int bias_type, const int* positions, const int* seq_of_token,
                             const int* block_table, int bt_stride, const float* inv_freq, int pairing, int rot,
                             void* q_out, void* k_pool, void* v_pool, int page_size, int64_t page_stride, int T,
                             int nh, int nkv, int hd, int write_kv, const int* cu_seqlens, const int* slots,
                             const int* start, int B, int max_new, hipStream_t st) {
   if (T <= 0) return 0;
   if (rot < 0 || rot > hd || (rot & 1) || (pairing != 0 && pairing != 1)) return TQ_ERR_BAD_ARG;
+  if (bias && bias_type != TQ_F32 && bias_type != TQ_BF16) return TQ_ERR_BAD_ARG;
   constexpr int VEC = 16 / (int)sizeof(act_t);
   const size_t vt_shmem = (size_t)hd * (VT_POS + VEC) * sizeof(act_t);
   const bool tiles = write_kv && cu_seqlens && slots && start && B > 0 && B <= 65535 && nkv <= 65535 && max_new > 8 &&
@@ -379,15 +427,15 @@ TQ_API int tq_rope_kv_write(const float* qkv, const int* positions, const int* s
   int spb = 4;
   while (spb < heads && (int64_t)T * ((heads + spb - 1) / spb) > 4096) spb *= 2;
   if ((heads + spb - 1) / spb > 65535) return TQ_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL(rope_kv_write_kernel, dim3(T, (heads + spb - 1) / spb), dim3(256), 0, st, qkv, positions,
-                     seq_of_token, block_table, bt_stride, inv_freq, pairing, rot, (act_t*)q_out, (act_t*)k_pool,
+  hipLaunchKernelGGL(rope_kv_write_kernel, dim3(T, (heads + spb - 1) / spb), dim3(256), 0, st, qkv, bias,
+                     bias_type, positions, seq_of_token, block_table, bt_stride, inv_freq, pairing, rot, (act_t*)q_out, (act_t*)k_pool,
                      (act_t*)v_pool, page_size, page_stride, nh, nkv, hd, write_kv, spb);
   TQ_LAUNCH_CHECK();
   if (tiles) {
     if (vt_shmem > 48 * 1024)
       (void)hipFuncSetAttribute((const void*)v_write_tile_kernel<VEC>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)vt_shmem);
     hipLaunchKernelGGL(v_write_tile_kernel<VEC>, dim3((max_new + VT_POS - 1) / VT_POS + 1, nkv, B), dim3(256), vt_shmem,
-                       st, qkv, cu_seqlens, slots, start, block_table, bt_stride, (act_t*)v_pool, page_size,
+                       st, qkv, bias, bias_type, cu_seqlens, slots, start, block_table, bt_stride, (act_t*)v_pool, page_size,
                        page_stride, nh, nkv, hd);
     TQ_LAUNCH_CHECK();
   }

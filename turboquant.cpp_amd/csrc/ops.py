@@ -10,6 +10,7 @@ from __future__ import annotations
 import ctypes
 import dataclasses
 import math
+import os
 
 import torch
 
@@ -30,10 +31,11 @@ _c_int, _c_i64, _c_f32, _c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, c
 _SIGNATURES = {
     "tq_embed": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_f32, _c_ptr],
     "tq_softcap": [_c_ptr, _c_i64, _c_f32, _c_ptr],
+    "tq_gated_act": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "tq_head_rmsnorm": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_f32, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "tq_add_rmsnorm": [_c_ptr, _c_ptr, _c_int, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_f32,
                        _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr],
-    "tq_rope_kv_write": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
+    "tq_rope_kv_write": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
                          _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
                          _c_ptr],
     "tq_moe_combine": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
@@ -263,8 +265,10 @@ def head_rmsnorm(qkv: torch.Tensor, q_weight: torch.Tensor | None, k_weight: tor
 def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor,
                   inv_freq: torch.Tensor, pairing: int, rotary_dim: int, k_pages: torch.Tensor | None,
                   v_pages: torch.Tensor | None, layer_offset: int, page_size: int, page_stride: int,
-                  num_heads: int, num_kv_heads: int, head_dim: int, act, runs: dict | None = None) -> torch.Tensor:
+                  num_heads: int, num_kv_heads: int, head_dim: int, act, runs: dict | None = None,
+                  bias: torch.Tensor | None = None) -> torch.Tensor:
     """Rotates queries and keys, returns the queries [T, nh*hd] and writes keys and values into the pages.
+    ``bias`` [width] is added to ``qkv`` as it is read, for a product that left its bias out.
     ``k_pages``/``v_pages`` are the flat page pools of the cache group (None: nothing is written, for a
     layer that reads another layer's cache); ``layer_offset`` is the layer's offset inside a page.  ``runs``
     (as for ``attention``) describes the tokens as one run of consecutive positions per sequence; with it the
@@ -273,6 +277,8 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torc
     T = positions.numel()
     width = (num_heads + 2 * num_kv_heads) * head_dim
     _check(qkv, k, "qkv", torch.float32, (T, width))
+    if bias is not None:
+        _check(bias, k, "bias", tuple(_WTYPE), (width,))
     _check(positions, k, "positions", torch.int32, (T,))
     _check(seq_of_token, k, "seq_of_token", torch.int32, (T,))
     _check(block_table, k, "block_table", torch.int32)
@@ -298,7 +304,8 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torc
         _check(slots, k, "slots", torch.int32, (B,))
         _check(start, k, "start", torch.int32, (B,))
         _need(int(runs["max_end"]) <= block_table.shape[1] * page_size, k, "positions reach beyond the page table")
-    _run(k, library(act).tq_rope_kv_write(_ptr(qkv), _ptr(positions), _ptr(seq_of_token), _ptr(block_table),
+    _run(k, library(act).tq_rope_kv_write(_ptr(qkv), _ptr(bias), _WTYPE[bias.dtype] if bias is not None else 0,
+                                          _ptr(positions), _ptr(seq_of_token), _ptr(block_table),
                                           block_table.shape[1], _ptr(inv_freq), pairing, rotary_dim, _ptr(q), kp, vp,
                                           page_size, page_stride, T, num_heads, num_kv_heads, head_dim, int(write),
                                           _ptr(cu), _ptr(slots), _ptr(start), B, max_new, _stream()))
@@ -320,9 +327,12 @@ def qkv_rope_write(a: torch.Tensor, qkv_weight: torch.Tensor, qkv_bias: torch.Te
              and head_dim % 32 == 0 and _use_mfma(act, a, qkv_weight, K)
              and (qkv_bias is None or qkv_bias.dtype in _WTYPE))
     if not fused:
-        qkv = gemm(a, qkv_weight, act, bias=qkv_bias)
+        # the vendor library's product has no bias of its own that costs nothing: the rotation adds it as it reads
+        late = qkv_bias is not None and a.dim() == 2 and _vendor_product(act, a, qkv_weight, T, K)
+        qkv = gemm(a, qkv_weight, act, bias=None if late else qkv_bias)
         return rope_kv_write(qkv, positions, seq_of_token, block_table, inv_freq, pairing, rotary_dim, k_pages, v_pages,
-                             layer_offset, page_size, page_stride, num_heads, num_kv_heads, head_dim, act, runs=runs)
+                             layer_offset, page_size, page_stride, num_heads, num_kv_heads, head_dim, act, runs=runs,
+                             bias=qkv_bias if late else None)
     adt = ACT_DTYPES[dtype_name(act)]
     width = (num_heads + 2 * num_kv_heads) * head_dim
     _check(a, k, "a", adt)
@@ -427,6 +437,59 @@ def _gemm_problem(k: str, a, w, act, bias, w2, out_act, a_rows, tile_group, n_ti
     return M, N, K, tile_rows, gstride
 
 
+# Plain bfloat16 products of many rows may go through the vendor's matrix library (hipBLASLt behind torch.mm), as the
+# reference's engine hands its products to a BLAS (/root/reference/src/engine/tq_ops.c:1088-1131): measured on
+# gfx950 it is 25 to 35 % faster than the tile kernel here from 512 rows on ([2048, 2048] x [6144, 2048]: 48 against
+# 63 us; 13,199 rows: 282 against 401), slower or equal below and where k is long and the rows are not many
+# ([4096, 20480] x [3584, 20480]: 724 against 687 us).  TQ_PLAIN_PRODUCTS=own keeps every product in this
+# library's kernels.  Products over experts, gated pairs, products with a bias that nothing behind them can add,
+# products of few rows, steps under graph capture and the 32-bit path never leave them.
+VENDOR_MIN_ROWS = 512
+_VENDOR = os.environ.get("TQ_PLAIN_PRODUCTS", "vendor") != "own"
+
+
+def _vendor_product(act, a, w, M: int, K: int) -> bool:
+    return (_VENDOR and M >= VENDOR_MIN_ROWS and (K < 16384 or M >= 8192) and dtype_name(act) == "bfloat16"
+            and w.dtype == torch.bfloat16 and a.stride(1) == 1 and w.is_contiguous()
+            and not torch.cuda.is_current_stream_capturing())
+
+
+def _vendor_gemm(a, w, out_act: bool) -> torch.Tensor:
+    """a w^T by the vendor library: sums in float32, stored as bfloat16 or float32.  It adds no bias: its product
+    with one takes a pass more over the result (77 against 48 us), so a product with a bias stays here unless the
+    caller has a kernel behind it that adds the bias on its way."""
+    return torch.mm(a, w.t()) if out_act else torch.mm(a, w.t(), out_dtype=torch.float32)
+
+
+VENDOR_GATED_ROWS = 4096      # rows of a gated pair that go through the vendor library at a time
+
+
+def side_by_side(first: torch.Tensor, second: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """The two matrices of a gated pair in one piece of memory, the second right behind the first: so laid, ``gemm``
+    may hand a pair of many rows to the vendor library as one product over both."""
+    both = torch.cat([first, second])
+    return both[:first.shape[0]], both[first.shape[0]:]
+
+
+def _behind(w: torch.Tensor, w2: torch.Tensor) -> bool:
+    return (w2.is_contiguous() and w2.untyped_storage().data_ptr() == w.untyped_storage().data_ptr()
+            and w2.data_ptr() == w.data_ptr() + w.numel() * w.element_size())
+
+
+def _vendor_gated(a, w, N: int, K: int, gate: int, act) -> torch.Tensor:
+    """f(a w^T) * (a w2^T) with w2 behind w: one product of the vendor library over both matrices into float32, a
+    few thousand rows at a time, and the gate's activation in a pass of its own."""
+    both = torch.as_strided(w, (2 * N, K), (K, 1))
+    M = a.shape[0]
+    out = torch.empty((M, N), dtype=ACT_DTYPES[dtype_name(act)], device=a.device)
+    lib = library(act)
+    for r in range(0, M, VENDOR_GATED_ROWS):
+        rows = min(VENDOR_GATED_ROWS, M - r)
+        gu = torch.mm(a[r:r + rows], both.t(), out_dtype=torch.float32)
+        _run("gated_act", lib.tq_gated_act(_ptr(gu), 2 * N, _ptr(out[r:]), rows, N, gate, _stream()))
+    return out
+
+
 def _gate_code(k: str, activation: str) -> int:
     _need(activation in GATES, k, lambda: f"unknown activation {activation!r}; known: {', '.join(sorted(GATES))}")
     return GATES[activation]
@@ -463,6 +526,12 @@ def gemm(a: torch.Tensor, w: torch.Tensor, act, bias: torch.Tensor | None = None
               "partial sums are for plain products into float32")
     lib = library(act)
     gate = _gate_code(k, activation)
+    if not grouped and a_rows is None and bias is None and _vendor_product(act, a, w, M, K):
+        if w2 is None:
+            out = _vendor_gemm(a, w, out_act)
+            return out[None] if partial_sums else out
+        if out_act and _behind(w, w2):
+            return _vendor_gated(a, w, N, K, gate, act)
     if _use_mfma(act, a, w, K) and (bias is None or bias.dtype in _WTYPE):
         splits = lib.tq_gemm_mfma_splits(M, N, K) if partial_sums else 1
         out = torch.empty((splits, M, N) if partial_sums else (M, N), dtype=adt if out_act else torch.float32,

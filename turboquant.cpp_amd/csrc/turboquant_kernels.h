@@ -26,10 +26,12 @@ int tq_add_rmsnorm(float* x, const float* delta, int S, int64_t delta_stride, co
         int R, void* out, float* out32, int H, hipStream_t st);
 int tq_head_rmsnorm(float* qkv, const void* wq, const void* wk, int wtype, float eps, int T, int nh, int nkv,
         int hd, hipStream_t st);
-int tq_rope_kv_write(const float* qkv, const int* positions, const int* seq_of_token, const int* block_table,
-        int bt_stride, const float* inv_freq, int pairing, int rot, void* q_out, void* k_pool, void* v_pool,
-        int page_size, int64_t page_stride, int T, int nh, int nkv, int hd, int write_kv, const int* cu_seqlens,
-        const int* slots, const int* start, int B, int max_new, hipStream_t st);
+int tq_gated_act(const float* gu, int64_t ld, void* out, int M, int N, int gate, hipStream_t st);
+int tq_rope_kv_write(const float* qkv, const void* bias, int bias_type, const int* positions,
+        const int* seq_of_token, const int* block_table, int bt_stride, const float* inv_freq, int pairing,
+        int rot, void* q_out, void* k_pool, void* v_pool, int page_size, int64_t page_stride, int T, int nh, int nkv,
+        int hd, int write_kv, const int* cu_seqlens, const int* slots, const int* start, int B, int max_new,
+        hipStream_t st);
 int tq_moe_combine(const float* y, const int* pair_slot, const float* weights, int topk, const float* shared,
         int S, int64_t shared_stride, const float* gate, float* out, int T, int H, hipStream_t st);
 // gemm_generic.hip: the plain multiply-add product (both libraries)

@@ -33,6 +33,10 @@ class DenseSwiGLU(Part):
                 "up": ParamSpec((self.inner_size, self.hidden_size)),
                 "down": ParamSpec((self.hidden_size, self.inner_size))}
 
+    def prepare(self, device, act):
+        # gate and up side by side: a long prompt's pair may then go out as one product over both
+        self.gate, self.up = ops.side_by_side(self.gate, self.up)
+
     def forward(self, normed, normed32, ctx):
         h = ops.gemm(normed, self.gate, ctx.act, w2=self.up, out_act=True, activation=self.activation)
         return ops.gemm(h, self.down, ctx.act, partial_sums=True)
@@ -67,6 +71,10 @@ class SparseMoE(Part):
             if self.shared_gated:
                 specs["shared_scale"] = ParamSpec((1, H))
         return specs
+
+    def prepare(self, device, act):
+        if self.shared_size > 0:     # as in the dense part; the experts' products never leave this library's kernels
+            self.shared_gate, self.shared_up = ops.side_by_side(self.shared_gate, self.shared_up)
 
     def forward(self, normed, normed32, ctx):
         T = normed.shape[0]
