@@ -283,14 +283,17 @@ TQ_API int tq_head_rmsnorm(float* qkv, const void* wq, const void* wk, int wtype
 // A workgroup of four waves takes `spb` heads of one token (grid (T, ceil(heads / spb))); a wave takes every
 // fourth of them and turns pair i of all its heads with one sine and cosine.  write_kv: 0 queries only, 1 keys
 // and values, 2 keys only (the values of whole runs of tokens go through v_write_tile_kernel below).
-// element i of a bias that the product before did not add (null: none); float32 or bfloat16 as bias_type says
-__device__ __forceinline__ float bias_elem(const void* bias, int bias_type, size_t i) {
-  if (!bias) return 0.f;
-  return bias_type == TQ_F32 ? ((const float*)bias)[i] : to_f32(((const bf16_t*)bias)[i]);
+// element i of a bias that the product before did not add; BIAS: 0 none, 1 float32, 2 bfloat16 (a template
+// argument, so that the loads of the bias go out beside those of the row and not behind a branch)
+template <int BIAS>
+__device__ __forceinline__ float bias_elem(const void* bias, size_t i) {
+  if (BIAS == 0) return 0.f;
+  return BIAS == 1 ? ((const float*)bias)[i] : to_f32(((const bf16_t*)bias)[i]);
 }
 
+template <int BIAS>
 __global__ __launch_bounds__(256) void rope_kv_write_kernel(const float* __restrict__ qkv, const void* __restrict__ bias,
-                                     int bias_type, const int* __restrict__ positions,
+                                     const int* __restrict__ positions,
                                      const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
                                      int bt_stride, const float* __restrict__ inv_freq, int pairing, int rot,
                                      act_t* __restrict__ q_out, act_t* __restrict__ k_pool,
@@ -323,8 +326,8 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(const float* __restr
     for (int s = s0; s < rot_end; s += 4) {
       const float* src = src_t + (size_t)s * hd;
       act_t* dst = s < nh ? q_t + (size_t)s * hd : k_t + (size_t)(s - nh) * kv_head_stride;
-      const float a = src[ia] + bias_elem(bias, bias_type, (size_t)s * hd + ia);
-      const float b = src[ib] + bias_elem(bias, bias_type, (size_t)s * hd + ib);
+      const float a = src[ia] + bias_elem<BIAS>(bias, (size_t)s * hd + ia);
+      const float b = src[ib] + bias_elem<BIAS>(bias, (size_t)s * hd + ib);
       dst[ia] = from_f32<act_t>(a * cs - b * sn);
       dst[ib] = from_f32<act_t>(a * sn + b * cs);
     }
@@ -333,7 +336,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(const float* __restr
     const float* src = src_t + (size_t)s * hd;
     act_t* dst = s < nh ? q_t + (size_t)s * hd : k_t + (size_t)(s - nh) * kv_head_stride;
     for (int i = rot + lane; i < hd; i += TQ_WAVE)
-      dst[i] = from_f32<act_t>(src[i] + bias_elem(bias, bias_type, (size_t)s * hd + i));
+      dst[i] = from_f32<act_t>(src[i] + bias_elem<BIAS>(bias, (size_t)s * hd + i));
   }
   if (write_kv != 1) return;
   for (int s = s0; s < s1; s += 4) {           // values lie transposed, [hd][row]
@@ -341,7 +344,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(const float* __restr
     const float* src = src_t + (size_t)s * hd;
     act_t* col = v_t + (size_t)(s - nh - nkv) * kv_head_stride;
     for (int i = lane; i < hd; i += TQ_WAVE)
-      col[(size_t)i * page_size] = from_f32<act_t>(src[i] + bias_elem(bias, bias_type, (size_t)s * hd + i));
+      col[(size_t)i * page_size] = from_f32<act_t>(src[i] + bias_elem<BIAS>(bias, (size_t)s * hd + i));
   }
 }
 
@@ -350,9 +353,9 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(const float* __restr
 // [position][hd] into [hd][position] in LDS and writes every dimension's positions 16 bytes at a time, where the
 // token-by-token write above would touch a cache line per dimension for two bytes.
 #define VT_POS 64
-template <int VEC>      // positions per 16-byte store
+template <int VEC, int BIAS>      // positions per 16-byte store; the bias as in rope_kv_write_kernel
 __global__ __launch_bounds__(256) void v_write_tile_kernel(const float* __restrict__ qkv,
-                                                           const void* __restrict__ bias, int bias_type,
+                                                           const void* __restrict__ bias,
                                                            const int* __restrict__ cu_seqlens,
                                                            const int* __restrict__ slots,
                                                            const int* __restrict__ start,
@@ -379,15 +382,15 @@ __global__ __launch_bounds__(256) void v_write_tile_kernel(const float* __restri
       const int r = idx / q4, d = (idx % q4) * 4;
       const f32x4 v = load4f(src0 + r * row_stride + d);
       act_t* to = ts + d * TS + (lo + r - P0);
-      to[0] = from_f32<act_t>(v.x + bias_elem(bias, bias_type, bias0 + d));
-      to[TS] = from_f32<act_t>(v.y + bias_elem(bias, bias_type, bias0 + d + 1));
-      to[2 * TS] = from_f32<act_t>(v.z + bias_elem(bias, bias_type, bias0 + d + 2));
-      to[3 * TS] = from_f32<act_t>(v.w + bias_elem(bias, bias_type, bias0 + d + 3));
+      to[0] = from_f32<act_t>(v.x + bias_elem<BIAS>(bias, bias0 + d));
+      to[TS] = from_f32<act_t>(v.y + bias_elem<BIAS>(bias, bias0 + d + 1));
+      to[2 * TS] = from_f32<act_t>(v.z + bias_elem<BIAS>(bias, bias0 + d + 2));
+      to[3 * TS] = from_f32<act_t>(v.w + bias_elem<BIAS>(bias, bias0 + d + 3));
     }
   } else {
     for (int r = wave; r < hi - lo; r += 4)
       for (int d = lane; d < hd; d += TQ_WAVE)
-        ts[d * TS + (lo + r - P0)] = from_f32<act_t>(src0[r * row_stride + d] + bias_elem(bias, bias_type, bias0 + d));
+        ts[d * TS + (lo + r - P0)] = from_f32<act_t>(src0[r * row_stride + d] + bias_elem<BIAS>(bias, bias0 + d));
   }
   __syncthreads();
   const int page = block_table[(size_t)slots[b] * bt_stride + P0 / page_size];
@@ -427,16 +430,30 @@ TQ_API int tq_rope_kv_write(const float* qkv, const void* bias, int bias_type, c
   int spb = 4;
   while (spb < heads && (int64_t)T * ((heads + spb - 1) / spb) > 4096) spb *= 2;
   if ((heads + spb - 1) / spb > 65535) return TQ_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL(rope_kv_write_kernel, dim3(T, (heads + spb - 1) / spb), dim3(256), 0, st, qkv, bias,
-                     bias_type, positions, seq_of_token, block_table, bt_stride, inv_freq, pairing, rot, (act_t*)q_out, (act_t*)k_pool,
-                     (act_t*)v_pool, page_size, page_stride, nh, nkv, hd, write_kv, spb);
+  const int bias_kind = !bias ? 0 : bias_type == TQ_F32 ? 1 : 2;
+#define TQ_ROPE_LAUNCH(BIAS)                                                                                          \
+  hipLaunchKernelGGL(rope_kv_write_kernel<BIAS>, dim3(T, (heads + spb - 1) / spb), dim3(256), 0, st, qkv, bias,       \
+                     positions, seq_of_token, block_table, bt_stride, inv_freq, pairing, rot, (act_t*)q_out,          \
+                     (act_t*)k_pool, (act_t*)v_pool, page_size, page_stride, nh, nkv, hd, write_kv, spb)
+  if (bias_kind == 0) TQ_ROPE_LAUNCH(0);
+  else if (bias_kind == 1) TQ_ROPE_LAUNCH(1);
+  else TQ_ROPE_LAUNCH(2);
+#undef TQ_ROPE_LAUNCH
   TQ_LAUNCH_CHECK();
   if (tiles) {
-    if (vt_shmem > 48 * 1024)
-      (void)hipFuncSetAttribute((const void*)v_write_tile_kernel<VEC>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)vt_shmem);
-    hipLaunchKernelGGL(v_write_tile_kernel<VEC>, dim3((max_new + VT_POS - 1) / VT_POS + 1, nkv, B), dim3(256), vt_shmem,
-                       st, qkv, bias, bias_type, cu_seqlens, slots, start, block_table, bt_stride, (act_t*)v_pool, page_size,
-                       page_stride, nh, nkv, hd);
+#define TQ_VT_LAUNCH(BIAS)                                                                                            \
+  do {                                                                                                                \
+    if (vt_shmem > 48 * 1024)                                                                                         \
+      (void)hipFuncSetAttribute((const void*)v_write_tile_kernel<VEC, BIAS>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                (int)vt_shmem);                                                                       \
+    hipLaunchKernelGGL((v_write_tile_kernel<VEC, BIAS>), dim3((max_new + VT_POS - 1) / VT_POS + 1, nkv, B), dim3(256), \
+                       vt_shmem, st, qkv, bias, cu_seqlens, slots, start, block_table, bt_stride, (act_t*)v_pool,     \
+                       page_size, page_stride, nh, nkv, hd);                                                          \
+  } while (0)
+    if (bias_kind == 0) TQ_VT_LAUNCH(0);
+    else if (bias_kind == 1) TQ_VT_LAUNCH(1);
+    else TQ_VT_LAUNCH(2);
+#undef TQ_VT_LAUNCH
     TQ_LAUNCH_CHECK();
   }
   return 0;
