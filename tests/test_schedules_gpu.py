@@ -217,7 +217,8 @@ def test_configurations_drawn_at_random(seed, tmp_path):
 def test_a_long_prompt_takes_the_taller_expert_tiles(sharp, monkeypatch):
     """From 256 rows per expert on, the bfloat16 products over experts take tiles of 128 rows: a prompt of 1,400 tokens
     with one expert of five per token goes that way through the engine (and one of 700 does not), and every
-    position agrees with the plain model."""
+    position agrees with the plain model.  From 1,024 rows per expert on the row order's unit is 256 (here the
+    bound is lowered to 256 rows, since the configuration's positions end at 2,048)."""
     from turboquant_cpp_amd.csrc import ops
     from turboquant_cpp_amd.engine.step import Engine
     d, plain, model = sharp("C", "bfloat16")
@@ -230,7 +231,8 @@ def test_a_long_prompt_takes_the_taller_expert_tiles(sharp, monkeypatch):
 
     monkeypatch.setattr(ops, "route", spy)
     eng = Engine(model, max_tokens=64 * 40, page_size=64)
-    for n, unit in ((1400, 128), (700, 64)):
+    for n, unit in ((1400, 128), (700, 64), (1400, 256)):
+        monkeypatch.setattr(ops, "EXPERT_256_FROM", 256 if unit == 256 else 1024)
         (prompt,) = prompts_for("C", [n], seed=29)
         del units[:]
         slots = eng.open(1)

@@ -27,6 +27,7 @@ struct MfmaGemmArgs {
   int k_per;                // k is split into runs of k_per, run z going to out + z * split_stride (float)
   int64_t split_stride;
   int gate;                 // activation of the gated pair
+  int group_ratio;          // tile kernel: row tiles per entry of tile_group and unit of n_tiles (0 or 1: one)
 };
 
 // For bytes that are read once (a matrix streamed past a few rows): a load that tells the caches so.  Measured on

@@ -343,7 +343,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g)
   // 12 % faster, the more the more row tiles an expert has); only the row tiles in use are dealt.
   int tile_m, tile_n;
   {
-    const int gx = g.tile_group && g.n_tiles ? min(g.n_tiles[0], (int)gridDim.x) : (int)gridDim.x;
+    // an entry of tile_group (and a unit of n_tiles) stands for `ratio` row tiles of this kernel where the row
+    // order was padded to a multiple of the tile's height
+    const int ratio = g.group_ratio > 1 ? g.group_ratio : 1;
+    const int gx = g.tile_group && g.n_tiles ? min(g.n_tiles[0] * ratio, (int)gridDim.x) : (int)gridDim.x;
     const int gy = gridDim.y, total = gx * gy;
     const int id = blockIdx.y * gridDim.x + blockIdx.x;
     const int die = id % 8, q = total / 8, rem = total % 8;
@@ -352,10 +355,12 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g)
     if (g.tile_group) {
       // the expert whose row tiles [lo, hi) hold row tile logical / gy; within it column by column, the expert's
       // row tiles of a column one after the other, so that they read that column's rows of w at the same time
-      const int t = logical / gy, e = g.tile_group[t];
-      int lo = t, hi = t + 1;
+      const int u = logical / gy / ratio, e = g.tile_group[u], gu = gx / ratio;
+      int lo = u, hi = u + 1;
       while (lo > 0 && g.tile_group[lo - 1] == e) --lo;
-      while (hi < gx && g.tile_group[hi] == e) ++hi;
+      while (hi < gu && g.tile_group[hi] == e) ++hi;
+      lo *= ratio;
+      hi *= ratio;
       const int local = logical - lo * gy, n_e = hi - lo;
       tile_n = local / n_e;
       tile_m = lo + local % n_e;
@@ -366,10 +371,12 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g)
       tile_n = in_band / bh;
     }
   }
-  const int group = g.tile_group ? g.tile_group[tile_m] : 0;
+  const int group = g.tile_group ? g.tile_group[tile_m / (g.group_ratio > 1 ? g.group_ratio : 1)] : 0;
   const bf16_t* w = g.w + (size_t)group * g.group_stride;
   const bf16_t* w2 = DUAL ? g.w2 + (size_t)group * g.group_stride : nullptr;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
+  // an expert's rows stand at the head of its units: a tile that begins with a row of padding holds nothing else
+  if (g.tile_group && g.a_rows && g.a_rows[min(m0, g.M - 1)] < 0) return;
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int wm = wave / WN, wn = wave % WN;
   // this workgroup's run of k: k_lo .. k_lo + Kl (all of k unless the product is split), and where its sums go
@@ -626,7 +633,7 @@ TQ_API int tq_gemm_mfma_splits(int M, int N, int K) {
 }
 
 // a: bfloat16 [.., K] with row stride lda (a multiple of 8, as K must be); w, w2: bfloat16.
-// tile_rows: with tile_group set, the padding unit of the row order (16, 64 or 128); else a hint that is ignored.
+// tile_rows: with tile_group set, the padding unit of the row order (16, 64, 128 or 256); else a hint that is ignored.
 // splits > 1 (as tq_gemm_mfma_splits says, for a plain product into float): run z of k goes to out + z * M * ldc,
 // the bias to run 0; the sum over the runs is the caller's.
 TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gather, const void* w, const void* w2,
@@ -641,7 +648,7 @@ TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gat
   if (splits > 1 && (dual || out_act || tile_group || a_rows || splits != tq_gemm_mfma_splits(M, N, K))) return TQ_ERR_BAD_ARG;
   const int k_per = ((K + TBK - 1) / TBK + splits - 1) / splits * TBK;
   MfmaGemmArgs g{(const bf16_t*)a, lda, a_rows, a_gather, (const bf16_t*)w, (const bf16_t*)w2, group_stride,
-                 tile_group, n_tiles, bias, bias_type, out, ldc, M, N, K, splits > 1 ? k_per : K, (int64_t)M * ldc, gate};
+                 tile_group, n_tiles, bias, bias_type, out, ldc, M, N, K, splits > 1 ? k_per : K, (int64_t)M * ldc, gate, 1};
   int rc = 0;
   if (tile_group) {
     if (tile_rows == 16) {
@@ -653,6 +660,18 @@ TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gat
     } else if (tile_rows == 128) {     // experts with hundreds of rows each: the taller tile's rate for little padding
       if ((N + TBN - 1) / TBN > 65535 || M % 128) return TQ_ERR_UNSUPPORTED;
       rc = launch_tile<128, 4, 2>(g, dual, out_act, 1, st);
+    } else if (tile_rows == 256) {
+      // A thousand rows and more each.  The gated pair takes tiles as tall as the unit, a wave's 64 x 64 outputs per
+      // pass over its operands (13,199 tokens x 8 of 64 experts of 2,560 x 3,584: 4.37 ms against 5.09 in tiles of 128
+      // rows); the plain product, whose k is the shorter one, stays with two tiles of 128 to a unit (2.85 ms; 3.00 as
+      // tiles of 256), of which one that holds padding only ends at once.
+      if ((N + TBN - 1) / TBN > 65535 || M % 256) return TQ_ERR_UNSUPPORTED;
+      if (dual) {
+        rc = launch_tile<256, 4, 2>(g, dual, out_act, 1, st);
+      } else {
+        g.group_ratio = 2;
+        rc = launch_tile<128, 4, 2>(g, dual, out_act, 1, st);
+      }
     } else {
       return TQ_ERR_BAD_ARG;
     }
@@ -715,7 +734,7 @@ TQ_API int tq_gemm_mfma_pair(const int64_t* d1, const int64_t* d2, int splits2, 
     if (((uintptr_t)p[0] | (uintptr_t)p[4] | (uintptr_t)p[5]) % 16 != 0) return TQ_ERR_BAD_ARG;
     g[i] = MfmaGemmArgs{(const bf16_t*)p[0], p[1], (const int*)p[2], (int)p[3], (const bf16_t*)p[4], (const bf16_t*)p[5],
                         p[6], (const int*)p[7], (const int*)p[8], (const void*)p[9], (int)p[10], (void*)p[11], p[12],
-                        M, N, K, K, 0, (int)p[18]};
+                        M, N, K, K, 0, (int)p[18], 1};
     if (g[i].gate < 0 || g[i].gate >= TQ_GATE_COUNT) return TQ_ERR_BAD_ARG;
     dual[i] = p[5] != 0;
     out_act[i] = p[13] != 0;
@@ -767,7 +786,7 @@ TQ_API int tq_qkv_rope_write(const void* a, int64_t lda, const void* w, const vo
   const int heads = k_pool ? nh + 2 * nkv : nh;
   const int N = (nh + 2 * nkv) * hd;
   MfmaGemmArgs g{(const bf16_t*)a, lda, nullptr, 1, (const bf16_t*)w, nullptr, 0, nullptr, nullptr, bias, bias_type,
-                 nullptr, 0, T, N, K, K, 0};
+                 nullptr, 0, T, N, K, K, 0, 0, 1};
   RopeWriteArgs p{positions, seq_of_token, block_table, bt_stride, inv_freq, (bf16_t*)q_out, (bf16_t*)k_pool,
                   (bf16_t*)v_pool, page_size, page_stride, nh, nkv, hd};
   int nw = split_k_waves(heads * hd / 2, K, false);

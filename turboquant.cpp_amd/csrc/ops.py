@@ -388,15 +388,19 @@ def _use_mfma(act, a: torch.Tensor, w: torch.Tensor, K: int) -> bool:
             and has_kernel(act, "tq_gemm_mfma"))
 
 
+EXPERT_256_FROM = 1024
+
+
 def expert_tile_rows(n_pairs: int, num_experts: int, act, a: torch.Tensor, w: torch.Tensor) -> int:
     """Rows per tile (the padding unit of the row order) that suit a product over experts: 16 while the pairs are so
     few that most experts have at most a tile of them (the streaming kernel), 128 from 256 rows per expert on average
     where the bfloat16 matrix-core product runs (its taller tile is 8 to 17 % faster there and slower below; at 137
-    rows per expert it lost 35 %), else 64."""
+    rows per expert it lost 35 %), 256 from 1,024 rows per expert (the gated pair in tiles of 256 rows is 8 to 14 %
+    faster there, the second product keeps tiles of 128: both together 4 to 8 %), else 64."""
     if n_pairs <= 16 * num_experts:
         return 16
     if n_pairs >= 256 * num_experts and _use_mfma(act, a, w, a.shape[1]):
-        return 128
+        return 256 if n_pairs >= EXPERT_256_FROM * num_experts else 128
     return 64
 
 
@@ -410,10 +414,10 @@ def _gemm_problem(k: str, a, w, act, bias, w2, out_act, a_rows, tile_group, n_ti
     grouped = tile_group is not None
     if grouped:
         _need(w.dim() == 3 and w.shape[2] == K, k, lambda: f"grouped w must be [G, N, {K}], is {tuple(w.shape)}")
-        _need(a_rows is not None and n_tiles is not None and tile_rows in (16, 64, 128), k,
-              "grouped product needs a_rows, n_tiles and tile_rows of 16, 64 or 128")
-        _need(tile_rows != 128 or _use_mfma(act, a, w, a.shape[1]), k,
-              "tiles of 128 rows are for the bfloat16 matrix-core product")
+        _need(a_rows is not None and n_tiles is not None and tile_rows in (16, 64, 128, 256), k,
+              "grouped product needs a_rows, n_tiles and tile_rows of 16, 64, 128 or 256")
+        _need(tile_rows < 128 or _use_mfma(act, a, w, a.shape[1]), k,
+              "tiles of 128 and 256 rows are for the bfloat16 matrix-core product")
         _check(a_rows, k, "a_rows", torch.int32)
         _check(tile_group, k, "tile_group", torch.int32)
         _check(n_tiles, k, "n_tiles", torch.int32)
@@ -730,7 +734,7 @@ def route(x32: torch.Tensor, router: torch.Tensor, shared_scale: torch.Tensor | 
     tile_expert, n_tiles), with the same results; a handful of tokens takes one kernel less."""
     k = "route"
     T, H, E, ids, weights, gate, logits = _router_outputs(k, x32, router, shared_scale, top_k)
-    _need(unit in (16, 64, 128), k, "unit must be 16, 64 or 128")
+    _need(unit in (16, 64, 128, 256), k, "unit must be 16, 64, 128 or 256")
     cap, sorted_token, pair_slot, tile_expert, n_tiles = _align_outputs(T, top_k, E, unit, x32.device)
     _run(k, library(act).tq_route(_ptr(x32), _ptr(router), _ptr(shared_scale), _WTYPE[router.dtype], E, top_k,
                                   int(bool(renormalize)), _ptr(ids), _ptr(weights), _ptr(gate), _ptr(logits), unit, cap,
