@@ -242,6 +242,34 @@ def test_a_long_prompt_takes_the_taller_expert_tiles(sharp, monkeypatch):
         check_sequence(got, plain, prompt, "bfloat16", f"C bfloat16 {n} tokens at once")
 
 
+# ------------------------------------------------------------------------------------------------ whose product it is
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_a_long_prompt_whole_cut_and_with_every_product_in_own_kernels(name, sharp, monkeypatch):
+    """A bfloat16 prompt step of 512 tokens and more hands its plain products (q, k, v without their bias; o; the
+    dense and the shared gated pairs and their down products) to the vendor's matrix library.  A prompt of 700
+    tokens taken whole that way, whole with every product in this library's kernels, and cut into steps of 250 that
+    never reach the library: all three against the plain model at every position."""
+    from turboquant_cpp_amd.csrc import ops
+    from turboquant_cpp_amd.engine.step import Engine
+    d, plain, model = sharp(name, "bfloat16")
+    (prompt,) = prompts_for(name, [700], seed=33)
+    calls = []
+    real = torch.mm
+    monkeypatch.setattr(torch, "mm", lambda *x, **kw: (calls.append(1), real(*x, **kw))[1])
+    eng = Engine(model, max_tokens=64 * 24, page_size=64)
+    for vendor, cuts, label in ((True, [700], "whole"), (False, [700], "whole, own products"), (True, [250, 250, 200], "cut")):
+        monkeypatch.setattr(ops, "_VENDOR", vendor)
+        del calls[:]
+        slots = eng.open(1)
+        rows, at = [], 0
+        for n in cuts:
+            rows.append(eng.step(slots, [prompt[at:at + n]], [list(range(n))]).clone())
+            at += n
+        eng.close(slots)
+        assert bool(calls) == (vendor and cuts == [700]), (label, len(calls))
+        check_sequence(torch.cat(rows), plain, prompt, "bfloat16", f"{name} bfloat16 700 tokens {label}")
+
+
 # ------------------------------------------------------------------------------------------------ entry points
 @pytest.mark.parametrize("act", ACTS)
 def test_the_command_line_generates(act, sharp):
