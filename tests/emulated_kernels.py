@@ -229,7 +229,7 @@ def head_rmsnorm(qkv, q_weight, k_weight, eps, num_heads, num_kv_heads, head_dim
 
 
 def expert_tile_rows(n_pairs, num_experts, act, a, w):
-    return 16 if n_pairs <= 16 * num_experts else 64
+    return 16 if n_pairs <= 12 * num_experts else 64
 
 
 def qkv_rope_write(a, qkv_weight, qkv_bias, positions, seq_of_token, block_table, inv_freq, pairing, rotary_dim, k_pages,

@@ -244,12 +244,12 @@ def test_gemm_rows_do_not_depend_on_the_batch(ops, act):
 
 
 def test_the_height_of_expert_tiles(ops):
-    """16 while the pairs are few, 128 from 256 rows per expert and 256 from 1,024 where the bfloat16 matrix-core product
+    """16 up to 12 pairs per expert, 128 from 256 rows per expert and 256 from 1,024 where the bfloat16 matrix-core product
     runs, else 64."""
     a16, w16 = torch.zeros((1, 64), dtype=torch.bfloat16), torch.zeros((1, 8, 64), dtype=torch.bfloat16)
     a32, w32 = a16.float(), w16.float()
-    assert ops.expert_tile_rows(60 * 16, 60, "bfloat16", a16, w16) == 16
-    assert ops.expert_tile_rows(60 * 16 + 1, 60, "bfloat16", a16, w16) == 64
+    assert ops.expert_tile_rows(60 * 12, 60, "bfloat16", a16, w16) == 16
+    assert ops.expert_tile_rows(60 * 12 + 1, 60, "bfloat16", a16, w16) == 64
     assert ops.expert_tile_rows(60 * 256 - 1, 60, "bfloat16", a16, w16) == 64
     assert ops.expert_tile_rows(60 * 256, 60, "bfloat16", a16, w16) == 128
     assert ops.expert_tile_rows(60 * 1024 - 1, 60, "bfloat16", a16, w16) == 128

@@ -392,12 +392,15 @@ EXPERT_256_FROM = 1024
 
 
 def expert_tile_rows(n_pairs: int, num_experts: int, act, a: torch.Tensor, w: torch.Tensor) -> int:
-    """Rows per tile (the padding unit of the row order) that suit a product over experts: 16 while the pairs are so
-    few that most experts have at most a tile of them (the streaming kernel), 128 from 256 rows per expert on average
-    where the bfloat16 matrix-core product runs (its taller tile is 8 to 17 % faster there and slower below; at 137
-    rows per expert it lost 35 %), 256 from 1,024 rows per expert (the gated pair in tiles of 256 rows is 8 to 14 %
-    faster there, the second product keeps tiles of 128: both together 4 to 8 %), else 64."""
-    if n_pairs <= 16 * num_experts:
+    """Rows per tile (the padding unit of the row order) that suit a product over experts: 16 (the streaming kernel,
+    which passes an expert's matrices once per 16 of its rows) up to 12 pairs per expert on average, where few experts
+    have more than 16 rows (60 experts of 1,408 x 2,048, 4 per token: 207 us for both products against 231 in tiles of
+    64 rows at 12 rows per expert, 277 against 236 at 16; 64 experts of 2,560 x 3,584, 8 per token: 700 against 650 at
+    12, 898 against 638 at 16); 128 from 256 rows per expert where the bfloat16 matrix-core product runs (its taller
+    tile is 8 to 17 % faster there and slower below; at 137 rows per expert it lost 35 %), 256 from 1,024 rows per
+    expert (the gated pair in tiles of 256 rows is 8 to 14 % faster there, the second product keeps tiles of 128: both
+    together 4 to 8 %), else 64."""
+    if n_pairs <= 12 * num_experts:
         return 16
     if n_pairs >= 256 * num_experts and _use_mfma(act, a, w, a.shape[1]):
         return 256 if n_pairs >= EXPERT_256_FROM * num_experts else 128
