@@ -244,12 +244,16 @@ def test_gemm_rows_do_not_depend_on_the_batch(ops, act):
 
 
 def test_the_height_of_expert_tiles(ops):
-    """16 up to 12 pairs per expert, 128 from 256 rows per expert and 256 from 1,024 where the bfloat16 matrix-core product
+    """16 up to 8 pairs per expert and 32 up to 22 where the bfloat16 matrix-core product runs (else 16 up to 12), 128 from 256 rows per expert and 256 from 1,024 where the bfloat16 matrix-core product
     runs, else 64."""
     a16, w16 = torch.zeros((1, 64), dtype=torch.bfloat16), torch.zeros((1, 8, 64), dtype=torch.bfloat16)
     a32, w32 = a16.float(), w16.float()
-    assert ops.expert_tile_rows(60 * 12, 60, "bfloat16", a16, w16) == 16
-    assert ops.expert_tile_rows(60 * 12 + 1, 60, "bfloat16", a16, w16) == 64
+    assert ops.expert_tile_rows(60 * 8, 60, "bfloat16", a16, w16) == 16
+    assert ops.expert_tile_rows(60 * 8 + 1, 60, "bfloat16", a16, w16) == 32
+    assert ops.expert_tile_rows(60 * 22, 60, "bfloat16", a16, w16) == 32
+    assert ops.expert_tile_rows(60 * 22 + 1, 60, "bfloat16", a16, w16) == 64
+    assert ops.expert_tile_rows(60 * 12, 60, "float32", a32, w32) == 16
+    assert ops.expert_tile_rows(60 * 12 + 1, 60, "float32", a32, w32) == 64
     assert ops.expert_tile_rows(60 * 256 - 1, 60, "bfloat16", a16, w16) == 64
     assert ops.expert_tile_rows(60 * 256, 60, "bfloat16", a16, w16) == 128
     assert ops.expert_tile_rows(60 * 1024 - 1, 60, "bfloat16", a16, w16) == 128
@@ -260,15 +264,16 @@ def test_the_height_of_expert_tiles(ops):
 
 
 @pytest.mark.parametrize("act", ACTS)
-@pytest.mark.parametrize("unit", [16, 64, 128, 256])
+@pytest.mark.parametrize("unit", [16, 32, 64, 128, 256])
 @pytest.mark.parametrize("T,E,k,H,I", [(1, 5, 2, 72, 40), (9, 7, 3, 136, 88), (150, 6, 2, 64, 200), (700, 3, 2, 64, 136)])
 def test_expert_products(ops, act, unit, T, E, k, H, I):
     """Pairs ordered by expert, the gated product over gathered rows, the second product over rows in place.
-    Units of 128 and 256 rows are the bfloat16 matrix-core product's alone (with 256, the gated pair runs in tiles of
+    Units of 32, 128 and 256 rows are the bfloat16 matrix-core product's alone (32: the streaming kernel with two row
+    tiles to a wave; with 256, the gated pair runs in tiles of
     256 rows and the second product in two tiles of 128 to a unit; 700 tokens give each expert a whole unit and
     a part of one)."""
-    if unit >= 128 and act != "bfloat16":
-        pytest.skip("tiles of 128 and 256 rows are for the bfloat16 matrix-core product")
+    if unit not in (16, 64) and act != "bfloat16":
+        pytest.skip("tiles of 32, 128 and 256 rows are for the bfloat16 matrix-core product")
     g = torch.Generator().manual_seed(40)
     ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32)
     x = rnd((T, H), adt(act), 41)

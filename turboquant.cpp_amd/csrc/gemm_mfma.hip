@@ -633,7 +633,8 @@ TQ_API int tq_gemm_mfma_splits(int M, int N, int K) {
 }
 
 // a: bfloat16 [.., K] with row stride lda (a multiple of 8, as K must be); w, w2: bfloat16.
-// tile_rows: with tile_group set, the padding unit of the row order (16, 64, 128 or 256); else a hint that is ignored.
+// tile_rows: with tile_group set, the padding unit of the row order (16, 32, 64, 128 or 256); else a hint that is
+// ignored.
 // splits > 1 (as tq_gemm_mfma_splits says, for a plain product into float): run z of k goes to out + z * M * ldc,
 // the bias to run 0; the sum over the runs is the caller's.
 TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gather, const void* w, const void* w2,
@@ -654,6 +655,9 @@ TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gat
     if (tile_rows == 16) {
       if (M % 16) return TQ_ERR_BAD_ARG;
       rc = launch_stream<1>(g, dual, out_act, M / 16, st);
+    } else if (tile_rows == 32) {      // the streaming kernel with two row tiles and two column tiles to a wave
+      if (M % 32) return TQ_ERR_BAD_ARG;
+      rc = launch_stream<2>(g, dual, out_act, M / 32, st);
     } else if (tile_rows == 64) {
       if ((N + TBN - 1) / TBN > 65535) return TQ_ERR_UNSUPPORTED;
       rc = launch_tile<64, 2, 4>(g, dual, out_act, 1, st);

@@ -392,17 +392,21 @@ EXPERT_256_FROM = 1024
 
 
 def expert_tile_rows(n_pairs: int, num_experts: int, act, a: torch.Tensor, w: torch.Tensor) -> int:
-    """Rows per tile (the padding unit of the row order) that suit a product over experts: 16 (the streaming kernel,
-    which passes an expert's matrices once per 16 of its rows) up to 12 pairs per expert on average, where few experts
-    have more than 16 rows (60 experts of 1,408 x 2,048, 4 per token: 207 us for both products against 231 in tiles of
-    64 rows at 12 rows per expert, 277 against 236 at 16; 64 experts of 2,560 x 3,584, 8 per token: 700 against 650 at
-    12, 898 against 638 at 16); 128 from 256 rows per expert where the bfloat16 matrix-core product runs (its taller
-    tile is 8 to 17 % faster there and slower below; at 137 rows per expert it lost 35 %), 256 from 1,024 rows per
-    expert (the gated pair in tiles of 256 rows is 8 to 14 % faster there, the second product keeps tiles of 128: both
-    together 4 to 8 %), else 64."""
-    if n_pairs <= 12 * num_experts:
+    """Rows per tile (the padding unit of the row order) that suit a product over experts, by the pairs per expert on
+    average.  Up to 8: 16, the streaming kernel, which passes an expert's matrices once per 16 of its rows.  Up to 22,
+    where the bfloat16 matrix-core product runs: 32, the same kernel with two row tiles and two column tiles to a wave
+    (60 experts of 1,408 x 2,048, 4 per token, both products: 202 us at 16 rows per expert against 270 in tiles of 16
+    and 233 in tiles of 64 rows; 64 experts of 2,560 x 3,584, 8 per token: 617 against 888 and 640; at 8 rows the three
+    are within 5 % of each other, at 26 the tiles of 64 rows win).  Without that kernel 16 up to 12.  From 256: 128
+    (the taller tile is 8 to 17 % faster there and slower below; at 137 rows per expert it lost 35 %); from 1,024:
+    256 (the gated pair in tiles of 256 rows is 8 to 14 % faster there, the second product keeps tiles of 128: both
+    together 4 to 8 %); else 64."""
+    mfma = _use_mfma(act, a, w, a.shape[1])
+    if n_pairs <= (8 if mfma else 12) * num_experts:
         return 16
-    if n_pairs >= 256 * num_experts and _use_mfma(act, a, w, a.shape[1]):
+    if mfma and n_pairs <= 22 * num_experts:
+        return 32
+    if n_pairs >= 256 * num_experts and mfma:
         return 256 if n_pairs >= EXPERT_256_FROM * num_experts else 128
     return 64
 
@@ -417,10 +421,10 @@ def _gemm_problem(k: str, a, w, act, bias, w2, out_act, a_rows, tile_group, n_ti
     grouped = tile_group is not None
     if grouped:
         _need(w.dim() == 3 and w.shape[2] == K, k, lambda: f"grouped w must be [G, N, {K}], is {tuple(w.shape)}")
-        _need(a_rows is not None and n_tiles is not None and tile_rows in (16, 64, 128, 256), k,
+        _need(a_rows is not None and n_tiles is not None and tile_rows in (16, 32, 64, 128, 256), k,
               "grouped product needs a_rows, n_tiles and tile_rows of 16, 64, 128 or 256")
-        _need(tile_rows < 128 or _use_mfma(act, a, w, a.shape[1]), k,
-              "tiles of 128 and 256 rows are for the bfloat16 matrix-core product")
+        _need(tile_rows in (16, 64) or _use_mfma(act, a, w, a.shape[1]), k,
+              "tiles of 32, 128 and 256 rows are for the bfloat16 matrix-core product")
         _check(a_rows, k, "a_rows", torch.int32)
         _check(tile_group, k, "tile_group", torch.int32)
         _check(n_tiles, k, "n_tiles", torch.int32)
@@ -737,7 +741,7 @@ def route(x32: torch.Tensor, router: torch.Tensor, shared_scale: torch.Tensor | 
     tile_expert, n_tiles), with the same results; a handful of tokens takes one kernel less."""
     k = "route"
     T, H, E, ids, weights, gate, logits = _router_outputs(k, x32, router, shared_scale, top_k)
-    _need(unit in (16, 64, 128, 256), k, "unit must be 16, 64, 128 or 256")
+    _need(unit in (16, 32, 64, 128, 256), k, "unit must be 16, 32, 64, 128 or 256")
     cap, sorted_token, pair_slot, tile_expert, n_tiles = _align_outputs(T, top_k, E, unit, x32.device)
     _run(k, library(act).tq_route(_ptr(x32), _ptr(router), _ptr(shared_scale), _WTYPE[router.dtype], E, top_k,
                                   int(bool(renormalize)), _ptr(ids), _ptr(weights), _ptr(gate), _ptr(logits), unit, cap,
