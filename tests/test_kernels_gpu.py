@@ -452,6 +452,29 @@ def test_router_random(ops, act, E, k, H, renorm):
 
 
 @pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("E,k,H,shared", [(60, 4, 2048, True), (64, 8, 3584, True), (5, 2, 72, False), (130, 8, 1000, True),
+                                          (17, 3, 4100, True), (8, 2, 70, True)])
+def test_router_results_do_not_depend_on_the_number_of_tokens(ops, act, E, k, H, shared):
+    """How many tokens a workgroup of the router takes and how many rows a wave takes at a time depend on the number of
+    tokens; the order in which a logit is summed does not: choices, weights and the shared expert's gate of a token
+    are the same bits in a step of 700 tokens, of 300, and of 7."""
+    T = 700
+    x = rnd((T, H), torch.float32, 67).to(DEV)
+    wr = rnd((E, H), adt(act), 68, 0.3).to(DEV)
+    sg = rnd((1, H), adt(act), 69, 0.1).to(DEV) if shared else None
+    ids, w, gate = ops.router_topk(x, wr, sg, k, False, act)
+    logits = x.cpu().double() @ wr.cpu().double().T
+    top = torch.topk(logits, k, dim=-1)
+    gap = (top.values[:, -1] - torch.topk(logits, min(k + 1, E), dim=-1).values[:, -1]).abs()
+    clear = gap > 1e-3 * logits.abs().max()
+    assert clear.sum() > T // 2 and torch.equal(ids.cpu().long()[clear], top.indices[clear])
+    for lo, hi in ((0, 300), (300, 307), (693, 700), (400, 655), (0, 256)):
+        i2, w2, g2 = ops.router_topk(x[lo:hi].contiguous(), wr, sg, k, False, act)
+        assert torch.equal(i2, ids[lo:hi]) and torch.equal(w2, w[lo:hi])
+        assert (g2 is None and gate is None) or torch.equal(g2, gate[lo:hi])
+
+
+@pytest.mark.parametrize("act", ACTS)
 @pytest.mark.parametrize("E,k,H,renorm,shared", [(5, 5, 72, True, True), (60, 4, 2048, False, True), (130, 8, 70, True, False)])
 def test_routing_in_one_call(ops, act, E, k, H, renorm, shared):
     """``route`` is router_topk followed by moe_align; up to 16 tokens take a kernel that chooses and orders at
