@@ -459,6 +459,24 @@ VENDOR_MIN_ROWS = 512
 _VENDOR = os.environ.get("TQ_PLAIN_PRODUCTS", "vendor") != "own"
 
 
+class own_products:
+    """``with own_products(True):`` keeps every product inside in this library's kernels: what a decode step runs
+    eagerly must be what its capture will replay, however many sequences it has."""
+
+    def __init__(self, on: bool = True):
+        self.on = on
+
+    def __enter__(self):
+        global _VENDOR
+        self.before = _VENDOR
+        if self.on:
+            _VENDOR = False
+
+    def __exit__(self, *exc):
+        global _VENDOR
+        _VENDOR = self.before
+
+
 def _vendor_product(act, a, w, M: int, K: int) -> bool:
     return (_VENDOR and M >= VENDOR_MIN_ROWS and (K < 16384 or M >= 8192) and dtype_name(act) == "bfloat16"
             and w.dtype == torch.bfloat16 and a.stride(1) == 1 and w.is_contiguous()

@@ -12,6 +12,7 @@ from __future__ import annotations
 import torch
 
 from ..cache.paged import CacheError
+from ..csrc import ops
 from .batch import pack_step
 from .context import StepContext
 from .graph import DecodeGraphs
@@ -151,4 +152,5 @@ class Engine:
         # a second stream for what does not depend on the main line (the parts decide what they put there)
         ctx = StepContext(batch=batch, cache=self.cache, act=self.model.act, device=self.device,
                           side_stream=self.side_stream)
-        return self.model.forward(ctx)
+        with ops.own_products(max(batch.n_new) == 1):      # a decode step runs the kernels that its replay runs
+            return self.model.forward(ctx)
