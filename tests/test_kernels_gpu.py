@@ -244,14 +244,14 @@ def test_gemm_rows_do_not_depend_on_the_batch(ops, act):
 
 
 def test_the_height_of_expert_tiles(ops):
-    """16 up to 8 pairs per expert and 32 up to 22 where the bfloat16 matrix-core product runs (else 16 up to 12), 128 from 256 rows per expert and 256 from 1,024 where the bfloat16 matrix-core product
+    """16 up to 5 pairs per expert and 32 up to 10 where the bfloat16 matrix-core product runs (else 16 up to 12), 128 from 256 rows per expert and 256 from 1,024 where the bfloat16 matrix-core product
     runs, else 64."""
     a16, w16 = torch.zeros((1, 64), dtype=torch.bfloat16), torch.zeros((1, 8, 64), dtype=torch.bfloat16)
     a32, w32 = a16.float(), w16.float()
-    assert ops.expert_tile_rows(60 * 8, 60, "bfloat16", a16, w16) == 16
-    assert ops.expert_tile_rows(60 * 8 + 1, 60, "bfloat16", a16, w16) == 32
-    assert ops.expert_tile_rows(60 * 22, 60, "bfloat16", a16, w16) == 32
-    assert ops.expert_tile_rows(60 * 22 + 1, 60, "bfloat16", a16, w16) == 64
+    assert ops.expert_tile_rows(60 * 5, 60, "bfloat16", a16, w16) == 16
+    assert ops.expert_tile_rows(60 * 5 + 1, 60, "bfloat16", a16, w16) == 32
+    assert ops.expert_tile_rows(60 * 10, 60, "bfloat16", a16, w16) == 32
+    assert ops.expert_tile_rows(60 * 10 + 1, 60, "bfloat16", a16, w16) == 64
     assert ops.expert_tile_rows(60 * 12, 60, "float32", a32, w32) == 16
     assert ops.expert_tile_rows(60 * 12 + 1, 60, "float32", a32, w32) == 64
     assert ops.expert_tile_rows(60 * 256 - 1, 60, "bfloat16", a16, w16) == 64

@@ -389,22 +389,27 @@ def _use_mfma(act, a: torch.Tensor, w: torch.Tensor, K: int) -> bool:
 
 
 EXPERT_256_FROM = 1024
+EXPERT_16_UPTO, EXPERT_32_UPTO = 5, 10
 
 
 def expert_tile_rows(n_pairs: int, num_experts: int, act, a: torch.Tensor, w: torch.Tensor) -> int:
     """Rows per tile (the padding unit of the row order) that suit a product over experts, by the pairs per expert on
-    average.  Up to 8: 16, the streaming kernel, which passes an expert's matrices once per 16 of its rows.  Up to 22,
-    where the bfloat16 matrix-core product runs: 32, the same kernel with two row tiles and two column tiles to a wave
-    (60 experts of 1,408 x 2,048, 4 per token, both products: 202 us at 16 rows per expert against 270 in tiles of 16
-    and 233 in tiles of 64 rows; 64 experts of 2,560 x 3,584, 8 per token: 617 against 888 and 640; at 8 rows the three
-    are within 5 % of each other, at 26 the tiles of 64 rows win).  Without that kernel 16 up to 12.  From 256: 128
-    (the taller tile is 8 to 17 % faster there and slower below; at 137 rows per expert it lost 35 %); from 1,024:
-    256 (the gated pair in tiles of 256 rows is 8 to 14 % faster there, the second product keeps tiles of 128: both
-    together 4 to 8 %); else 64."""
+    average.  Up to 5: 16, the streaming kernel, which passes an expert's matrices once per 16 of its rows.  Up to 10,
+    where the bfloat16 matrix-core product runs: 32, the same kernel with two row tiles and two column tiles to a wave.
+    Beyond: tiles of 64 rows.  Where the borders lie depends on how evenly the router deals: with tokens dealt evenly
+    (60 experts of 1,408 x 2,048, 4 per token, both products) units of 16 are best up to 8 rows per expert by 3 to 6 %,
+    units of 32 from 10 to 24 by 9 to 13 % (202 us at 16 rows per expert against 270 and 233), tiles of 64 rows beyond;
+    with a router of random weights, which gives some experts three times the rows of others, units of 32 are best up
+    to 6 rows per expert (64 experts, 8 per token: up to 12) and tiles of 64 rows win by 10 to 18 % from 12 on, since a
+    crowded expert's matrices pass the streaming kernel once per unit.  The borders here lose at most 6 % either way (a replayed decode step of 64 sequences, 4.3 rows per expert, is 2 %
+    faster with units of 16 than of 32).
+    Without the matrix-core product 16 up to 12.  From 256: 128 (the taller tile is 8 to 17 % faster there and slower
+    below; at 137 rows per expert it lost 35 %); from 1,024: 256 (the gated pair in tiles of 256 rows is 8 to 14 %
+    faster there, the second product keeps tiles of 128: both together 4 to 8 %)."""
     mfma = _use_mfma(act, a, w, a.shape[1])
-    if n_pairs <= (8 if mfma else 12) * num_experts:
+    if n_pairs <= (EXPERT_16_UPTO if mfma else 12) * num_experts:
         return 16
-    if mfma and n_pairs <= 22 * num_experts:
+    if mfma and n_pairs <= EXPERT_32_UPTO * num_experts:
         return 32
     if n_pairs >= 256 * num_experts and mfma:
         return 256 if n_pairs >= EXPERT_256_FROM * num_experts else 128
