@@ -824,6 +824,42 @@ def test_decoding_over_long_caches(ops, act, window):
                               torch.tensor([slots[i]], dtype=torch.int32).to(DEV), table.to(DEV), page, page_stride, nh, nkv,
                               hd, window, scale, act, runs=runs1).cpu()
         assert torch.equal(alone[0], out[i])
+    # and so does a step with so many waves that the kernel does not fetch tiles ahead (the batch four times over)
+    rep = 4
+    runs4 = {"cu_seqlens": torch.arange(rep * B + 1, dtype=torch.int32).to(DEV), "slots": torch.tensor(slots * rep, dtype=torch.int32).to(DEV),
+             "start": positions.repeat(rep).to(DEV), "max_new": 1, "max_end": max(lens), "decode": True}
+    out4 = ops.attention(torch.stack(qs * rep).reshape(rep * B, nh * hd).to(DEV), kp.to(DEV), vp.to(DEV), 0,
+                         positions.repeat(rep).to(DEV), torch.tensor(slots * rep, dtype=torch.int32).to(DEV), table.to(DEV), page,
+                         page_stride, nh, nkv, hd, window, scale, act, runs=runs4).cpu()
+    assert torch.equal(out4, out.repeat(rep, 1))
+
+
+@pytest.mark.parametrize("hd,nh,nkv", [(128, 16, 16), (128, 28, 4), (64, 8, 8)])
+def test_decoding_with_tiles_fetched_ahead_gives_the_same_bits(ops, hd, nh, nkv):
+    """A decode step of few waves (up to one per SIMD) runs the form of the kernel that keeps the next tile of keys
+    and values in registers; a token's result is the same bits as in a step of many sequences, at positions below and
+    beyond 4,096 (runs of one and of three tiles) and with a window."""
+    act, page = "bfloat16", 64
+    lens = [100, 2500, 4097, 8200]
+    table, slots, page_stride, kp, vp = paged_setup(lens, page, nkv, hd, 1, act, 97)
+    kp.copy_(rnd((kp.numel(),), adt(act), 98, 0.5))
+    vp.copy_(rnd((vp.numel(),), adt(act), 99))
+    scale = 1.0 / math.sqrt(hd)
+    B, rep = len(lens), 40
+    q = rnd((B, nh * hd), adt(act), 100)
+    positions = torch.tensor([n - 1 for n in lens], dtype=torch.int32)
+    for window in (None, 3000):
+        def run(idx):
+            n = len(idx)
+            runs = {"cu_seqlens": torch.arange(n + 1, dtype=torch.int32).to(DEV),
+                    "slots": torch.tensor([slots[i] for i in idx], dtype=torch.int32).to(DEV),
+                    "start": positions[idx].to(DEV), "max_new": 1, "max_end": max(lens[i] for i in idx), "decode": True}
+            return ops.attention(q[idx].to(DEV), kp.to(DEV), vp.to(DEV), 0, positions[idx].to(DEV), runs["slots"], table.to(DEV), page,
+                                 page_stride, nh, nkv, hd, window, scale, act, runs=runs).cpu()
+        many = run(list(range(B)) * rep)          # 160 sequences: thousands of waves
+        assert many.abs().max() > 0.01
+        for i in range(B):
+            assert torch.equal(run([i])[0], many[i]) and torch.equal(many[i], many[i + B * (rep - 1)])
 
 
 # ------------------------------------------------------------------------------------------------ sampling

@@ -115,6 +115,66 @@ __device__ __forceinline__ int k_swz(int row, int ch) {
 }
 __device__ __forceinline__ int v_swz(int d, int ch) { return d * TILE + ((ch ^ (d & 7)) << 3); }
 
+// The part of a tile between its two products, for QG groups of 16 columns: s holds the tile's scores (rows of
+// block jt as tile_step says); afterwards m_run, l_run and o are brought to the new running maximum and pf holds the
+// probabilities 2^(s * scale2 - m) as the operand of the second product.
+template <int DT, int QG>
+__device__ __forceinline__ void softmax_tile(f32x4 (&s)[QG][4], f32x4 (&o)[QG][DT], float (&m_run)[QG], float (&l_run)[QG],
+                                             int pos0, const int (&p_q)[QG], const int (&lo_q)[QG], float scale2,
+                                             bool masked, bf16x8 (&pf)[2][QG]) {
+  const int c = (threadIdx.x % 64) / 16;
+  // mask, running maximum, probabilities
+#pragma unroll
+  for (int g = 0; g < QG; ++g) {
+    float m_tile = -INFINITY;
+    if (masked) {
+#pragma unroll
+      for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int key = pos0 + 32 * (jt / 2) + 8 * c + 4 * (jt % 2) + v;
+          const bool ok = key <= p_q[g] && key >= lo_q[g];
+          s[g][jt][v] = ok ? s[g][jt][v] : -INFINITY;
+          m_tile = fmaxf(m_tile, s[g][jt][v]);
+        }
+    } else {
+#pragma unroll
+      for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) m_tile = fmaxf(m_tile, s[g][jt][v]);
+    }
+    m_tile = group_max(m_tile) * scale2;
+    const float m_new = fmaxf(m_run[g], m_tile);
+    const bool any = m_new != -INFINITY;
+    const float alpha = any && m_run[g] != -INFINITY ? __builtin_amdgcn_exp2f(m_run[g] - m_new) : (any ? 0.f : 1.f);
+    const float m_use = any ? m_new : 0.f;       // 2^(-inf - 0) = 0 for masked keys, also when all are masked
+    float l_tile = 0.f;
+#pragma unroll
+    for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const float p = __builtin_amdgcn_exp2f(fmaf(s[g][jt][v], scale2, -m_use));
+        s[g][jt][v] = p;
+        l_tile += p;
+      }
+    l_run[g] = l_run[g] * alpha + group_sum(l_tile);
+    m_run[g] = m_new;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) o[g][dt][v] *= alpha;
+  }
+  // the probabilities as the second product's operand: what the lane holds already
+#pragma unroll
+  for (int pr = 0; pr < 2; ++pr)
+#pragma unroll
+    for (int g = 0; g < QG; ++g) {
+      const u32x4 pw = {pack2(s[g][2 * pr][0], s[g][2 * pr][1]), pack2(s[g][2 * pr][2], s[g][2 * pr][3]),
+                        pack2(s[g][2 * pr + 1][0], s[g][2 * pr + 1][1]), pack2(s[g][2 * pr + 1][2], s[g][2 * pr + 1][3])};
+      pf[pr][g] = __builtin_bit_cast(bf16x8, pw);
+    }
+}
+
 // One tile of 64 positions for QG groups of 16 columns that share the tile's keys and values.  kt: the tile's
 // keys, row i at kt + i * k_stride; vt: the tile's values transposed, dimension d at vt + d * v_stride (memory or
 // LDS).  DT: number of 16-wide blocks of hd held in registers (hd <= 16 * DT).  p_q: position of this lane's
@@ -171,57 +231,8 @@ __device__ __forceinline__ void tile_step(f32x4 (&o)[QG][DT], float (&m_run)[QG]
       }
     }
   }
-  // mask, running maximum, probabilities
-#pragma unroll
-  for (int g = 0; g < QG; ++g) {
-    float m_tile = -INFINITY;
-    if (masked) {
-#pragma unroll
-      for (int jt = 0; jt < 4; ++jt)
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-          const int key = pos0 + 32 * (jt / 2) + 8 * c + 4 * (jt % 2) + v;
-          const bool ok = key <= p_q[g] && key >= lo_q[g];
-          s[g][jt][v] = ok ? s[g][jt][v] : -INFINITY;
-          m_tile = fmaxf(m_tile, s[g][jt][v]);
-        }
-    } else {
-#pragma unroll
-      for (int jt = 0; jt < 4; ++jt)
-#pragma unroll
-        for (int v = 0; v < 4; ++v) m_tile = fmaxf(m_tile, s[g][jt][v]);
-    }
-    m_tile = group_max(m_tile) * scale2;
-    const float m_new = fmaxf(m_run[g], m_tile);
-    const bool any = m_new != -INFINITY;
-    const float alpha = any && m_run[g] != -INFINITY ? __builtin_amdgcn_exp2f(m_run[g] - m_new) : (any ? 0.f : 1.f);
-    const float m_use = any ? m_new : 0.f;       // 2^(-inf - 0) = 0 for masked keys, also when all are masked
-    float l_tile = 0.f;
-#pragma unroll
-    for (int jt = 0; jt < 4; ++jt)
-#pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        const float p = __builtin_amdgcn_exp2f(fmaf(s[g][jt][v], scale2, -m_use));
-        s[g][jt][v] = p;
-        l_tile += p;
-      }
-    l_run[g] = l_run[g] * alpha + group_sum(l_tile);
-    m_run[g] = m_new;
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-      for (int v = 0; v < 4; ++v) o[g][dt][v] *= alpha;
-  }
-  // values
   bf16x8 pf[2][QG];
-#pragma unroll
-  for (int pr = 0; pr < 2; ++pr)
-#pragma unroll
-    for (int g = 0; g < QG; ++g) {
-      const u32x4 pw = {pack2(s[g][2 * pr][0], s[g][2 * pr][1]), pack2(s[g][2 * pr][2], s[g][2 * pr][3]),
-                        pack2(s[g][2 * pr + 1][0], s[g][2 * pr + 1][1]), pack2(s[g][2 * pr + 1][2], s[g][2 * pr + 1][3])};
-      pf[pr][g] = __builtin_bit_cast(bf16x8, pw);
-    }
+  softmax_tile<DT, QG>(s, o, m_run, l_run, pos0, p_q, lo_q, scale2, masked, pf);
   if (ONCE) {
     // a row of values (64 positions of one dimension) is one line: both halves of the tile come with it
 #pragma unroll
@@ -265,6 +276,91 @@ __device__ __forceinline__ void attend(f32x4 (&o)[1][DT], float (&m_run)[1], flo
     const bool masked = pos0 + TILE - 1 > p || pos0 < lo_q;      // the same for all lanes
     tile_step<DT, 1, EXACT, false, EXACT>(o, m_run, l_run, qf, kt, hd, vt, page_size, hd, pos0, pq, lq, scale2, masked);
   }
+}
+
+// The same run of tiles for a step that has few waves (a handful of sequences): then a wave has a SIMD's registers
+// to itself, and keeps a whole tile of keys and values in them (2 DT registers of 16 bytes each, fetched by whole
+// lines as in tile_step) while it works on the tile before.  Every product and sum is the one of `attend`, in the same
+// order: only the loads go out earlier.
+template <int DT>
+struct TileRegs {
+  u32x4 k[4][DT / 2];       // block jt, step ks of hd (before the exchange between lanes)
+  u32x4 v[DT][2];           // block dt of hd, the two halves of the tile's positions
+};
+template <int DT>
+__device__ __forceinline__ void fetch_tile(TileRegs<DT>& t, const bf16_t* kt, int k_stride, const bf16_t* vt, int v_stride) {
+  const int lane = threadIdx.x % 64, r = lane % 16, c = lane / 16;
+  const int r8 = r % 8, q8 = (c + 4 * (r / 8)) * 8;
+#pragma unroll
+  for (int jt = 0; jt < 4; ++jt) {
+    const int row_a = 32 * (jt / 2) + 8 * (r8 / 4) + 4 * (jt % 2) + r8 % 4, row_b = row_a + 16;
+#pragma unroll
+    for (int p = 0; p < DT / 4; ++p) {
+      t.k[jt][2 * p] = ld16_once(kt + row_a * k_stride + 64 * p + q8);
+      t.k[jt][2 * p + 1] = ld16_once(kt + row_b * k_stride + 64 * p + q8);
+    }
+  }
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    t.v[dt][0] = ld16_once(vt + (16 * dt + r8) * v_stride + q8);
+    t.v[dt][1] = ld16_once(vt + (16 * dt + 8 + r8) * v_stride + q8);
+  }
+}
+template <int DT>
+__device__ __forceinline__ void tile_step_regs(f32x4 (&o)[1][DT], float (&m_run)[1], float (&l_run)[1],
+                                               const bf16x8 (&qf)[1][DT / 2], TileRegs<DT>& t, int pos0,
+                                               const int (&p_q)[1], const int (&lo_q)[1], float scale2, bool masked) {
+  f32x4 s[1][4];
+#pragma unroll
+  for (int jt = 0; jt < 4; ++jt) {
+    s[0][jt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int p = 0; p < DT / 4; ++p) to_own_row(t.k[jt][2 * p], t.k[jt][2 * p + 1]);
+#pragma unroll
+    for (int ks = 0; ks < DT / 2; ++ks)
+      s[0][jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, t.k[jt][ks]), qf[0][ks], s[0][jt], 0, 0, 0);
+  }
+  bf16x8 pf[2][1];
+  softmax_tile<DT, 1>(s, o, m_run, l_run, pos0, p_q, lo_q, scale2, masked, pf);
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    to_own_row(t.v[dt][0], t.v[dt][1]);
+    o[0][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, t.v[dt][0]), pf[0][0], o[0][dt], 0, 0, 0);
+    o[0][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, t.v[dt][1]), pf[1][0], o[0][dt], 0, 0, 0);
+  }
+}
+template <int DT>
+__device__ __forceinline__ void attend_ahead(f32x4 (&o)[1][DT], float (&m_run)[1], float (&l_run)[1],
+                                             const bf16x8 (&qf)[1][DT / 2], const bf16_t* kh, const bf16_t* vh,
+                                             const int* table, int page_size, int64_t page_stride, int tile_beg,
+                                             int tile_end, int p, bool valid, int lo_q, float scale2) {
+  constexpr int hd = 16 * DT;
+  const int pq[1] = {valid ? p : -1}, lq[1] = {lo_q};
+  TileRegs<DT> t0, t1;
+#define TQ_FETCH_TILE(regs, tile)                                                                          \
+  do {                                                                                                     \
+    const int pos0_ = (tile) * TILE;                                                                       \
+    const int64_t base_ = (int64_t)table[pos0_ / page_size] * page_stride;                                 \
+    const int in_page_ = pos0_ % page_size;                                                                \
+    fetch_tile<DT>(regs, kh + base_ + (int64_t)in_page_ * hd, hd, vh + base_ + in_page_, page_size);       \
+  } while (0)
+#define TQ_STEP_TILE(regs, tile)                                                                           \
+  do {                                                                                                     \
+    const int pos0_ = (tile) * TILE;                                                                       \
+    const bool masked_ = pos0_ + TILE - 1 > p || pos0_ < lo_q;                                             \
+    tile_step_regs<DT>(o, m_run, l_run, qf, regs, pos0_, pq, lq, scale2, masked_);                         \
+  } while (0)
+  TQ_FETCH_TILE(t0, tile_beg);
+  for (int tile = tile_beg; tile < tile_end; tile += 2) {
+    if (tile + 1 < tile_end) TQ_FETCH_TILE(t1, tile + 1);
+    TQ_STEP_TILE(t0, tile);
+    if (tile + 1 < tile_end) {
+      if (tile + 2 < tile_end) TQ_FETCH_TILE(t0, tile + 2);
+      TQ_STEP_TILE(t1, tile + 1);
+    }
+  }
+#undef TQ_FETCH_TILE
+#undef TQ_STEP_TILE
 }
 
 template <int DT>
@@ -416,8 +512,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 // then take the further runs in turn (wave x the runs x, x + the grid's runs, ...), each into its own place, so
 // that no wave has more than one or two of them (left to the last wave alone, 30 runs in a row made a step with
 // one sequence beyond position 4096 and seven shorter ones a third slower).
-template <int DT, bool EXACT>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DT > 8 ? 2 : 3))) void attn_decode_kernel(AttnArgs a) {
+// AHEAD (with EXACT): the form for steps of few waves, which fetches a tile ahead (attend_ahead).
+template <int DT, bool EXACT, bool AHEAD = false>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(AHEAD ? 1 : (DT > 8 ? 2 : 3)))) void attn_decode_kernel(AttnArgs a) {
   const int b = blockIdx.z;
   const int g = a.nh / a.nkv, ngc = (g + 15) / 16;
   const int kvh = blockIdx.y / ngc, cg = blockIdx.y % ngc;
@@ -442,8 +539,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DT > 8 ? 2 :
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[0][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     float m_run[1] = {-INFINITY}, l_run[1] = {0.f};
-    attend<DT, EXACT>(o, m_run, l_run, qf, a.k_pool + head_off, a.v_pool + head_off, table, a.page_size, a.page_stride,
-                      a.hd, tile_beg, tile_end, p, valid, lo, a.scale * LOG2E);
+    if constexpr (AHEAD)
+      attend_ahead<DT>(o, m_run, l_run, qf, a.k_pool + head_off, a.v_pool + head_off, table, a.page_size, a.page_stride,
+                       tile_beg, tile_end, p, valid, lo, a.scale * LOG2E);
+    else
+      attend<DT, EXACT>(o, m_run, l_run, qf, a.k_pool + head_off, a.v_pool + head_off, table, a.page_size, a.page_stride,
+                        a.hd, tile_beg, tile_end, p, valid, lo, a.scale * LOG2E);
     if (!valid) continue;
     float* out = a.partial + (((size_t)b * a.nh + h) * a.max_runs + run) * (a.hd + 2);
 #pragma unroll
@@ -523,7 +624,13 @@ static int launch_prefill(const AttnArgs& a, int B, int max_new, hipStream_t st)
 template <int DT, bool EXACT>
 static void launch_decode(const AttnArgs& a, int B, int grid_runs, hipStream_t st) {
   const int g = a.nh / a.nkv;
-  hipLaunchKernelGGL((attn_decode_kernel<DT, EXACT>), dim3(grid_runs, a.nkv * ((g + 15) / 16), B), dim3(64), 0, st, a);
+  const dim3 grid(grid_runs, a.nkv * ((g + 15) / 16), B);
+  // at most a wave to a SIMD: each has the registers to fetch a tile ahead (one sequence at position 8,191: 2.38 ms a
+  // step against 2.61; with more waves than that the form is no faster, from twice as many on slower)
+  if (EXACT && DT <= 8 && (int64_t)grid.x * grid.y * grid.z <= 1024)
+    hipLaunchKernelGGL((attn_decode_kernel<DT, EXACT, EXACT && DT <= 8>), grid, dim3(64), 0, st, a);
+  else
+    hipLaunchKernelGGL((attn_decode_kernel<DT, EXACT>), grid, dim3(64), 0, st, a);
   hipLaunchKernelGGL(attn_join_kernel, dim3(a.nh, B), dim3(64), 0, st, a);
 }
 
