@@ -878,6 +878,44 @@ def test_negative_log_likelihood(ops, V):
     assert torch.isnan(out[3]) and torch.isnan(out[4])
 
 
+@pytest.mark.parametrize("V", [10, 1000, 40001])
+def test_probabilities_in_16_bits_and_their_divergence(ops, V):
+    """A row's probabilities as the reference stores them (/root/reference/tools/quant.c:166-174, :594-602: made in
+    double, cut to a float and then to a 16-bit float whose mantissa is cut and whose small values are zero) and the
+    divergence of a baseline of such rows against them (:623-631), each against the same formulas in numpy."""
+    import numpy as np
+    R = 5
+    logits = rnd((R, V), torch.float32, 120, 3.0)
+    logits[1, 3] = 40.0                                    # one towering logit: everything else is cut to zero
+    other = logits + rnd((R, V), torch.float32, 121, 0.3)
+    def widen(h):
+        h = h.astype(np.uint32)
+        e, m = (h >> 10) & 0x1f, h & 0x3ff
+        return np.where(e == 0, 0, ((e + 112) << 23) | (m << 13)).astype(np.uint32).view(np.float32)
+    def cut(p):
+        bits = p.astype(np.float32).view(np.uint32)
+        e = ((bits >> 23) & 0xff).astype(np.int64) - 127 + 15
+        return np.where(e <= 0, 0, (e.clip(0, 30) << 10) | ((bits >> 13) & 0x3ff)).astype(np.uint16)
+    probs, none = ops.probs_half(logits.to(DEV), "float32")
+    assert none is None and probs.dtype == torch.int16
+    got = probs.cpu().numpy().view(np.uint16)
+    l64 = logits.double().numpy()
+    p = np.exp((l64 - l64.max(1, keepdims=True)) - np.log(np.exp(l64 - l64.max(1, keepdims=True)).sum(1, keepdims=True)))
+    want = cut(p)
+    assert (np.abs(got.astype(np.int64) - want.astype(np.int64)) <= 1).all() and (got == want).mean() > 0.999
+    assert (got[1] != 0).sum() == 1
+    base, _ = ops.probs_half(other.to(DEV), "float32")
+    same, kl = ops.probs_half(logits.to(DEV), "float32", want_probs=True, base=base)
+    assert torch.equal(same, probs) and kl.dtype == torch.float64
+    pb, pc = widen(base.cpu().numpy().view(np.uint16)).astype(np.float64), widen(got).astype(np.float64)
+    ref = np.where(pb > 1e-12, pb * (np.log(np.maximum(pb, 1e-300)) - np.log(np.maximum(pc, 1e-20))), 0.0).sum(1)
+    assert np.allclose(kl.cpu().numpy(), ref, rtol=1e-9, atol=1e-12)
+    zero = ops.probs_half(logits.to(DEV), "float32", want_probs=False, base=probs)[1]
+    assert torch.equal(zero, torch.zeros(R, dtype=torch.float64, device=zero.device))
+    with pytest.raises(ops.KernelError):
+        ops.probs_half(logits.to(DEV), "float32", want_probs=False)
+
+
 @pytest.mark.parametrize("V", [10, 1000, 151937])
 def test_argmax_first_maximum(ops, V):
     logits = rnd((3, V), torch.float32, 100)

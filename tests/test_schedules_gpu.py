@@ -344,6 +344,47 @@ def test_the_command_line_scores_a_file_of_tokens(act, sharp, tmp_path):
     assert json.loads(gen.stdout.strip().splitlines()[-1]) == json.loads(direct.stdout.strip().splitlines()[-1])
 
 
+def test_saved_probabilities_and_the_divergence_between_two_runs(sharp, tmp_path):
+    """``--save-logits`` and ``--kl-baseline`` beside ``--ppl`` (/root/reference/tools/quant.c:542-556, :594-636): the
+    32-bit run writes a header of two int32 and every scored position's probabilities as 16-bit floats; the same run
+    against its own file diverges by exactly 0, the bfloat16 run by little; a row of the file is the plain model's
+    softmax cut to the reference's 16-bit floats."""
+    import numpy as np
+    d, plain, _ = sharp("B", "float32")
+    d16, _, _ = sharp("B", "bfloat16")
+    (ids,) = prompts_for("B", [600], seed=34)
+    ids[100] = 10 ** 6
+    f = tmp_path / "tokens.txt"
+    f.write_text(" ".join(str(t) for t in ids) + "\n")
+    base = tmp_path / "base.bin"
+    quant = os.path.join(ROOT, "bin", "quant")
+    first = subprocess.run([sys.executable, quant, d, "--ppl", str(f), "--json", "--dtype", "float32", "--ctx", "1024",
+                            "--save-logits", str(base)], capture_output=True, text=True, timeout=300)
+    assert first.returncode == 0, first.stderr[-2000:]
+    assert f"Saved logits to {base}" in first.stderr
+    V = TINY["B"][0]["vocab_size"]
+    raw = np.fromfile(base, dtype="<u2", offset=8)
+    header = np.fromfile(base, dtype="<i4", count=2)
+    assert header.tolist() == [599, V] and raw.size == 598 * V        # the position before the stray token has no row
+    # row 0 against the plain model: p cut to 10 bits of mantissa, zero below 2^-14
+    fed = [t if t < 10 ** 6 else 0 for t in ids]
+    p = torch.softmax(plain.logits(fed)[0].double(), dim=-1).float().numpy()
+    bits = p.view(np.uint32)
+    e = ((bits >> 23) & 0xff).astype(np.int64) - 127 + 15
+    want = np.where(e <= 0, 0, (e.clip(0, 30) << 10) | ((bits >> 13) & 0x3ff)).astype(np.uint16)
+    got = raw[:V]
+    assert (np.abs(got.astype(np.int64) - want.astype(np.int64)) <= 1).all() and (got == want).mean() > 0.9
+    out = {}
+    for act, folder in (("float32", d), ("bfloat16", d16)):
+        run = subprocess.run([sys.executable, quant, folder, "--ppl", str(f), "--json", "--dtype", act, "--ctx", "1024",
+                              "--kl-baseline", str(base)], capture_output=True, text=True, timeout=300)
+        assert run.returncode == 0, run.stderr[-2000:]
+        out[act] = json.loads(run.stdout)
+        assert "KL divergence (baseline || this run): mean = " in run.stderr
+    assert out["float32"]["kl_tokens"] == 598 and out["float32"]["mean_kl"] == 0.0
+    assert out["bfloat16"]["kl_tokens"] == 598 and 0.0 < out["bfloat16"]["mean_kl"] < 0.01, out["bfloat16"]
+
+
 def test_a_context_length_binds_and_a_full_cache_ends_sequences(sharp):
     from turboquant_cpp_amd import Model
     d, plain, _ = sharp("A", "float32")

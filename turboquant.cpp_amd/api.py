@@ -10,6 +10,7 @@ import math
 import os
 from typing import Iterator, Sequence
 
+import numpy as np
 import torch
 
 from .csrc import ops
@@ -80,12 +81,18 @@ class Model:
         """Yields the tokens of one continuation (the reference's ``generate`` yields text pieces)."""
         yield from self.generate(list(prompt), **overrides)
 
-    def perplexity(self, tokens: Sequence[int], chunk: int = 512) -> dict:
+    def perplexity(self, tokens: Sequence[int], chunk: int = 512, save_logits: str | None = None,
+                   kl_baseline: str | None = None) -> dict:
         """Teacher-forced evaluation of a token sequence as the reference's ``--ppl`` does it
         (/root/reference/tools/quant.c:430-720): the sequence, cut to the context length, goes through the model once
         (here ``chunk`` tokens a step), and every token but the first is scored by the logits of the position
         before it.  Returns ``tokens``, ``tokens_evaluated`` (targets outside the vocabulary are left out, :575),
-        ``avg_nll`` and ``perplexity`` = exp(avg_nll)."""
+        ``avg_nll`` and ``perplexity`` = exp(avg_nll).
+
+        ``save_logits``: a file that receives, as the reference's ``--save-logits`` writes it (:542-547, :594-611), two
+        int32 (tokens - 1, vocabulary) and then every scored position's probabilities as 16-bit floats.
+        ``kl_baseline``: such a file of another run (another activation type, say); the result then also holds
+        ``mean_kl``, the mean over the scored positions of KL(baseline || this run), and ``kl_tokens`` (:612-636)."""
         self._ensure_open()
         tokens = [int(t) for t in tokens][:self.context_length]
         if len(tokens) < 2:
@@ -93,9 +100,18 @@ class Model:
         eng, act = self._engine, self._model.act
         V = eng.vocab_size
         feed = [t if 0 <= t < V else 0 for t in tokens]      # a token outside the vocabulary is fed as token 0, never scored
+        save_f = base_f = None
+        total, n_eval, total_kl, n_kl = 0.0, 0, 0.0, 0
         slot = eng.open(1)
-        total, n_eval = 0.0, 0
         try:
+            if save_logits:
+                save_f = open(save_logits, "wb")
+                save_f.write(np.array([len(tokens) - 1, V], dtype="<i4").tobytes())
+            if kl_baseline:
+                base_f = open(kl_baseline, "rb")
+                header = np.frombuffer(base_f.read(8), dtype="<i4")
+                if header.size != 2 or int(header[1]) != V:
+                    raise ValueError(f"KL baseline header mismatch (expected vocab={V})")
             for lo in range(0, len(tokens) - 1, chunk):
                 hi = min(lo + chunk, len(tokens) - 1)           # positions lo .. hi - 1 predict tokens lo + 1 .. hi
                 logits = eng.step(slot, [feed[lo:hi]], [list(range(hi - lo))])
@@ -104,12 +120,41 @@ class Model:
                 scored = ~torch.isnan(nll)
                 total += float(nll[scored].sum())
                 n_eval += int(scored.sum())
+                if save_f is None and base_f is None:
+                    continue
+                rows = torch.nonzero(scored).flatten()
+                if rows.numel() == 0:
+                    continue
+                if rows.numel() < hi - lo:                    # only scored positions have a row in either file
+                    logits = logits[rows.to(logits.device)].contiguous()
+                base = None
+                if base_f is not None:
+                    raw = np.frombuffer(base_f.read(rows.numel() * V * 2), dtype="<i2")
+                    have = raw.size // V                        # a baseline that ends early is compared as far as it goes
+                    if have:
+                        base = torch.from_numpy(raw[:have * V].reshape(have, V).copy()).to(logits.device)
+                probs = ops.probs_half(logits, act)[0] if save_f is not None else None
+                kl = None
+                if base is not None:
+                    cur = logits if base.shape[0] == logits.shape[0] else logits[:base.shape[0]].contiguous()
+                    kl = ops.probs_half(cur, act, want_probs=False, base=base)[1]
+                if save_f is not None:
+                    save_f.write(probs.cpu().numpy().astype("<i2").tobytes())
+                if kl is not None:
+                    total_kl += float(kl.sum())
+                    n_kl += kl.numel()
         finally:
             eng.close(slot)
+            for f in (save_f, base_f):
+                if f is not None:
+                    f.close()
         if n_eval == 0:
             raise ValueError("no token of the sequence is a token of the vocabulary")
         avg = total / n_eval
-        return {"tokens": len(tokens), "tokens_evaluated": n_eval, "avg_nll": avg, "perplexity": math.exp(avg)}
+        res = {"tokens": len(tokens), "tokens_evaluated": n_eval, "avg_nll": avg, "perplexity": math.exp(avg)}
+        if kl_baseline:
+            res.update({"mean_kl": total_kl / n_kl if n_kl else float("nan"), "kl_tokens": n_kl})
+        return res
 
     # ------------------------------------------------------------ lower level, for tests and tools
     @property

@@ -5,7 +5,9 @@ tokenizer in this library, so a prompt is a list of token ids (``-p "5,17,3"``; 
 ``;`` and run as one batch), or ``--random-prompt LEN[,LEN...]`` draws them.  ``--random-weights CONFIG.json --save
 DIR`` is the random-weights mode: it writes a model folder for a configuration and a seed and exits.  ``--ppl FILE``
 is the reference's teacher-forced perplexity (/root/reference/tools/quant.c:430-720) over a file of token ids, with its
-report and, with ``--json``, its JSON.
+report and, with ``--json``, its JSON; ``--save-logits FILE`` and ``--kl-baseline FILE`` go with it as in the reference
+(:542-556, :594-636): the first writes every scored position's probabilities, the second reports the mean KL divergence
+of such a file against this run (the 32-bit path against the bfloat16 path, for instance).
 """
 from __future__ import annotations
 
@@ -32,6 +34,10 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("-p", dest="prompt", default=None, help='token ids of the prompt, e.g. "5,17,3"; ";" separates prompts')
     ap.add_argument("--tokens-file", default=None, metavar="FILE", help="prompts from a file: one prompt of token ids a line")
     ap.add_argument("--ppl", default=None, metavar="FILE", help="compute perplexity on a file of token ids (teacher-forced)")
+    ap.add_argument("--save-logits", default=None, metavar="FILE",
+                    help="with --ppl: write every scored position's probabilities (16-bit floats) to FILE")
+    ap.add_argument("--kl-baseline", default=None, metavar="FILE",
+                    help="with --ppl: mean KL(baseline || this run) against a file that --save-logits wrote")
     ap.add_argument("-n", dest="max_tokens", type=int, default=256, help="max tokens to generate (default: 256)")
     ap.add_argument("-T", dest="temperature", type=float, default=0.7, help="sampling temperature (default: 0.7)")
     ap.add_argument("-P", dest="top_p", type=float, default=0.9, help="top-p sampling (default: 0.9)")
@@ -95,7 +101,7 @@ def main(argv=None) -> int:
         print(f"PPL evaluation: {min(len(ids), model.context_length)} tokens from {args.ppl}", file=sys.stderr)
         torch.cuda.synchronize()
         t1 = time.time()
-        res = model.perplexity(ids)
+        res = model.perplexity(ids, save_logits=args.save_logits, kl_baseline=args.kl_baseline)
         elapsed = time.time() - t1
         rate = res["tokens_evaluated"] / elapsed if elapsed > 0 else 0.0
         print("\n=== Perplexity Results ===", file=sys.stderr)
@@ -106,12 +112,18 @@ def main(argv=None) -> int:
         print(f"Perplexity:   {res['perplexity']:.4f}", file=sys.stderr)
         print(f"Time:         {elapsed:.1f}s ({rate:.1f} tok/s)", file=sys.stderr)
         print("==========================", file=sys.stderr)
+        if args.kl_baseline and res["kl_tokens"]:
+            print(f"KL divergence (baseline || this run): mean = {res['mean_kl']:.6f} over {res['kl_tokens']} tokens", file=sys.stderr)
+        if args.save_logits:
+            print(f"Saved logits to {args.save_logits}", file=sys.stderr)
         print(f"PPL_CSV:{res['tokens_evaluated']},{res['avg_nll']:.6f},{res['perplexity']:.4f}", file=sys.stderr)
         if args.json:
             print(json.dumps({"model": args.model, "benchmark": args.ppl, "tokens": res["tokens"],
                               "tokens_evaluated": res["tokens_evaluated"], "kv_type": args.dtype,
                               "perplexity": round(res["perplexity"], 4), "avg_nll": round(res["avg_nll"], 6),
-                              "elapsed_s": round(elapsed, 2), "tok_per_s": round(rate, 1)}, indent=2))
+                              "elapsed_s": round(elapsed, 2), "tok_per_s": round(rate, 1),
+                              **({"mean_kl": res["mean_kl"], "kl_tokens": res["kl_tokens"]} if args.kl_baseline else {})},
+                             indent=2))
         model.close()
         return 0
     if args.tokens_file:

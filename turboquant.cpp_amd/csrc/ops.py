@@ -50,6 +50,7 @@ _SIGNATURES = {
                  _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
     "tq_argmax": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr],
     "tq_nll": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr],
+    "tq_probs_half": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
     "tq_rep_penalty": [_c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_ptr, _c_f32, _c_ptr],
     "tq_sample_topp_scratch": [_c_int],
     "tq_sample_topp": [_c_ptr, _c_int, _c_int, _c_f32, _c_f32, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
@@ -805,6 +806,26 @@ def nll(logits: torch.Tensor, targets: torch.Tensor, act) -> torch.Tensor:
     out = torch.empty((R,), dtype=torch.float32, device=logits.device)
     _run(k, library(act).tq_nll(_ptr(logits), R, V, _ptr(targets), _ptr(out), _stream()))
     return out
+
+
+def probs_half(logits: torch.Tensor, act, want_probs: bool = True,
+               base: torch.Tensor | None = None) -> tuple[torch.Tensor | None, torch.Tensor | None]:
+    """Each row's probabilities as the reference stores them with ``--save-logits`` (16-bit floats made by its own
+    conversion: the mantissa cut, below 2^-14 zero; int16 [R, V], the bit patterns) and, with ``base`` (such rows of
+    another run), the KL divergence of ``base`` against this row, float64 [R]
+    (/root/reference/tools/quant.c:594-636)."""
+    k = "probs_half"
+    _check(logits, k, "logits", torch.float32)
+    _need(logits.dim() == 2, k, "logits must be [R, V]")
+    R, V = logits.shape
+    _need(want_probs or base is not None, k, "nothing is asked for")
+    probs = torch.empty((R, V), dtype=torch.int16, device=logits.device) if want_probs else None
+    kl = None
+    if base is not None:
+        _check(base, k, "base", torch.int16, (R, V))
+        kl = torch.empty((R,), dtype=torch.float64, device=logits.device)
+    _run(k, library(act).tq_probs_half(_ptr(logits), R, V, _ptr(probs), _ptr(base), _ptr(kl), _stream()))
+    return probs, kl
 
 
 def rep_penalty(logits: torch.Tensor, recent: torch.Tensor, counts: torch.Tensor, penalty: float, act) -> None:

@@ -96,6 +96,78 @@ TQ_API int tq_nll(const float* logits, int R, int V, const int* target, float* o
   return 0;
 }
 
+// ---------------------------------------------------------------- a row's probabilities as 16-bit floats, and KL against such rows
+// What the reference writes per scored position with --save-logits and compares with --kl-baseline
+// (/root/reference/tools/quant.c:594-636): p[j] = exp((l[j] - max) - log sum exp(l - max)) in double, made a float and
+// then a 16-bit float by its own conversion (:166-174: the mantissa cut, not rounded; below 2^-14 zero; no NaN).
+// KL(baseline || current) = sum over j with pb > 1e-12 of pb (log pb - log max(pc, 1e-20)) in double, pb and pc being
+// the 16-bit values widened again (:175-185).  One workgroup per row, sums over threads and waves in a fixed order.
+__device__ __forceinline__ unsigned short half_cut(float v) {
+  const uint32_t u = __float_as_uint(v);
+  const uint32_t sign = (u >> 16) & 0x8000u;
+  const int e = (int)((u >> 23) & 0xffu) - 127 + 15;
+  if (e <= 0) return (unsigned short)sign;
+  if (e >= 31) return (unsigned short)(sign | 0x7c00u);
+  return (unsigned short)(sign | ((uint32_t)e << 10) | ((u >> 13) & 0x3ffu));
+}
+__device__ __forceinline__ float half_widen(unsigned short h) {
+  const uint32_t sign = ((uint32_t)h & 0x8000u) << 16, e = (h >> 10) & 0x1fu, m = h & 0x3ffu;
+  if (e == 0) return __uint_as_float(sign);
+  if (e == 31) return __uint_as_float(sign | 0x7f800000u | (m << 13));
+  return __uint_as_float(sign | ((e - 15 + 127) << 23) | (m << 13));
+}
+__device__ __forceinline__ double block_sum_double(double v, double* dred) {
+#pragma unroll
+  for (int o = TQ_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, TQ_WAVE);
+  __syncthreads();
+  if (threadIdx.x % TQ_WAVE == 0) dred[threadIdx.x / TQ_WAVE] = v;
+  __syncthreads();
+  double total = 0.0;
+  for (int w = 0; w < ST / TQ_WAVE; ++w) total += dred[w];
+  return total;
+}
+
+// probs (null, or [R][V]): the row's probabilities; base (null, or [R][V]) with kl [R]: KL of base against them.
+__global__ __launch_bounds__(ST) void probs_half_kernel(const float* __restrict__ logits, int V,
+                                                        unsigned short* __restrict__ probs,
+                                                        const unsigned short* __restrict__ base, double* __restrict__ kl) {
+  __shared__ float red[ST / TQ_WAVE];
+  __shared__ double dred[ST / TQ_WAVE];
+  const float* row = logits + (size_t)blockIdx.x * V;
+  float mx = -INFINITY;
+  for (int i = threadIdx.x; i < V; i += ST) mx = fmaxf(mx, row[i]);
+  mx = block_max(mx, red);
+  double sum = 0.0;
+  for (int i = threadIdx.x; i < V; i += ST) sum += exp((double)(row[i] - mx));
+  const double log_sum = log(block_sum_double(sum, dred));
+  double part = 0.0;
+  for (int i = threadIdx.x; i < V; i += ST) {
+    const unsigned short h = half_cut((float)exp((double)(row[i] - mx) - log_sum));
+    if (probs) probs[(size_t)blockIdx.x * V + i] = h;
+    if (base) {
+      const float pb = half_widen(base[(size_t)blockIdx.x * V + i]);
+      float pc = half_widen(h);
+      if (pb > 1e-12f) {
+        if (pc < 1e-20f) pc = 1e-20f;
+        part += (double)pb * (log((double)pb) - log((double)pc));
+      }
+    }
+  }
+  if (base) {
+    const double total = block_sum_double(part, dred);
+    if (threadIdx.x == 0) kl[blockIdx.x] = total;
+  }
+}
+
+TQ_API int tq_probs_half(const float* logits, int R, int V, void* probs, const void* base, double* kl, hipStream_t st) {
+  if (R <= 0) return 0;
+  if ((!probs && !base) || (base && !kl)) return TQ_ERR_BAD_ARG;
+  hipLaunchKernelGGL(probs_half_kernel, dim3(R), dim3(ST), 0, st, logits, V, (unsigned short*)probs,
+                     (const unsigned short*)base, kl);
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
 // ---------------------------------------------------------------- repetition penalty
 // For each of the last `count` tokens of a row's history, once per occurrence: a positive logit is
 // divided by the penalty, any other multiplied (/root/reference/src/engine/tq_generate.c:387-400).

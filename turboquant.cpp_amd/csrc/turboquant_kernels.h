@@ -84,6 +84,7 @@ int tq_route(const float* x, const void* wr, const void* shared_w, int wtype, in
 // sampling.hip: greedy choice, negative log-likelihood, repetition penalty, temperature and top-p (both libraries; the two *_static entry points are declared in no_alloc.h)
 int tq_argmax(const float* logits, int R, int V, int* out, hipStream_t st);
 int tq_nll(const float* logits, int R, int V, const int* target, float* out, hipStream_t st);
+int tq_probs_half(const float* logits, int R, int V, void* probs, const void* base, double* kl, hipStream_t st);
 int tq_rep_penalty(float* logits, int R, int V, const int* recent, int window, const int* counts, float penalty,
         hipStream_t st);
 int64_t tq_sample_topp_scratch(int R);
