@@ -387,3 +387,42 @@ def test_generate_with_the_default_options_matches_the_plain_loop(cpu_engine, mo
         assert got.tokens == want
         reasons.append(got.finish_reason)
     assert "loop" in reasons
+
+
+def test_a_sequence_goes_back_to_an_earlier_position():
+    """``truncate`` forgets the positions from a point on and gives their pages back; it refuses where a window has
+    dropped pages that the earlier position would look at, and where the model keeps fixed-size state."""
+    from turboquant_cpp_amd.cache.paged import CacheError, PagedCache
+    from turboquant_cpp_amd.parts.base import CacheNeed, StateNeed
+    cache = PagedCache([(CacheNeed(2, 16), None, None), (CacheNeed(2, 16, window=100), None, None)], 64 * 10, torch.float32,
+                       None, page_size=64, max_slots=2)
+    s = cache.open()
+    cache.reserve(s, 200)
+    cache.commit(s)
+    assert cache.pages_held() == {0: 4, 1: 3}              # the window of 100 has let page 0 go
+    with pytest.raises(CacheError, match="window"):
+        cache.truncate(s, 120)                             # position 120 looks back to 21: page 0
+    cache.truncate(s, 170)                                 # looks back to 71: page 1
+    assert cache.length(s) == 170 and cache.pages_held() == {0: 3, 1: 2}
+    cache.truncate(s, 170)
+    with pytest.raises(CacheError):
+        cache.truncate(s, 171)
+    assert cache.reserve(s, 30) == 170
+    cache.commit(s)
+    assert cache.length(s) == 200 and cache.pages_held() == {0: 4, 1: 3}
+    cache.close(s)
+    assert cache.pages_held() == {0: 0, 1: 0}
+    plain = PagedCache([(CacheNeed(2, 16), None, None)], 64 * 4, torch.float32, None, page_size=64, max_slots=1)
+    s = plain.open()
+    plain.reserve(s, 130)
+    with pytest.raises(CacheError, match="reserved"):
+        plain.truncate(s, 10)
+    plain.commit(s)
+    plain.truncate(s, 0)
+    assert plain.length(s) == 0 and plain.pages_held() == {0: 0}
+    stateful = PagedCache([(None, StateNeed((4,)), None)], 64, torch.float32, None, page_size=64, max_slots=1)
+    s = stateful.open()
+    stateful.reserve(s, 5)
+    stateful.commit(s)
+    with pytest.raises(CacheError, match="state"):
+        stateful.truncate(s, 2)

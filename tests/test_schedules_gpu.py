@@ -385,6 +385,67 @@ def test_saved_probabilities_and_the_divergence_between_two_runs(sharp, tmp_path
     assert out["bfloat16"]["kl_tokens"] == 598 and 0.0 < out["bfloat16"]["mean_kl"] < 0.01, out["bfloat16"]
 
 
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_a_conversation_keeps_its_cache_between_turns(name, sharp, tmp_path):
+    """``Model.chat`` (the reference's chat, /root/reference/quant.h:17634-17700): every turn sends the whole history
+    and only what the cache does not hold yet is run; a history that parts from the cached tokens takes the cache back
+    to where they part (configuration A) or, where a window has dropped pages, starts over (B).  Every turn gives the
+    tokens that ``generate`` gives for the same history.  ``save_context`` / ``load_context`` carry the conversation
+    into another model object, which goes on with the same tokens; ``--save-kv`` / ``--load-kv`` do so on the command line
+    (/root/reference/src/engine/tq_generate.c:268-362)."""
+    from turboquant_cpp_amd import ChatContextOverflow, Model
+    d, _, _ = sharp(name, "float32")
+    opts = dict(dtype="float32", temperature=0.0, max_tokens=6, context_length=512)
+    h1, extra, other, more = prompts_for(name, [70, 9, 150, 5], seed=35)
+    with Model(d, **opts) as m, Model(d, **opts) as fresh:
+        brought = []
+        step = m.engine.step
+        m.engine.step = lambda slots, toks, *a, **k: (brought.append(len(toks[0])), step(slots, toks, *a, **k))[1]
+        out1 = m.chat(h1)
+        assert out1 == fresh.generate([h1])[0] and len(out1) == 6 and brought[0] == 70
+        del brought[:]
+        h2 = h1 + out1 + extra
+        out2 = m.chat(h2)
+        assert brought[0] == 1 + len(extra)           # the last token of turn 1 was never run, the new ones follow
+        assert out2 == fresh.generate([h2])[0]
+        ctx_file = str(tmp_path / "talk.kv")
+        m.save_context(ctx_file)
+        del brought[:]
+        h3 = h1[:40] + other                           # parts from the cache at token 40
+        out3 = m.chat(h3)
+        assert out3 == fresh.generate([h3])[0]
+        assert brought[0] == (len(h3) - 40 if name == "A" else len(h3)), brought
+        del brought[:]
+        assert m.chat(h3) == out3 and brought[0] == 1  # the same history again: only its last token is run
+        with pytest.raises(ChatContextOverflow):
+            m.chat(list(range(3)) * 200)
+        assert m.chat(None) == [] and m._chat_slot is None
+        # the saved conversation in another model object
+        with Model(d, **opts) as later:
+            later.load_context(ctx_file)
+            seen = []
+            lstep = later.engine.step
+            later.engine.step = lambda slots, toks, *a, **k: (seen.append(len(toks[0])), lstep(slots, toks, *a, **k))[1]
+            h4 = h2 + out2 + more
+            out4 = later.chat(h4)
+            assert seen[0] == 1 + len(more) and out4 == fresh.generate([h4])[0]
+        with Model(d, **dict(opts, dtype="bfloat16")) as wrong, pytest.raises(RuntimeError, match="float32"):
+            wrong.load_context(ctx_file)
+    # the command line: a prompt's cache saved once it has run, and a later run that goes on behind it
+    quant = [sys.executable, os.path.join(ROOT, "bin", "quant"), d, "--dtype", "float32", "-n", "6", "-T", "0", "--json",
+             "--ctx", "512"]
+    text = lambda toks: ",".join(str(t) for t in toks)
+    kv = str(tmp_path / "prompt.kv")
+    first = subprocess.run(quant + ["-p", text(h1), "--save-kv", kv], capture_output=True, text=True, timeout=300)
+    assert first.returncode == 0 and f"[save-kv] Saved {len(h1)} tokens to {kv}" in first.stderr, first.stderr[-2000:]
+    assert json.loads(first.stdout.strip().splitlines()[-1])[0]["tokens"] == out1
+    second = subprocess.run(quant + ["-p", text(extra), "--load-kv", kv], capture_output=True, text=True, timeout=300)
+    whole = subprocess.run(quant + ["-p", text(h1 + extra)], capture_output=True, text=True, timeout=300)
+    assert second.returncode == 0 and whole.returncode == 0, second.stderr[-2000:] + whole.stderr[-2000:]
+    assert f"[load-kv] Loaded {len(h1)} tokens from {kv}" in second.stderr
+    assert json.loads(second.stdout.strip().splitlines()[-1]) == json.loads(whole.stdout.strip().splitlines()[-1])
+
+
 def test_a_context_length_binds_and_a_full_cache_ends_sequences(sharp):
     from turboquant_cpp_amd import Model
     d, plain, _ = sharp("A", "float32")

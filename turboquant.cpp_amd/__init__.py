@@ -5,6 +5,6 @@ tokens and its next token.
 ``bin/trace_run`` replays given tokens step by step.
 """
 from . import config, parts, models  # noqa: F401  (importing registers parts and architectures)
-from .api import Model, load  # noqa: F401
+from .api import ChatContextOverflow, Model, load  # noqa: F401
 
 __version__ = "0.2.0"

@@ -6,6 +6,7 @@ part of the library).
 """
 from __future__ import annotations
 
+import json
 import math
 import os
 from typing import Iterator, Sequence
@@ -14,9 +15,15 @@ import numpy as np
 import torch
 
 from .csrc import ops
-from .engine.generate import GenerationOptions, GenerationResult, generate
+from .cache.paged import CacheError
+from .engine.generate import GenerationOptions, GenerationResult, continue_in_slot, generate
 from .engine.model import load_model, random_model
 from .engine.step import Engine
+
+
+class ChatContextOverflow(RuntimeError):
+    """The conversation no longer fits the context; the session has been reset
+    (/root/reference/bindings/python/quantcpp/__init__.py:44-60)."""
 
 
 class Model:
@@ -57,6 +64,7 @@ class Model:
         ctx = context_length if context_length > 0 else min(plan.max_positions, 4096)
         ctx = min(ctx, plan.max_positions)
         self.context_length = ctx
+        self._chat_slot, self._chat_tokens, self.last_finish_reason = None, [], None
         self.options = GenerationOptions(
             max_tokens=max_tokens, temperature=temperature, top_p=top_p, seed=seed, rep_penalty=rep_penalty,
             stop_tokens=tuple(stop_tokens) if stop_tokens is not None else tuple(plan.stop_tokens), max_batch=max_batch)
@@ -80,6 +88,136 @@ class Model:
     def stream(self, prompt: Sequence[int], **overrides) -> Iterator[int]:
         """Yields the tokens of one continuation (the reference's ``generate`` yields text pieces)."""
         yield from self.generate(list(prompt), **overrides)
+
+    # ------------------------------------------------------------ a conversation that keeps its cache
+    def chat(self, history: Sequence[int] | None, **overrides) -> list[int]:
+        """A turn of a conversation whose cache stays between calls, as the reference's ``chat``
+        (/root/reference/bindings/python/quantcpp/__init__.py:514-601, /root/reference/quant.h:17634-17700): send the
+        whole history every turn (token ids here); what it has in common with the tokens already in the cache is not
+        run again, only the rest is, and the continuation comes back.  ``None`` ends the conversation, as
+        ``reset_chat``.  Where the history parts from what the cache holds, the cache goes back to that point if it
+        can (no window has dropped pages there), else the conversation starts over.  Raises
+        :class:`ChatContextOverflow` (and resets) when the history does not fit the context."""
+        self._ensure_open()
+        if history is None:
+            self.reset_chat()
+            return []
+        history = self._align_chat(history)
+        opts = GenerationOptions(**{**self.options.__dict__, **overrides})
+        try:
+            res = continue_in_slot(self._engine, self._chat_slot, history, opts)
+        except BaseException:
+            self.reset_chat()
+            raise
+        self._chat_tokens = history + res.tokens
+        self.last_finish_reason = res.finish_reason
+        return res.tokens
+
+    def feed(self, history: Sequence[int]) -> int:
+        """Runs a history into the conversation's cache without generating (a long text read once, to be saved or
+        asked about later); returns the number of tokens the cache then holds."""
+        self._ensure_open()
+        history = self._align_chat(history, keep_last=False)
+        eng = self._engine
+        rest = history[eng.length(self._chat_slot):]
+        if rest:
+            try:
+                eng.step([self._chat_slot], [rest], [[]])
+            except BaseException:
+                self.reset_chat()
+                raise
+        self._chat_tokens = list(history)
+        return eng.length(self._chat_slot)
+
+    @property
+    def chat_tokens(self) -> list[int]:
+        """The tokens that the conversation's cache holds."""
+        if self._chat_slot is None:
+            return []
+        return self._chat_tokens[:self._engine.length(self._chat_slot)]
+
+    def _align_chat(self, history, keep_last: bool = True) -> list[int]:
+        """Brings the conversation's cache to the longest beginning that it shares with ``history`` (all but the
+        history's last token at most, if ``keep_last``: that one is run for its logits)."""
+        history = [int(t) for t in history]
+        if not history:
+            raise ValueError("the history needs at least one token")
+        eng = self._engine
+        if len(history) >= self.context_length:
+            self.reset_chat()
+            raise ChatContextOverflow("conversation history exceeds the model's context window; the session has "
+                                      "been reset, retry with a shorter history")
+        if self._chat_slot is None:
+            self._chat_slot, self._chat_tokens = eng.open(1)[0], []
+        held = self._chat_tokens[:eng.length(self._chat_slot)]
+        limit = min(len(held), len(history) - (1 if keep_last else 0))
+        common = 0
+        while common < limit and held[common] == history[common]:
+            common += 1
+        if common < len(held):
+            try:
+                eng.cache.truncate(self._chat_slot, common)
+            except CacheError:
+                eng.close([self._chat_slot])
+                self._chat_slot = eng.open(1)[0]
+        return history
+
+    def reset_chat(self) -> None:
+        """Forgets the conversation; the next ``chat`` starts afresh."""
+        if self._chat_slot is not None and self._engine is not None:
+            self._engine.close([self._chat_slot])
+        self._chat_slot, self._chat_tokens = None, []
+
+    def save_context(self, path: str) -> None:
+        """Writes the conversation's cache and tokens to a file, as the reference's ``save_context`` does
+        (/root/reference/quant.h:17518-17563; here a safetensors file: per cache group the pages the sequence holds,
+        the rows of fixed-size state, and the tokens): read a long text once, ask about it in later processes."""
+        self._ensure_open()
+        if self._chat_slot is None:
+            raise RuntimeError("there is no conversation to save")
+        from .weights.safetensors_io import write_safetensors
+        data = self._engine.cache.export_slot(self._chat_slot)
+        tensors = {"tokens": torch.tensor(self._chat_tokens[:data["length"]], dtype=torch.int32)}
+        groups = []
+        for i, g in enumerate(data["groups"]):
+            tensors[f"group.{i}.keys"] = g["keys"]
+            if g["values"] is not None:
+                tensors[f"group.{i}.values"] = g["values"]
+            groups.append({"first_page": g["first_page"], "entries": g["entries"], "key": list(g["key"])})
+        for e, st in data["states"].items():
+            tensors[f"state.{e}"] = st
+        meta = {"format": "turboquant_cpp_amd.context.1", "length": str(data["length"]), "page_size": str(data["page_size"]),
+                "groups": json.dumps(groups), "dtype": self._model.act}
+        write_safetensors(path, tensors, metadata=meta)
+
+    def load_context(self, path: str) -> None:
+        """Restores a conversation that ``save_context`` wrote (by a model of the same configuration and activation
+        type); the next ``chat`` runs only what its history holds beyond the saved tokens
+        (/root/reference/quant.h:17565-17622)."""
+        self._ensure_open()
+        from .weights.safetensors_io import SafetensorsFolder
+        with SafetensorsFolder(os.path.dirname(path) or ".", files=[path]) as f:
+            meta = f.metadata
+            if meta.get("format") != "turboquant_cpp_amd.context.1":
+                raise RuntimeError(f"{path} is no saved context")
+            if meta.get("dtype") != self._model.act:
+                raise RuntimeError(f"{path} was saved by a {meta.get('dtype')} model, this one is {self._model.act}")
+            groups = []
+            for i, g in enumerate(json.loads(meta["groups"])):
+                values = f.read(f"group.{i}.values").clone() if f"group.{i}.values" in f.entries else None
+                groups.append({"first_page": g["first_page"], "entries": g["entries"], "key": tuple(g["key"]),
+                               "keys": f.read(f"group.{i}.keys").clone(), "values": values})
+            states = {int(n.split(".")[1]): f.read(n).clone() for n in f.entries if n.startswith("state.")}
+            tokens = f.read("tokens").tolist()
+            data = {"length": int(meta["length"]), "page_size": int(meta["page_size"]), "groups": groups, "states": states}
+        if data["length"] >= self.context_length:
+            raise ChatContextOverflow(f"{path} holds {data['length']} tokens, the context is {self.context_length}")
+        self.reset_chat()
+        try:
+            self._chat_slot = self._engine.cache.import_slot(data)
+        except CacheError as e:
+            raise RuntimeError(f"cannot load {path}: {e}") from e
+        self._chat_tokens = tokens
 
     def perplexity(self, tokens: Sequence[int], chunk: int = 512, save_logits: str | None = None,
                    kl_baseline: str | None = None) -> dict:
@@ -171,6 +309,7 @@ class Model:
         return self._model.config
 
     def close(self) -> None:
+        self.reset_chat()
         self._engine = None
         self._model = None
 

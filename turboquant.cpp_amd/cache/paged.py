@@ -330,6 +330,92 @@ class PagedCache:
                     row[old] = -1
                     g.dirty.add(slot)
 
+    # ------------------------------------------------------------ a sequence that outlives its request
+    def truncate(self, slot: int, length: int) -> None:
+        """Forgets the positions from ``length`` on, so that the sequence can go on from there with other tokens.
+        Refused (CacheError) where that cannot be done: a group with a window has given back pages that a token at
+        ``length`` would look at, or the model keeps fixed-size state per sequence, which has no earlier value."""
+        s = self._live(slot)
+        if s.reserved:
+            raise CacheError(f"slot {slot} has positions reserved for a running step")
+        if not 0 <= length <= s.length:
+            raise CacheError(f"slot {slot} holds {s.length} positions, not {length}")
+        if length == s.length:
+            return
+        if any(state is not None for _c, state, _o in self._needs):
+            raise CacheError("a model with fixed-size state per sequence cannot go back to an earlier position")
+        last = (length - 1) // self.page_size if length else -1
+        for g in self.groups:
+            row = g.host_table[slot]
+            if any(row[p] < 0 for p in range(g.first_needed_page(length), last + 1)):
+                raise CacheError(f"the window of a group has given back pages that position {length} would look at")
+        for g in self.groups:
+            row = g.host_table[slot]
+            gone = [p for p in range(g.max_pages_per_seq) if row[p] >= 0 and (p > last or p < g.first_needed_page(length))]
+            if gone:
+                g.pool.give_back(row[gone].tolist())
+                row[gone] = -1
+                g.dirty.add(slot)
+        s.length = length
+
+    def export_slot(self, slot: int) -> dict:
+        """What the cache holds of one sequence, on the host: its length, per group the logical pages it holds
+        (first page, keys [pages, page elements], values) and per entry its row of fixed-size state."""
+        s = self._live(slot)
+        if s.reserved:
+            raise CacheError(f"slot {slot} has positions reserved for a running step")
+        out = {"length": s.length, "page_size": self.page_size, "groups": [], "states": {}}
+        last = (s.length - 1) // self.page_size if s.length else -1
+        for g in self.groups:
+            first = g.first_needed_page(s.length)
+            row = g.host_table[slot]
+            pages = [int(row[p]) for p in range(first, last + 1)]
+            if any(p < 0 for p in pages):
+                raise CacheError(f"slot {slot} does not hold all pages of its {s.length} positions")
+            idx = torch.tensor(pages, dtype=torch.int64, device=self.device)
+            entry = {"first_page": first, "entries": list(g.entries), "key": (g.key.num_kv_heads, g.key.head_dim, g.key.value_dim, g.key.window),
+                     "keys": g.k_pages.view(-1, g.page_stride)[idx].cpu(), "values": None}
+            if g.v_pages is not None:
+                entry["values"] = g.v_pages.view(-1, g.v_page_stride)[idx].cpu()
+            out["groups"].append(entry)
+        for e, st in self.states.items():
+            out["states"][e] = st[slot].cpu()
+        return out
+
+    def import_slot(self, data: dict) -> int:
+        """A new slot that holds what ``export_slot`` gave (of a cache of the same model, page size and type)."""
+        if data["page_size"] != self.page_size or len(data["groups"]) != len(self.groups):
+            raise CacheError("the saved sequence comes from a cache of another layout")
+        for g, d in zip(self.groups, data["groups"]):
+            if tuple(d["key"]) != (g.key.num_kv_heads, g.key.head_dim, g.key.value_dim, g.key.window) or \
+                    list(d["entries"]) != list(g.entries) or d["keys"].dtype != self.dtype or \
+                    d["keys"].shape[1] != g.page_stride or (d["values"] is None) != (g.v_pages is None):
+                raise CacheError("the saved sequence comes from a cache of another layout")
+        slot = self.open()
+        try:
+            length = int(data["length"])
+            if length:
+                self.reserve(slot, length)
+                self.commit(slot)
+            last = (length - 1) // self.page_size if length else -1
+            for g, d in zip(self.groups, data["groups"]):
+                first = g.first_needed_page(length)
+                if d["first_page"] != first or d["keys"].shape[0] != last + 1 - first:
+                    raise CacheError("the saved pages do not cover the saved length")
+                row = g.host_table[slot]
+                idx = torch.tensor([int(row[p]) for p in range(first, last + 1)], dtype=torch.int64, device=self.device)
+                if idx.numel():
+                    g.k_pages.view(-1, g.page_stride)[idx] = d["keys"].to(self.device)
+                    if g.v_pages is not None:
+                        g.v_pages.view(-1, g.v_page_stride)[idx] = d["values"].to(self.device)
+            for e, st in data["states"].items():
+                self.states[int(e)][slot].copy_(st.to(self.device))
+        except BaseException:
+            self.slots[slot].reserved = 0
+            self.close(slot)
+            raise
+        return slot
+
     def sync(self) -> None:
         for g in self.groups:
             g.sync()

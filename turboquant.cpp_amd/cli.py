@@ -7,7 +7,9 @@ DIR`` is the random-weights mode: it writes a model folder for a configuration a
 is the reference's teacher-forced perplexity (/root/reference/tools/quant.c:430-720) over a file of token ids, with its
 report and, with ``--json``, its JSON; ``--save-logits FILE`` and ``--kl-baseline FILE`` go with it as in the reference
 (:542-556, :594-636): the first writes every scored position's probabilities, the second reports the mean KL divergence
-of such a file against this run (the 32-bit path against the bfloat16 path, for instance).
+of such a file against this run (the 32-bit path against the bfloat16 path, for instance).  ``--save-kv FILE`` and
+``--load-kv FILE`` are the reference's too (/root/reference/src/engine/tq_generate.c:268-362): the cache of one prompt
+saved once it has run, and a later run that starts from it with its prompt behind the saved tokens.
 """
 from __future__ import annotations
 
@@ -34,6 +36,10 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("-p", dest="prompt", default=None, help='token ids of the prompt, e.g. "5,17,3"; ";" separates prompts')
     ap.add_argument("--tokens-file", default=None, metavar="FILE", help="prompts from a file: one prompt of token ids a line")
     ap.add_argument("--ppl", default=None, metavar="FILE", help="compute perplexity on a file of token ids (teacher-forced)")
+    ap.add_argument("--save-kv", default=None, metavar="FILE",
+                    help="one prompt: save the cache after the prompt has been run, before anything is generated")
+    ap.add_argument("--load-kv", default=None, metavar="FILE",
+                    help="one prompt: start from a saved cache; the prompt goes on behind its tokens")
     ap.add_argument("--save-logits", default=None, metavar="FILE",
                     help="with --ppl: write every scored position's probabilities (16-bit floats) to FILE")
     ap.add_argument("--kl-baseline", default=None, metavar="FILE",
@@ -139,7 +145,25 @@ def main(argv=None) -> int:
         prompts = parse_prompts(args.prompt if args.prompt is not None else "1")
     torch.cuda.synchronize()
     t1 = time.time()
-    results = model.generate_detailed(prompts)
+    if args.save_kv or args.load_kv:
+        # the reference's --load-kv / --save-kv (/root/reference/src/engine/tq_generate.c:268-362): the loaded cache
+        # holds the first positions and the prompt goes on behind them; the cache is saved when the prompt has run
+        from .engine.generate import GenerationResult
+        if len(prompts) != 1:
+            raise ValueError("--save-kv and --load-kv take one prompt")
+        before = []
+        if args.load_kv:
+            model.load_context(args.load_kv)
+            before = model.chat_tokens
+            print(f"[load-kv] Loaded {len(before)} tokens from {args.load_kv}", file=sys.stderr)
+        history = before + list(prompts[0])
+        if args.save_kv:
+            n = model.feed(history)
+            model.save_context(args.save_kv)
+            print(f"[save-kv] Saved {n} tokens to {args.save_kv}", file=sys.stderr)
+        results = [GenerationResult(model.chat(history), model.last_finish_reason)]
+    else:
+        results = model.generate_detailed(prompts)
     torch.cuda.synchronize()
     elapsed = time.time() - t1
     n_generated = sum(len(r.tokens) for r in results)

@@ -230,3 +230,41 @@ def generate(engine, prompts: Sequence[Sequence[int]], options: GenerationOption
         finally:
             engine.close(list(slot_of.values()))
     return results
+
+
+def continue_in_slot(engine, slot: int, history: Sequence[int], options: GenerationOptions | None = None) -> GenerationResult:
+    """One sequence that outlives the call, as the reference's chat keeps its state between turns
+    (/root/reference/quant.h:17634-17700): ``history`` is everything the sequence has seen and is to see, the slot's
+    cache holds its first ``engine.length(slot)`` tokens (fewer than all of them), the rest is run as one prompt step
+    and a continuation is generated.  The slot stays open; afterwards its cache holds the history and the generated
+    tokens but the last, if that one ended the turn by its number (``engine.length(slot)`` says how many)."""
+    o = options or GenerationOptions()
+    cached = engine.length(slot)
+    if not 0 <= cached < len(history):
+        raise ValueError(f"the cache holds {cached} tokens, the history {len(history)}: at least one must be new")
+    max_pos = engine.cache.max_positions
+    if len(history) > max_pos:
+        return GenerationResult([], "context")
+    if o.max_tokens < 1:
+        return GenerationResult([], "length")
+    sampler = Sampler(o.sampling(), engine.model.act, engine.device)
+    track = SequenceTrack.start(0, history, o, max_pos)
+    state = sampler.new_sequence(0, list(history))
+    fetch = TokenFetch(engine.device, 1)
+    try:
+        logits = engine.step([slot], [list(history[cached:])])
+    except CacheFull:
+        return GenerationResult([], "context")
+    while True:
+        ids = sampler.launch(logits, [state])
+        fetch.start(ids)
+        tokens = fetch.wait()
+        sampler.finish(tokens, [state])
+        if not track.accept(tokens[0]):
+            break
+        try:
+            logits = engine.step([slot], [[tokens[0]]])
+        except CacheFull:
+            track.finish_reason = "context"
+            break
+    return GenerationResult(track.out, track.finish_reason)

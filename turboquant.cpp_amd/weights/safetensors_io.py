@@ -45,14 +45,17 @@ class TensorEntry:
 
 
 class SafetensorsFolder:
-    """All shards of a model folder, memory-mapped; tensors are read by name."""
+    """All shards of a model folder (or the given files), memory-mapped; tensors are read by name.  ``metadata``
+    holds the files' ``__metadata__`` entries."""
 
-    def __init__(self, model_dir: str):
+    def __init__(self, model_dir: str, files: list[str] | None = None):
         self.model_dir = model_dir
-        files = find_shards(model_dir)
-        if not files:
-            raise SafetensorsError(f"no model.safetensors (or model-*-of-*.safetensors) in {model_dir!r}")
+        if files is None:
+            files = find_shards(model_dir)
+            if not files:
+                raise SafetensorsError(f"no model.safetensors (or model-*-of-*.safetensors) in {model_dir!r}")
         self.files = files
+        self.metadata: dict[str, str] = {}
         self._maps: list[mmap.mmap] = []
         self._handles = []
         self._data_start: list[int] = []
@@ -79,6 +82,7 @@ class SafetensorsFolder:
         self._data_start.append(start)
         for name, info in header.items():
             if name == "__metadata__":
+                self.metadata.update(info or {})
                 continue
             dtype = info.get("dtype")
             if dtype not in DTYPES:
