@@ -7,4 +7,4 @@ tokens and its next token.
 from . import config, parts, models  # noqa: F401  (importing registers parts and architectures)
 from .api import ChatContextOverflow, Model, load  # noqa: F401
 
-__version__ = "0.2.0"
+__version__ = "0.3.0"
