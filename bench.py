@@ -109,6 +109,14 @@ def probe() -> int:
     return 0
 
 
+def plain_products(short: str) -> str:
+    """Whose kernels run the plain products of a long prompt step (decode steps always run this library's own)."""
+    from turboquant_cpp_amd.csrc import ops
+    if short == "bf16" and ops._VENDOR:
+        return f"hipBLASLt from {ops.VENDOR_MIN_ROWS} rows (TQ_PLAIN_PRODUCTS=own: this library's)"
+    return "own kernels"
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -267,7 +275,7 @@ def main() -> int:
                        "weights": f"random N(0,0.02) seed {wl['seed']}", "kv_cache": short,
                        "experts_read_per_layer": round(used, 1), "parallelism": "single GPU"},
             "prefill": {"value": round(T / t_prompt, 1), "tokens": T, "ms": round(t_prompt * 1e3, 3),
-                        "frac": round(flops / t_prompt / PEAK_FLOPS[short], 4)},
+                        "frac": round(flops / t_prompt / PEAK_FLOPS[short], 4), "plain_products": plain_products(short)},
             "roofline": {"bound": "hbm", "achieved": round(read / sec / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": round(read / sec / 1e9 / PEAK_HBM_GBS, 4)},
             "decode": {"ms_total": round(t_decode * 1e3, 2), "gb_per_step": round(read / 1e9, 2)},
@@ -387,7 +395,8 @@ def main() -> int:
             "experts_read_per_layer": round(experts_used, 1),
         },
         "prefill": {"value": round(PREFILL_TOKENS / pf, 1), "tokens": PREFILL_TOKENS, "ms": round(pf * 1e3, 3),
-                    "frac": round(prefill_flops(cfg, args.layers, PREFILL_TOKENS) / pf / PEAK_FLOPS[short], 4)},
+                    "frac": round(prefill_flops(cfg, args.layers, PREFILL_TOKENS) / pf / PEAK_FLOPS[short], 4),
+                    "plain_products": plain_products(short)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4)},
         "points": points,
