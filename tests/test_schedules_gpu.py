@@ -311,6 +311,23 @@ def test_the_command_line_generates(act, sharp):
     assert info.returncode == 0 and "Qwen2MoeForCausalLM" in info.stdout
 
 
+def test_the_command_line_says_where_the_time_goes(sharp):
+    """``--profile`` in the reference's manner (/root/reference/src/engine/tq_transformer.c:2995-3020): after the
+    generation, a prompt step and sixteen decode steps run eagerly with an event behind every launch, and the time is
+    put down to products, experts, attention and the rest."""
+    d, _, _ = sharp("B", "bfloat16")
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "quant"), d, "-p", "5,17,3,9;8,1", "-n", "3", "-T", "0",
+                          "--profile"], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr[-2000:]
+    lines = [l for l in run.stderr.splitlines() if l.startswith("PROFILE_CSV:")]
+    assert [l.split(":")[1].split(",")[0] for l in lines] == ["prompt", "decode"]
+    for l, n_tok in zip(lines, (6, 32)):
+        f = l.split(":")[1].split(",")
+        total, parts = float(f[2]), [float(v) for v in f[3:]]
+        assert int(f[1]) == n_tok and total > 0 and all(v > 0 for v in parts) and abs(sum(parts) - total) < 1e-2 * total
+    assert "[Profile prompt, 6 tok] matmul=" in run.stderr and "[Profile decode, 32 tok] matmul=" in run.stderr
+
+
 @pytest.mark.parametrize("act", ACTS)
 def test_the_command_line_scores_a_file_of_tokens(act, sharp, tmp_path):
     """``bin/quant DIR --ppl FILE --json`` (the reference's teacher-forced perplexity, /root/reference/tools/quant.c:430-720):

@@ -176,20 +176,38 @@ def main(argv=None) -> int:
         print(f"{n_generated} tokens in {elapsed:.1f}s ({n_generated / elapsed:.1f} tok/s, {len(prompts)} sequences, "
               f"weights={args.dtype}, kv={args.dtype})", file=sys.stderr)
     if args.profile:
-        eng = model.engine
+        # Where the time of a forward pass goes, by kind of work, in the reference's line
+        # (/root/reference/src/engine/tq_transformer.c:2995-3020): steps run eagerly on one stream, an event behind
+        # every launch.
+        from .csrc import ops
+        from .engine.step import Engine
+        eng = Engine(model._model, max_tokens=sum(-(-(len(p) + 17) // 64) * 64 for p in prompts), page_size=64,
+                     max_slots=len(prompts), use_graphs=False)
+        eng.side_stream = None
         slots = eng.open(len(prompts))
-        torch.cuda.synchronize()
-        t = time.time()
+
+        def report(phase, n_tok, steps):
+            t = ops.profile_end()
+            per = t["total"] / n_tok if n_tok else 0.0
+            pct = {k: 100.0 * t[k] / t["total"] if t["total"] > 0 else 0.0 for k in ("matmul", "moe", "attn", "other")}
+            print(f"[Profile {phase}, {n_tok} tok] matmul={pct['matmul']:.1f}% moe={pct['moe']:.1f}% attn={pct['attn']:.1f}% "
+                  f"other={pct['other']:.1f}% | per-tok: {per:.4f}ms (mat={t['matmul'] / n_tok:.4f} moe={t['moe'] / n_tok:.4f} "
+                  f"attn={t['attn'] / n_tok:.4f} other={t['other'] / n_tok:.4f}) | per-step: {t['total'] / steps:.3f}ms",
+                  file=sys.stderr)
+            print(f"PROFILE_CSV:{phase},{n_tok},{t['total']:.3f},{t['matmul']:.3f},{t['moe']:.3f},{t['attn']:.3f},{t['other']:.3f}",
+                  file=sys.stderr)
+
+        eng.step(slots, [list(p) for p in prompts])            # the kernels' first launches are not timed
+        eng.close(slots)
+        slots = eng.open(len(prompts))
+        ops.profile_begin()
         eng.step(slots, [list(p) for p in prompts])
-        torch.cuda.synchronize()
-        t_prompt = time.time() - t
-        t = time.time()
+        report("prompt", sum(len(p) for p in prompts), 1)
+        eng.step(slots, [[1] for _ in prompts])
+        ops.profile_begin()
         for _ in range(16):
             eng.step(slots, [[1] for _ in prompts])
-        torch.cuda.synchronize()
-        t_dec = (time.time() - t) / 16
+        report("decode", 16 * len(prompts), 16)
         eng.close(slots)
-        print(f"profile: prompt step {t_prompt * 1e3:.2f} ms ({sum(len(p) for p in prompts)} tokens), "
-              f"decode step {t_dec * 1e3:.2f} ms ({len(prompts)} sequences)", file=sys.stderr)
     model.close()
     return 0

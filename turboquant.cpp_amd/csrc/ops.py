@@ -153,8 +153,44 @@ def _check(t: torch.Tensor, kernel: str, name: str, dtype=None, shape=None) -> N
         raise KernelError(f"{kernel}: {name} must have shape {tuple(shape)}, has {tuple(t.shape)}")
 
 
-def _run(kernel: str, code: int) -> None:
+# Timing by kind of work, as the reference's --profile has it (/root/reference/src/engine/tq_transformer.c:60-93,
+# :2995-3020: matmul, moe, attn and the rest): while a profile is open, an event is recorded behind every launch, and
+# the time between two events is put down to the kernel between them (the step must run on one stream).
+_PROFILE: list | None = None
+_KIND = {"gemm": "matmul", "gemm_mfma": "matmul", "gemm_f32": "matmul", "gemm_pair": "matmul", "qkv_rope_write": "matmul",
+         "gated_act": "matmul", "attention": "attn", "attention_mfma": "attn", "attention_f32": "attn",
+         "router_topk": "moe", "route": "moe", "moe_align": "moe", "moe_combine": "moe"}
+
+
+def profile_begin() -> None:
+    global _PROFILE
+    e = torch.cuda.Event(enable_timing=True)
+    e.record()
+    _PROFILE = [(None, e)]
+
+
+def profile_end() -> dict[str, float]:
+    """Milliseconds per kind since ``profile_begin`` ("matmul", "moe", "attn", "other") and "total"."""
+    global _PROFILE
+    marks, _PROFILE = _PROFILE or [], None
+    torch.cuda.synchronize()
+    out = {"matmul": 0.0, "moe": 0.0, "attn": 0.0, "other": 0.0}
+    for (_, before), (kind, after) in zip(marks, marks[1:]):
+        out[kind] += before.elapsed_time(after)
+    out["total"] = sum(out.values())
+    return out
+
+
+def _mark(kind: str) -> None:
+    e = torch.cuda.Event(enable_timing=True)
+    e.record()
+    _PROFILE.append((kind, e))
+
+
+def _run(kernel: str, code: int, kind: str | None = None) -> None:
     if code == 0:
+        if _PROFILE is not None:
+            _mark(kind or _KIND.get(kernel, "other"))
         return
     if code == -1:
         raise KernelError(f"{kernel}: arguments rejected by the launcher")
@@ -494,7 +530,10 @@ def _vendor_gemm(a, w, out_act: bool) -> torch.Tensor:
     """a w^T by the vendor library: sums in float32, stored as bfloat16 or float32.  It adds no bias: its product
     with one takes a pass more over the result (77 against 48 us), so a product with a bias stays here unless the
     caller has a kernel behind it that adds the bias on its way."""
-    return torch.mm(a, w.t()) if out_act else torch.mm(a, w.t(), out_dtype=torch.float32)
+    out = torch.mm(a, w.t()) if out_act else torch.mm(a, w.t(), out_dtype=torch.float32)
+    if _PROFILE is not None:
+        _mark("matmul")
+    return out
 
 
 VENDOR_GATED_ROWS = 4096      # rows of a gated pair that go through the vendor library at a time
@@ -522,6 +561,8 @@ def _vendor_gated(a, w, N: int, K: int, gate: int, act) -> torch.Tensor:
     for r in range(0, M, VENDOR_GATED_ROWS):
         rows = min(VENDOR_GATED_ROWS, M - r)
         gu = torch.mm(a[r:r + rows], both.t(), out_dtype=torch.float32)
+        if _PROFILE is not None:
+            _mark("matmul")
         _run("gated_act", lib.tq_gated_act(_ptr(gu), 2 * N, _ptr(out[r:]), rows, N, gate, _stream()))
     return out
 
@@ -575,7 +616,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, act, bias: torch.Tensor | None = None
         _run("gemm_mfma", lib.tq_gemm_mfma(_ptr(a), a.stride(0), _ptr(a_rows), int(gather), _ptr(w), _ptr(w2), gstride,
                                            _ptr(tile_group), _ptr(n_tiles), _ptr(bias),
                                            _WTYPE[bias.dtype] if bias is not None else 0, _ptr(out), N, int(out_act),
-                                           M, N, K, tile_rows, splits, gate, _stream()))
+                                           M, N, K, tile_rows, splits, gate, _stream()), "moe" if grouped else None)
         return out
     if _use_f32(act, a, w, K, gstride) and (w2 is None or w2.data_ptr() % 16 == 0):
         # a narrow matrix times few rows is cut into runs of k: they come back apart if the caller adds them up
@@ -588,13 +629,14 @@ def gemm(a: torch.Tensor, w: torch.Tensor, act, bias: torch.Tensor | None = None
         _run("gemm_f32", lib.tq_gemm_f32(_ptr(a), a.stride(0), _ptr(a_rows), int(gather), _ptr(w), _ptr(w2), gstride,
                                          _ptr(tile_group), _ptr(n_tiles), _ptr(bias),
                                          _WTYPE[bias.dtype] if bias is not None else 0, _ptr(out), N, M, N, K, tile_rows,
-                                         gate, _ptr(scratch), int(partial_sums and runs > 1), _stream()))
+                                         gate, _ptr(scratch), int(partial_sums and runs > 1), _stream()),
+             "moe" if grouped else None)
         return out
     out = torch.empty((1, M, N) if partial_sums else (M, N), dtype=adt if out_act else torch.float32, device=a.device)
     _run(k, lib.tq_gemm_generic(_ptr(a), a.stride(0), _ptr(a_rows), int(gather), _ptr(w), _ptr(w2), _WTYPE[w.dtype], gstride,
                                 _ptr(tile_group), _ptr(n_tiles), _ptr(bias),
                                 _WTYPE[bias.dtype] if bias is not None else 0, _ptr(out), N, int(out_act), M, N, K,
-                                tile_rows, gate, _stream()))
+                                tile_rows, gate, _stream()), "moe" if grouped else None)
     return out
 
 
@@ -643,7 +685,8 @@ def gemm_pair(first: dict, second: dict, act) -> tuple[torch.Tensor, torch.Tenso
                 _WTYPE[p["bias"].dtype] if p["bias"] is not None else 0, _ptr(out), N, int(p["out_act"]), M, N, K, tile_rows,
                 _gate_code(k, p["activation"])]
         descs.append((ctypes.c_int64 * 19)(*[0 if v is None else int(v) for v in vals]))
-    _run(k, lib.tq_gemm_mfma_pair(descs[0], descs[1], splits, _stream()))
+    _run(k, lib.tq_gemm_mfma_pair(descs[0], descs[1], splits, _stream()),
+         "moe" if any(p["tile_group"] is not None for p in probs) else None)
     return outs[0], outs[1]
 
 
