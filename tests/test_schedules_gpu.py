@@ -326,6 +326,37 @@ def test_the_command_line_says_where_the_time_goes(sharp):
         total, parts = float(f[2]), [float(v) for v in f[3:]]
         assert int(f[1]) == n_tok and total > 0 and all(v > 0 for v in parts) and abs(sum(parts) - total) < 1e-2 * total
     assert "[Profile prompt, 6 tok] matmul=" in run.stderr and "[Profile decode, 32 tok] matmul=" in run.stderr
+    assert "add_rmsnorm" in run.stderr and "(experts)" in run.stderr and " launches " in run.stderr
+
+
+def test_the_replay_tool_shows_the_stream_behind_every_layer(sharp, tmp_path):
+    """``bin/trace_run --dump-layers``: beside a step's logits, the residual stream behind every layer at the wanted
+    places (the reference prints activations under TQ_DEBUG, /root/reference/src/engine/tq_transformer.c:2340-2344);
+    against the plain model's stream layer by layer, in float32."""
+    import numpy as np
+    from plain_qwen2moe import rmsnorm
+    d, plain, _ = sharp("B", "float32")
+    (ids,) = prompts_for("B", [21], seed=36)
+    out = tmp_path / "out"
+    lines = [json.dumps({"step": 0, "entries": [{"id": "a", "tokens": ids[:20], "want": [0, 19]}], "end": []}),
+             json.dumps({"step": 1, "entries": [{"id": "a", "tokens": ids[20:], "want": [0]}], "end": ["a"]})]
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", d, "--dtype", "float32", "--out", str(out),
+                          "--max-tokens", "64", "--dump-layers"], input="\n".join(lines) + "\n", capture_output=True, text=True,
+                         timeout=300)
+    assert run.returncode == 0 and "done 1" in run.stdout, run.stderr[-2000:]
+    t, L, H = plain.t, plain.L, plain.cfg["hidden_size"]
+    x = t["model.embed_tokens.weight"][ids]
+    stream = []
+    for l in range(L):
+        x = x + plain.attention_layer(l, rmsnorm(x, t[f"model.layers.{l}.input_layernorm.weight"], plain.eps))
+        x = x + plain.ffn_layer(l, rmsnorm(x, t[f"model.layers.{l}.post_attention_layernorm.weight"], plain.eps))
+        stream.append(x.clone())
+    want = torch.stack(stream)                     # [L, 21, H]
+    got0 = torch.from_numpy(np.fromfile(out / "0.layers.f32", dtype="<f4").reshape(L, 2, H).copy()).double()
+    got1 = torch.from_numpy(np.fromfile(out / "1.layers.f32", dtype="<f4").reshape(L, 1, H).copy()).double()
+    scale = want.abs().max().item()
+    assert (got0 - want[:, [0, 19]]).abs().max().item() < 1e-5 * scale
+    assert (got1 - want[:, [20]]).abs().max().item() < 1e-5 * scale
 
 
 @pytest.mark.parametrize("act", ACTS)

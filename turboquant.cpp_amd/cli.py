@@ -196,6 +196,8 @@ def main(argv=None) -> int:
                   file=sys.stderr)
             print(f"PROFILE_CSV:{phase},{n_tok},{t['total']:.3f},{t['matmul']:.3f},{t['moe']:.3f},{t['attn']:.3f},{t['other']:.3f}",
                   file=sys.stderr)
+            for name, (calls, ms) in sorted(t["kernels"].items(), key=lambda kv: -kv[1][1]):
+                print(f"    {name:28s} {calls:6d} launches {ms:10.3f} ms {100.0 * ms / t['total']:5.1f}%", file=sys.stderr)
 
         eng.step(slots, [list(p) for p in prompts])            # the kernels' first launches are not timed
         eng.close(slots)

@@ -169,28 +169,36 @@ def profile_begin() -> None:
     _PROFILE = [(None, e)]
 
 
-def profile_end() -> dict[str, float]:
-    """Milliseconds per kind since ``profile_begin`` ("matmul", "moe", "attn", "other") and "total"."""
+def profile_end() -> dict:
+    """Milliseconds per kind since ``profile_begin`` ("matmul", "moe", "attn", "other"), "total", and "kernels":
+    name -> [launches, milliseconds]."""
     global _PROFILE
     marks, _PROFILE = _PROFILE or [], None
     torch.cuda.synchronize()
     out = {"matmul": 0.0, "moe": 0.0, "attn": 0.0, "other": 0.0}
-    for (_, before), (kind, after) in zip(marks, marks[1:]):
-        out[kind] += before.elapsed_time(after)
+    kernels: dict[str, list] = {}
+    for (_, before), ((kind, name), after) in zip(marks, marks[1:]):
+        ms = before.elapsed_time(after)
+        out[kind] += ms
+        row = kernels.setdefault(name, [0, 0.0])
+        row[0] += 1
+        row[1] += ms
     out["total"] = sum(out.values())
+    out["kernels"] = kernels
     return out
 
 
-def _mark(kind: str) -> None:
+def _mark(kind: str, name: str = "vendor product") -> None:
     e = torch.cuda.Event(enable_timing=True)
     e.record()
-    _PROFILE.append((kind, e))
+    _PROFILE.append(((kind, name), e))
 
 
 def _run(kernel: str, code: int, kind: str | None = None) -> None:
     if code == 0:
         if _PROFILE is not None:
-            _mark(kind or _KIND.get(kernel, "other"))
+            kind = kind or _KIND.get(kernel, "other")
+            _mark(kind, kernel + (" (experts)" if kind == "moe" and kernel.startswith("gemm") else ""))
         return
     if code == -1:
         raise KernelError(f"{kernel}: arguments rejected by the launcher")

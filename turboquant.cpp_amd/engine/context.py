@@ -17,6 +17,9 @@ class StepContext:
     device: torch.device
     side_stream: "torch.cuda.Stream | None" = None   # a second stream for work that does not depend on the main line
     capturing: bool = False      # the step is being recorded for replay: what the host pays now it pays once
+    # called with (schedule entry, the residual stream behind that entry [T, H] float32, the batch), for whoever wants
+    # to look at activations layer by layer (the reference prints them under TQ_DEBUG, tq_transformer.c:2340-2344)
+    layer_hook: "object | None" = None
 
     def kv(self, entry: int) -> KVView:
         """Keys and values of the schedule entry (or of the entry whose cache it reads)."""

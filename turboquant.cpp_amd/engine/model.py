@@ -116,6 +116,9 @@ class CausalLM:
         pending = None
         for entry, e in enumerate(self.schedule):
             pending = self.blocks[e.layer].forward(x, pending, ctx, entry)
+            if ctx.layer_hook is not None:      # the stream with what the entry has left for the next norm to add
+                held = pending.materialize(self.act) if isinstance(pending, ops.GatheredSum) else pending
+                ctx.layer_hook(entry, x.clone() if held is None else x + held.sum(0), b)
         if b.n_want == 0:
             return torch.empty((0, self.plan.vocab_size), dtype=torch.float32, device=x.device)
         normed, _ = self.final_norm.forward(x, pending, ctx, rows=b.want_rows)

@@ -39,6 +39,7 @@ class Engine:
         self.side_stream = torch.cuda.Stream(device=self.device) if on_gpu else None     # default priority
         # (which shapes of step are replayed is the parts' word, asked shape by shape: Part.replayable)
         self.graphs = DecodeGraphs(self) if use_graphs and on_gpu else None
+        self.layer_hook = None      # see StepContext.layer_hook; while it is set, steps run eagerly
 
     # ------------------------------------------------------------ sequences
     def open(self, n: int = 1) -> list[int]:
@@ -88,7 +89,7 @@ class Engine:
         starts = self._reserve(slots, [len(t) for t in token_lists])
         try:
             logits = None
-            if self.graphs is not None and all(len(t) == 1 for t in token_lists):
+            if self.graphs is not None and self.layer_hook is None and all(len(t) == 1 for t in token_lists):
                 all_rows = self.graphs.run(slots, starts, [t[0] for t in token_lists])
                 if all_rows is not None:       # the graph gives every row; hand out a copy of the wanted ones
                     rows = [i for i, w in enumerate(wants) for _ in w]
@@ -117,7 +118,7 @@ class Engine:
             raise StepError(f"tokens must be int32 [{len(slots)}] on the model's device")
         starts = self._reserve(slots, [1] * len(slots))
         try:
-            logits = self.graphs.run(slots, starts, tokens) if self.graphs is not None else None
+            logits = self.graphs.run(slots, starts, tokens) if self.graphs is not None and self.layer_hook is None else None
             if logits is None:
                 batch = pack_step(slots, starts, [[0]] * len(slots), [[0]] * len(slots), self.device)
                 batch.tokens.copy_(tokens)
@@ -151,6 +152,6 @@ class Engine:
     def _eager(self, batch) -> torch.Tensor:
         # a second stream for what does not depend on the main line (the parts decide what they put there)
         ctx = StepContext(batch=batch, cache=self.cache, act=self.model.act, device=self.device,
-                          side_stream=self.side_stream)
+                          side_stream=self.side_stream, layer_hook=self.layer_hook)
         with ops.own_products(max(batch.n_new) == 1):      # a decode step runs the kernels that its replay runs
             return self.model.forward(ctx)
