@@ -465,6 +465,14 @@ def test_a_conversation_keeps_its_cache_between_turns(name, sharp, tmp_path):
         assert brought[0] == (len(h3) - 40 if name == "A" else len(h3)), brought
         del brought[:]
         assert m.chat(h3) == out3 and brought[0] == 1  # the same history again: only its last token is run
+        # saved where a window has let the first pages go (B keeps 24 positions in one group), loaded, gone on with
+        far_file = str(tmp_path / "far.kv")
+        m.save_context(far_file)
+        with Model(d, **opts) as far:
+            far.load_context(far_file)
+            assert far.chat_tokens == (h3 + out3)[:len(far.chat_tokens)] and len(far.chat_tokens) >= len(h3)
+            h5 = h3 + out3 + more
+            assert far.chat(h5) == fresh.generate([h5])[0]
         with pytest.raises(ChatContextOverflow):
             m.chat(list(range(3)) * 200)
         assert m.chat(None) == [] and m._chat_slot is None
