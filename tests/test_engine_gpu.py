@@ -714,6 +714,24 @@ def test_a_mixer_with_state_of_its_own_is_registered_built_and_stepped():
                 b_ = slow.step([ss[i] for i in order], [[prompts[i][t]] for i in order])
                 assert torch.equal(a, b_), f"replayed step {t} differs from the eager one"
             eng.close(sf), slow.close(ss)
+        # a sequence that leaves the cache and comes back (its rows of state with it) goes on as if it had stayed;
+        # it cannot go back to an earlier position, having no earlier state
+        from turboquant_cpp_amd.cache.paged import CacheError
+        (a,) = eng.open(1)
+        eng.step([a], [prompts[2][:12]], [[]])
+        saved = eng.cache.export_slot(a)
+        assert saved["length"] == 12 and sorted(saved["states"]) == [0, 1] and saved["groups"] == []
+        with pytest.raises(CacheError, match="state"):
+            eng.cache.truncate(a, 5)
+        eng.close([a])
+        (other,) = eng.open(1)                                    # takes the slot and leaves its own state there
+        eng.step([other], [prompts[0]], [[]])
+        eng.close([other])
+        b_ = eng.cache.import_slot(saved)
+        assert eng.length(b_) == 12
+        lg = eng.step([b_], [prompts[2][12:]], [list(range(8))]).cpu().double()
+        assert (lg - refs[2][12:]).abs().max() < 1e-4
+        eng.close([b_])
     finally:
         unregister_part("mixer", "toy_decay")
 

@@ -82,6 +82,9 @@ class Model:
 
     def generate_detailed(self, prompts, **overrides) -> list[GenerationResult]:
         self._ensure_open()
+        if self._chat_slot is not None and self._engine.cache.n_free_slots == 0:
+            raise RuntimeError("the conversation holds the model's only slot: reset_chat() first, or open the model "
+                               "with max_batch > 1")
         opts = GenerationOptions(**{**self.options.__dict__, **overrides})
         return generate(self._engine, [list(p) for p in prompts], opts)
 
