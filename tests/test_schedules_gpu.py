@@ -317,7 +317,7 @@ def test_the_command_line_says_where_the_time_goes(sharp):
     put down to products, experts, attention and the rest."""
     d, _, _ = sharp("B", "bfloat16")
     run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "quant"), d, "-p", "5,17,3,9;8,1", "-n", "3", "-T", "0",
-                          "--profile"], capture_output=True, text=True, timeout=300)
+                          "--profile", "-M"], capture_output=True, text=True, timeout=300)
     assert run.returncode == 0, run.stderr[-2000:]
     lines = [l for l in run.stderr.splitlines() if l.startswith("PROFILE_CSV:")]
     assert [l.split(":")[1].split(",")[0] for l in lines] == ["prompt", "decode"]
@@ -327,6 +327,11 @@ def test_the_command_line_says_where_the_time_goes(sharp):
         assert int(f[1]) == n_tok and total > 0 and all(v > 0 for v in parts) and abs(sum(parts) - total) < 1e-2 * total
     assert "[Profile prompt, 6 tok] matmul=" in run.stderr and "[Profile decode, 32 tok] matmul=" in run.stderr
     assert "add_rmsnorm" in run.stderr and "(experts)" in run.stderr and " launches " in run.stderr
+    # -M: B keeps keys and values of 2 kv heads of 24 in 3 layers, in bfloat16: 2 * 3 * 2 * 24 * 2 bytes a token
+    mem = [l for l in run.stderr.splitlines() if l.startswith("MEMORY_CSV:")][0].split(":")[1].split(",")
+    n_tok = int(mem[0])
+    assert 6 < n_tok <= 12 and int(mem[1]) == n_tok * 2 * 3 * 2 * 24 * 2 == int(mem[2]) and float(mem[3]) == 1.0
+    assert "=== KV Cache Memory Stats ===" in run.stderr
 
 
 def test_the_replay_tool_shows_the_stream_behind_every_layer(sharp, tmp_path):

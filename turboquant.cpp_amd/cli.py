@@ -1,6 +1,7 @@
 """Command line in the manner of the reference's ``quant <model> [options]`` (/root/reference/tools/quant.c:126-163,
 defaults :196-239): the model path first, then ``-p`` prompt, ``-n`` max tokens (256), ``-T`` temperature (0.7),
-``-P`` top-p (0.9), ``-s`` seed (42), ``--ctx`` context length, ``--info``, ``--profile``, ``--version``.  There is no
+``-P`` top-p (0.9), ``-s`` seed (42), ``--ctx`` context length, ``--info``, ``--profile``, ``-M`` (the cache's memory per
+token, :1382-1461), ``--version``.  There is no
 tokenizer in this library, so a prompt is a list of token ids (``-p "5,17,3"``; several prompts are separated by
 ``;`` and run as one batch), or ``--random-prompt LEN[,LEN...]`` draws them.  ``--random-weights CONFIG.json --save
 DIR`` is the random-weights mode: it writes a model folder for a configuration and a seed and exits.  ``--ppl FILE``
@@ -56,6 +57,7 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--random-prompt", default=None, metavar="LEN[,LEN...]", help="prompts of random token ids of these lengths")
     ap.add_argument("--max-batch", type=int, default=8, help="sequences that generate together")
     ap.add_argument("--info", action="store_true", help="print model info and exit")
+    ap.add_argument("-M", "--memory", action="store_true", help="print what the cache holds per token after the generation")
     ap.add_argument("--profile", action="store_true", help="time the prompt step and the decode steps")
     ap.add_argument("--json", action="store_true", help="print results as JSON")
     ap.add_argument("--version", action="store_true")
@@ -175,6 +177,34 @@ def main(argv=None) -> int:
     if n_generated > 0 and elapsed > 0:
         print(f"{n_generated} tokens in {elapsed:.1f}s ({n_generated / elapsed:.1f} tok/s, {len(prompts)} sequences, "
               f"weights={args.dtype}, kv={args.dtype})", file=sys.stderr)
+    if args.memory and n_generated > 0:
+        # the reference's report (/root/reference/tools/quant.c:1382-1461), for a cache that is not compressed: what a
+        # token costs in every layer that keeps keys and values, against keys and values in 16-bit floats
+        cache = model.engine.cache
+        esz = 4 if args.dtype == "float32" else 2
+        n_tok = sum(len(p) + len(r.tokens) for p, r in zip(prompts, results))
+        k_per = sum(len(g.entries) * g.key.num_kv_heads * g.key.head_dim * esz for g in cache.groups)
+        v_per = sum(len(g.entries) * g.key.num_kv_heads * g.key.value_dim * esz for g in cache.groups)
+        f16_per = (k_per + v_per) // esz * 2
+        total, total16 = (k_per + v_per) * n_tok, f16_per * n_tok
+        ratio = total16 / total if total else 0.0
+        print("\n=== KV Cache Memory Stats ===", file=sys.stderr)
+        print(f"Tokens in cache:      {n_tok}", file=sys.stderr)
+        print("Model config:         " + "; ".join(
+            f"{len(g.entries)} layers, {g.key.num_kv_heads} kv_heads, head_dim={g.key.head_dim}"
+            + (f", window={g.key.window}" if g.key.window else "") for g in cache.groups), file=sys.stderr)
+        print(f"KV type:              {args.dtype}", file=sys.stderr)
+        print(f"Per-token K ({args.dtype}): {k_per / 1024:.2f} KB", file=sys.stderr)
+        print(f"Per-token V ({args.dtype}): {v_per / 1024:.2f} KB", file=sys.stderr)
+        print(f"Per-token K+V total:  {(k_per + v_per) / 1024:.2f} KB", file=sys.stderr)
+        print(f"Per-token K+V (FP16): {f16_per / 1024:.2f} KB", file=sys.stderr)
+        print(f"Total K+V:            {total / 1024 / 1024:.2f} MB", file=sys.stderr)
+        print(f"Total K+V (FP16):     {total16 / 1024 / 1024:.2f} MB", file=sys.stderr)
+        print(f"Compression ratio:    {ratio:.2f}x (K+V combined)", file=sys.stderr)
+        print(f"Weights:              {model._model.weight_bytes / 1024 / 1024:.2f} MB; cache pool: {cache.bytes() / 1024 / 1024:.2f} MB",
+              file=sys.stderr)
+        print("=============================", file=sys.stderr)
+        print(f"MEMORY_CSV:{n_tok},{total},{total16},{ratio:.4f}", file=sys.stderr)
     if args.profile:
         # Where the time of a forward pass goes, by kind of work, in the reference's line
         # (/root/reference/src/engine/tq_transformer.c:2995-3020): steps run eagerly on one stream, an event behind
