@@ -332,6 +332,14 @@ def test_the_command_line_says_where_the_time_goes(sharp):
     n_tok = int(mem[0])
     assert 6 < n_tok <= 12 and int(mem[1]) == n_tok * 2 * 3 * 2 * 24 * 2 == int(mem[2]) and float(mem[3]) == 1.0
     assert "=== KV Cache Memory Stats ===" in run.stderr
+    # the reference's two small benchmarks: decode speed behind five contexts, and a prompt of 200 tokens
+    bench = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "quant"), d, "--bench-memory", "--bench-prefill", "--ctx", "1024"],
+                           capture_output=True, text=True, timeout=300)
+    assert bench.returncode == 0, bench.stderr[-2000:]
+    rows = [l.split(":")[1].split(",") for l in bench.stderr.splitlines() if l.startswith("BENCH_CSV:")]
+    assert [int(r[0]) for r in rows] == [10, 50, 100, 200, 500] and all(float(r[1]) > 0 for r in rows)
+    (pre,) = [l.split(":")[1].split(",") for l in bench.stderr.splitlines() if l.startswith("PREFILL_CSV:")]
+    assert pre[0] == "bfloat16 (no quant)" and int(pre[1]) == 200 and float(pre[2]) > 0
 
 
 def test_the_replay_tool_shows_the_stream_behind_every_layer(sharp, tmp_path):

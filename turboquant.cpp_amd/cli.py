@@ -1,7 +1,7 @@
 """Command line in the manner of the reference's ``quant <model> [options]`` (/root/reference/tools/quant.c:126-163,
 defaults :196-239): the model path first, then ``-p`` prompt, ``-n`` max tokens (256), ``-T`` temperature (0.7),
 ``-P`` top-p (0.9), ``-s`` seed (42), ``--ctx`` context length, ``--info``, ``--profile``, ``-M`` (the cache's memory per
-token, :1382-1461), ``--version``.  There is no
+token, :1382-1461), ``--bench-memory`` and ``--bench-prefill`` (:726-860), ``--version``.  There is no
 tokenizer in this library, so a prompt is a list of token ids (``-p "5,17,3"``; several prompts are separated by
 ``;`` and run as one batch), or ``--random-prompt LEN[,LEN...]`` draws them.  ``--random-weights CONFIG.json --save
 DIR`` is the random-weights mode: it writes a model folder for a configuration and a seed and exits.  ``--ppl FILE``
@@ -57,6 +57,9 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--random-prompt", default=None, metavar="LEN[,LEN...]", help="prompts of random token ids of these lengths")
     ap.add_argument("--max-batch", type=int, default=8, help="sequences that generate together")
     ap.add_argument("--info", action="store_true", help="print model info and exit")
+    ap.add_argument("--bench-memory", action="store_true",
+                    help="decode speed behind contexts of 10 to 500 tokens (BENCH_CSV lines) and exit")
+    ap.add_argument("--bench-prefill", action="store_true", help="speed of a prompt of 200 tokens (a PREFILL_CSV line) and exit")
     ap.add_argument("-M", "--memory", action="store_true", help="print what the cache holds per token after the generation")
     ap.add_argument("--profile", action="store_true", help="time the prompt step and the decode steps")
     ap.add_argument("--json", action="store_true", help="print results as JSON")
@@ -103,6 +106,53 @@ def main(argv=None) -> int:
                   context_length=args.ctx, dtype=args.dtype, seed=args.seed, rep_penalty=args.rep_penalty,
                   max_batch=args.max_batch, stop_tokens=args.stop_id)
     print(f"loaded {args.model} in {time.time() - t0:.1f}s ({args.dtype}, context {model.context_length})", file=sys.stderr)
+    if args.bench_memory or args.bench_prefill:
+        # the reference's two small benchmarks (/root/reference/tools/quant.c:726-800, :804-860): one token, its token
+        # 1, repeated as the context
+        eng = model.engine
+        tok = min(1, eng.vocab_size - 1)
+        if args.bench_memory:
+            print("\n=== Memory Bandwidth Benchmark ===", file=sys.stderr)
+            print(f"KV type: {args.dtype}", file=sys.stderr)
+            print(f"{'Context':<12} {'Tok/s':<12} {'Time(s)':<12}", file=sys.stderr)
+            print("-------- -------- --------", file=sys.stderr)
+            for ctx in (10, 50, 100, 200, 500):
+                n_gen = min(20, model.context_length - ctx - 1)
+                if ctx >= model.context_length or n_gen < 1:
+                    continue
+                for timed in (False, True):          # the first pass loads kernels and captures the decode step
+                    slot = eng.open(1)
+                    eng.step(slot, [[tok] * ctx], [[]])
+                    torch.cuda.synchronize()
+                    t1 = time.time()
+                    for _ in range(n_gen):
+                        eng.step(slot, [[tok]])
+                    torch.cuda.synchronize()
+                    elapsed = time.time() - t1
+                    eng.close(slot)
+                print(f"{ctx:<12d} {n_gen / elapsed:<12.1f} {elapsed:<12.3f}", file=sys.stderr)
+                print(f"BENCH_CSV:{ctx},{n_gen / elapsed:.2f},{elapsed:.4f}", file=sys.stderr)
+            print("==================================", file=sys.stderr)
+        if args.bench_prefill:
+            n = min(200, model.context_length - 1)
+            print("\n=== Prefill Speed Benchmark ===", file=sys.stderr)
+            print(f"Prefill length: {n} tokens", file=sys.stderr)
+            print(f"{'KV Config':<28} {'Tok/s':<12} {'Time(s)':<12}", file=sys.stderr)
+            print("---------------------------- ------------ ------------", file=sys.stderr)
+            for timed in (False, True):
+                slot = eng.open(1)
+                torch.cuda.synchronize()
+                t1 = time.time()
+                eng.step(slot, [[tok] * n])
+                torch.cuda.synchronize()
+                elapsed = time.time() - t1
+                eng.close(slot)
+            name = f"{args.dtype} (no quant)"
+            print(f"{name:<28} {n / elapsed:<12.1f} {elapsed:<12.3f}", file=sys.stderr)
+            print(f"PREFILL_CSV:{name},{n},{n / elapsed:.2f},{elapsed:.4f}", file=sys.stderr)
+            print("===============================", file=sys.stderr)
+        model.close()
+        return 0
     if args.ppl:
         with open(args.ppl) as f:
             ids = [int(t) for t in f.read().replace(",", " ").split()]
