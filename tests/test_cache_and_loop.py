@@ -389,6 +389,43 @@ def test_generate_with_the_default_options_matches_the_plain_loop(cpu_engine, mo
     assert "loop" in reasons
 
 
+def test_a_sequence_that_outlives_its_request(cpu_engine):
+    """``continue_in_slot``: the slot's cache holds the beginning of a history, the rest is run as one prompt step and
+    a continuation is generated; what comes out is what ``generate`` gives for the whole history, turn after turn,
+    and the cache then holds all but a token that ended the turn by its number.  A cache that runs full ends the turn
+    with reason "context" and keeps what it holds."""
+    from turboquant_cpp_amd.engine.generate import continue_in_slot
+    eng = cpu_engine("A", max_tokens=64 * 6, max_slots=2)
+    greedy = dict(temperature=0.0, rep_penalty=1.0, loop_detection=False)
+    (slot,) = eng.open(1)
+    history = [3, 9, 4, 1, 7]
+    brought = []
+    step = eng.step
+    eng.step = lambda slots, toks, *a, **k: (brought.append(len(toks[0])), step(slots, toks, *a, **k))[1]
+    for turn, more in enumerate(([], [8, 8, 2], [5])):
+        history = history + more
+        before = eng.length(slot)
+        del brought[:]
+        res = continue_in_slot(eng, slot, history, GenerationOptions(max_tokens=4, **greedy))
+        assert brought[0] == len(history) - before and brought[1:] == [1] * 3
+        eng.step = step
+        want = generate(eng, [history], GenerationOptions(max_tokens=4, **greedy))[0]
+        eng.step = lambda slots, toks, *a, **k: (brought.append(len(toks[0])), step(slots, toks, *a, **k))[1]
+        assert res.tokens == want.tokens and res.finish_reason == "length"
+        assert eng.length(slot) == len(history) + 3            # the fourth token ended the turn and was never run
+        history = history + res.tokens
+    with pytest.raises(ValueError, match="at least one"):
+        continue_in_slot(eng, slot, history[:eng.length(slot)], GenerationOptions(max_tokens=4, **greedy))
+    assert continue_in_slot(eng, slot, history, GenerationOptions(max_tokens=0, **greedy)).finish_reason == "length"
+    eng.step = step
+    eng.close([slot])
+    small = cpu_engine("A", max_tokens=64, max_slots=1)
+    (slot,) = small.open(1)
+    res = continue_in_slot(small, slot, [3] * 60, GenerationOptions(max_tokens=12, **greedy))
+    assert res.finish_reason == "context" and len(res.tokens) == 4 and small.length(slot) == 63
+    small.close([slot])
+
+
 def test_a_sequence_goes_back_to_an_earlier_position():
     """``truncate`` forgets the positions from a point on and gives their pages back; it refuses where a window has
     dropped pages that the earlier position would look at, and where the model keeps fixed-size state."""
