@@ -107,10 +107,14 @@ def test_gemm_dense(ops, act, M, N, K, mode, monkeypatch):
 
 @pytest.mark.parametrize("M,N,K", [(512, 130, 264), (700, 6144, 2048), (2048, 257, 1000), (8192, 96, 16384), (600, 96, 16384)])
 def test_plain_products_of_many_rows(ops, M, N, K, monkeypatch):
-    """From 512 rows on a plain bfloat16 product without bias goes to the vendor's library unless k is long and the
-    rows are not many; its result and the own kernel's are the same product in another order of sums.  Gated
-    products, products with a bias and the 32-bit path stay; TQ_PLAIN_PRODUCTS=own (read at import) keeps all."""
+    """From VENDOR_MIN_ROWS rows on (512 here, to keep the sizes small) a plain bfloat16 product without bias goes to
+    the vendor's library unless k is long and the rows are not many; its result and the own kernel's are the same
+    product in another order of sums.  Gated products, products with a bias and the 32-bit path stay;
+    TQ_PLAIN_PRODUCTS=own (read at import) keeps all."""
     act = "bfloat16"
+    below = rnd((ops.VENDOR_MIN_ROWS - 1, K), adt(act), 13).to(DEV)
+    assert not ops._vendor_product(act, below, below, ops.VENDOR_MIN_ROWS - 1, K)       # the border as it ships
+    monkeypatch.setattr(ops, "VENDOR_MIN_ROWS", 512)
     a, w = rnd((M, K), adt(act), 14).to(DEV), rnd((N, K), adt(act), 15, 0.2).to(DEV)
     calls = []
     real = torch.mm
@@ -152,10 +156,11 @@ def test_the_gate_applied_afterwards(ops, act, activation, M, N, ld):
 @pytest.mark.parametrize("activation", ["silu", "gelu_tanh"])
 @pytest.mark.parametrize("M,N,K", [(512, 130, 264), (5000, 96, 72), (700, 1408, 2048)])
 def test_gated_pairs_of_many_rows(ops, activation, M, N, K, monkeypatch):
-    """A gated pair whose second matrix lies right behind the first goes, from 512 rows on, to the vendor's library
-    as one product over both, a few thousand rows at a time, with the gate in a pass of its own; matrices that lie
-    apart stay in this library's kernel.  Both are the same function."""
+    """A gated pair whose second matrix lies right behind the first goes, from VENDOR_MIN_ROWS rows on (512 here), to
+    the vendor's library as one product over both, a few thousand rows at a time, with the gate in a pass of its
+    own; matrices that lie apart stay in this library's kernel.  Both are the same function."""
     act = "bfloat16"
+    monkeypatch.setattr(ops, "VENDOR_MIN_ROWS", 512)
     a = rnd((M, K), adt(act), 17).to(DEV)
     w, w2 = rnd((N, K), adt(act), 18, 0.2).to(DEV), rnd((N, K), adt(act), 19, 0.2).to(DEV)
     g, u = ops.side_by_side(w, w2)
@@ -197,6 +202,13 @@ def test_gemm_partial_sums(ops, act, M, N, K, bias):
                 runs *= 2
         else:
             runs = 1 if K < 2048 else (2 if K < 4096 else 4)
+            if M <= 1024:   # tiles of 64 rows: up to 8 runs of at least 256 while the workgroups are few and the sums small
+                tiles, t = -(-M // 64) * -(-N // 128), 1
+                while t < 8 and tiles * t * 2 <= 512 and K // (t * 2) >= 256 and t * 2 * M * N * 4 <= 8 << 20:
+                    t *= 2
+                runs = max(runs, t)
+                while runs > 1 and (runs - 1) * (-(-(-(-K // 64)) // runs) * 64) >= K:    # no run begins past the end
+                    runs //= 2
         assert y.shape[0] == runs
     ref = ref_gemm(a, w, b, None)
     scale = ref.abs().max().item()
@@ -590,6 +602,7 @@ def test_queries_keys_values_of_a_long_prompt(ops, T, monkeypatch):
     queries and pages are those of this library's own product with the bias in it, up to the order of sums."""
     from plain_qwen2moe import rope_frequencies
     act, nh, nkv, hd, H, page = "bfloat16", 6, 2, 64, 264, 64
+    monkeypatch.setattr(ops, "VENDOR_MIN_ROWS", 512)
     table, slots, page_stride, kp, vp = paged_setup([T], page, nkv, hd, 1, act, 174)
     a = rnd((T, H), adt(act), 175).to(DEV)
     w = rnd(((nh + 2 * nkv) * hd, H), adt(act), 176, 0.2).to(DEV)

@@ -84,9 +84,11 @@ def test_decode_steps_of_many_sequences(name, n_seqs, act, sharp, monkeypatch):
     """More than 16 sequences decode together: the feed-forward leaves the launches it uses for a handful of tokens
     and puts the shared expert on a second stream, which a captured graph records as a fork and a join.  Replays
     are compared with eager steps bit for bit, and both with the plain model.  With 530 sequences a decode step has
-    the rows at which a prompt step hands its plain products to the vendor's library: a decode step does not, eager
-    or captured."""
+    the rows at which a prompt step hands its plain products to the vendor's library (from 512 rows on here): a
+    decode step does not, eager or captured."""
+    from turboquant_cpp_amd.csrc import ops
     from turboquant_cpp_amd.engine.step import Engine
+    monkeypatch.setattr(ops, "VENDOR_MIN_ROWS", 512)
     d, plain, model = sharp(name, act)
     calls = []
     real = torch.mm
@@ -253,13 +255,15 @@ def test_a_long_prompt_takes_the_taller_expert_tiles(sharp, monkeypatch):
 # ------------------------------------------------------------------------------------------------ whose product it is
 @pytest.mark.parametrize("name", ["B", "C"])
 def test_a_long_prompt_whole_cut_and_with_every_product_in_own_kernels(name, sharp, monkeypatch):
-    """A bfloat16 prompt step of 512 tokens and more hands its plain products (q, k, v without their bias; o; the
+    """A bfloat16 prompt step of VENDOR_MIN_ROWS tokens and more (512 here, so that the prompt can stay short) hands
+    its plain products (q, k, v without their bias; o; the
     dense and the shared gated pairs and their down products) to the vendor's matrix library.  A prompt of 700
     tokens taken whole that way, whole with every product in this library's kernels, and cut into steps of 250 that
     never reach the library: all three against the plain model at every position."""
     from turboquant_cpp_amd.csrc import ops
     from turboquant_cpp_amd.engine.step import Engine
     d, plain, model = sharp(name, "bfloat16")
+    monkeypatch.setattr(ops, "VENDOR_MIN_ROWS", 512)
     (prompt,) = prompts_for(name, [700], seed=33)
     calls = []
     real = torch.mm

@@ -612,6 +612,18 @@ static int plain_tile_choice(int M, int N, int splits) {
   return best;
 }
 
+// Whether a gated pair of a few hundred rows with one matrix goes in tiles of 64 rows rather than 128.  With so few
+// rows a workgroup's time is its steps over k, 1.0 us a step in the lower tile against 1.35 in the taller, as long as
+// it has its compute unit to itself; of the lower tiles two fit on a compute unit (80 KB of LDS each), of the
+// taller one.  So: the lower tile where it needs no more than one workgroup to a compute unit, or where the
+// taller one would need a second round and the lower fits in one (320 rows by 2 x 5,632 x 2,048: 34 us against
+// 46; 384 rows: 47 against 46; 192 rows by 2 x 20,480 x 3,584: 103 against 149; 128 rows: 110 against 92).
+static bool gated_pair_in_tiles_of_64(int M, int N) {
+  const int64_t cols = (N + TBN - 1) / TBN;
+  const int64_t lower = (int64_t)((M + 63) / 64) * cols, taller = (int64_t)((M + 127) / 128) * cols;
+  return lower <= 256 || (taller > 256 && lower <= 512);
+}
+
 // Into how many runs of k a plain product of M rows may be split when its partial sums are wanted apart.  Many
 // rows: a product whose tiles do not fill the chip twice, and that has k enough, goes faster in 2 to 4 runs, each
 // at least 1024 long.  17 to 64 rows of a narrow matrix with a long k (the streaming kernel with at most 8 waves
@@ -629,6 +641,18 @@ TQ_API int tq_gemm_mfma_splits(int M, int N, int K) {
   const int64_t tiles = (int64_t)((M + 127) / 128) * ((N + TBN - 1) / TBN);
   int s = 1;
   while (s < 4 && tiles * s < 512 && K / (s * 2) >= 1024) s *= 2;
+  if (M <= 64 * 16) {
+    // Up to 1,024 rows go in tiles of 64 rows, and a workgroup's time is its steps over k (about 0.6 us each,
+    // whatever the memory does): up to 8 runs, each at least 256 long, while the workgroups stay within two to a
+    // compute unit and the partial sums within 8 MB, which the kernel behind has to read (128 rows by
+    // 2,048 x 2,048: 8.7 us in eight runs against 14.6 in two; by 2,048 x 5,632: 13.7 against 19.3 in four).
+    const int64_t tiles64 = (int64_t)((M + 63) / 64) * ((N + TBN - 1) / TBN);
+    int t = 1;
+    while (t < 8 && tiles64 * t * 2 <= 512 && K / (t * 2) >= 256 && (int64_t)t * 2 * M * N * 4 <= (8 << 20)) t *= 2;
+    if (t > s) s = t;
+    // every run must begin before the end of k (runs are whole tiles of 64)
+    while (s > 1 && (int64_t)(s - 1) * (((K + TBK - 1) / TBK + s - 1) / s * TBK) >= K) s /= 2;
+  }
   return s;
 }
 
@@ -648,6 +672,7 @@ TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gat
   if (splits < 1 || splits > 64 || gate < 0 || gate >= TQ_GATE_COUNT) return TQ_ERR_BAD_ARG;
   if (splits > 1 && (dual || out_act || tile_group || a_rows || splits != tq_gemm_mfma_splits(M, N, K))) return TQ_ERR_BAD_ARG;
   const int k_per = ((K + TBK - 1) / TBK + splits - 1) / splits * TBK;
+  if (splits > 1 && (int64_t)(splits - 1) * k_per >= K) return TQ_ERR_BAD_ARG;
   MfmaGemmArgs g{(const bf16_t*)a, lda, a_rows, a_gather, (const bf16_t*)w, (const bf16_t*)w2, group_stride,
                  tile_group, n_tiles, bias, bias_type, out, ldc, M, N, K, splits > 1 ? k_per : K, (int64_t)M * ldc, gate, 1};
   int rc = 0;
@@ -694,6 +719,8 @@ TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gat
   } else {
     if ((N + TBN - 1) / TBN > 65535) return TQ_ERR_UNSUPPORTED;
     if (M <= 64 * 16 && !dual)
+      rc = launch_tile<64, 2, 4>(g, dual, out_act, splits, st);
+    else if (dual && gated_pair_in_tiles_of_64(M, N))
       rc = launch_tile<64, 2, 4>(g, dual, out_act, splits, st);
     else if (dual)
       rc = launch_tile<128, 4, 2>(g, dual, out_act, splits, st);

@@ -506,7 +506,7 @@ def _gemm_problem(k: str, a, w, act, bias, w2, out_act, a_rows, tile_group, n_ti
 # TQ_PLAIN_PRODUCTS=own keeps every product in this library's kernels.  Products over experts, gated pairs whose
 # matrices lie apart, products with a bias that nothing behind them can add, products of few rows, decode steps,
 # steps under graph capture and the 32-bit path never leave them.
-VENDOR_MIN_ROWS = 512
+VENDOR_MIN_ROWS = 768
 _VENDOR = os.environ.get("TQ_PLAIN_PRODUCTS", "vendor") != "own"
 
 
