@@ -502,7 +502,9 @@ def _gemm_problem(k: str, a, w, act, bias, w2, out_act, a_rows, tile_group, n_ti
 # reference's engine hands its plain products to a BLAS where it has one
 # (/root/reference/src/engine/tq_ops.c:296-305): measured on gfx950 it is 25 to 35 % faster than the tile kernel here
 # from 512 rows on ([2048, 2048] x [6144, 2048]: 48 against 63 us; 13,199 rows: 282 against 401), slower or equal
-# below and where k is long and the rows are not many ([4096, 20480] x [3584, 20480]: 724 against 687 us).
+# below and where k is long and the rows are not many ([4096, 20480] x [3584, 20480]: 724 against 687 us).  A call
+# into the library costs the host twice what a launch here costs, and a step of 512 to 767 rows is as long on the
+# host as on the chip (24 layers of 512 tokens: 9.7 ms through the library, 7.9 without), so it starts at 768 rows.
 # TQ_PLAIN_PRODUCTS=own keeps every product in this library's kernels.  Products over experts, gated pairs whose
 # matrices lie apart, products with a bias that nothing behind them can add, products of few rows, decode steps,
 # steps under graph capture and the 32-bit path never leave them.
