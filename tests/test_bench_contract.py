@@ -73,3 +73,16 @@ def test_the_line_of_a_short_run_on_the_gpu():
     assert abs(roof["achieved"] - detail["gb_per_step"] / (line["ms_per_step"] * 1e-3)) < 0.01 * roof["achieved"]
     pre = line["prefill"]
     assert pre["tokens"] == 2048 and abs(pre["value"] - 2048 / (pre["ms"] * 1e-3)) < 0.01 * pre["value"] and 0 < pre["frac"] < 1
+
+
+@pytest.mark.gpu
+def test_a_prompt_of_another_length_for_profiles():
+    """--prefill-only --prefill-tokens N times a prompt step of N tokens alone and says how long the host was busy
+    launching it (the default, and the contract's line, is 2,048 tokens)."""
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--layers", "1", "--prefill-only", "--prefill-tokens", "300"],
+                       capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    line = json.loads(r.stdout.strip().splitlines()[-1])
+    assert "300 tokens" in line["metric"] and line["layers"] == 1 and line["dtype"] == "bf16"
+    assert abs(line["value"] - 300 / (line["ms"] * 1e-3)) < 0.01 * line["value"]
+    assert 0 < line["host_ms"] <= line["ms"] * 1.01 and 0 < line["frac"] < 1
