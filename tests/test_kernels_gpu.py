@@ -182,6 +182,18 @@ def test_gated_pairs_of_many_rows(ops, activation, M, N, K, monkeypatch):
     assert len(calls) == -(-M // 2048)
 
 
+@pytest.mark.parametrize("M,N", [(320, 5632), (384, 5632), (128, 20480), (192, 20480), (260, 20480)])
+def test_a_gated_pair_of_a_few_hundred_rows_in_either_tile(ops, M, N):
+    """A gated pair with one matrix takes tiles of 64 rows where its workgroups need no more than a compute unit each
+    (or where the taller tile would need a second round and the lower fits in one), else tiles of 128: the sizes here
+    lie on both sides of both borders, and every one is the same function."""
+    act, K = "bfloat16", 136
+    a, w, w2 = rnd((M, K), adt(act), 31), rnd((N, K), adt(act), 32, 0.2), rnd((N, K), adt(act), 33, 0.2)
+    y = ops.gemm(a.to(DEV), w.to(DEV), act, w2=w2.to(DEV), out_act=True).cpu().double()
+    ref = ref_gemm(a, w, None, w2)
+    assert (y - ref).abs().max().item() < 2e-2 * ref.abs().max().item()
+
+
 @pytest.mark.parametrize("act", ACTS)
 @pytest.mark.parametrize("M,N,K,bias", [(300, 200, 2200, True), (129, 130, 4104, False), (70, 64, 1000, False), (9, 40, 4096, True),
                                         (40, 264, 8200, True), (64, 2048, 5632, False), (17, 72, 4096, False)])
