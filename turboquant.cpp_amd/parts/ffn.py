@@ -17,6 +17,9 @@ from ..csrc import ops
 from .base import ParamSpec, Part, register_part
 
 
+SIDE_STREAM_FROM = 320      # tokens of an eager step from which the shared expert goes to a second stream
+
+
 @register_part("ffn", "dense_swiglu")
 class DenseSwiGLU(Part):
     graph_safe = True
@@ -99,11 +102,12 @@ class SparseMoE(Part):
         shared, side = None, None
         if self.shared_size > 0:
             tiles = -(-T // 128) * -(-self.shared_size // 128)
-            # Up to 64 tokens the host's part of forking and joining (1.7 ms of a step of 24 layers) is more than the
-            # second stream gains: a prompt step of 17 tokens took 6.0 ms with it and 4.2 without, one of 128 tokens 6.7
-            # and 7.5.  A step that is being captured pays the host once and is replayed with the two streams (64
-            # sequences: 10.8 ms a step with them, 11.15 without).
-            worth = T > 64 or getattr(ctx, "capturing", False)
+            # Below some 300 tokens the host's part of forking and joining (2.6 ms of a step of 24 layers, which is
+            # then as long on the host as on the chip) is more than the second stream gains: a prompt step of 65 tokens
+            # took 6.8 ms with it and 5.4 without, one of 200 tokens 6.8 and 6.3, of 320 tokens 7.15 and 7.2, of 512
+            # tokens 7.9 and 8.8.  A step that is being captured pays the host once and is replayed with the two
+            # streams (64 sequences: 10.8 ms a step with them, 11.15 without).
+            worth = T >= SIDE_STREAM_FROM or getattr(ctx, "capturing", False)
             side = ctx.fork() if hasattr(ctx, "fork") and worth and tiles < 8 * 256 else None
             if side is not None:
                 with torch.cuda.stream(side):
