@@ -191,7 +191,9 @@ TQ_API int tq_add_rmsnorm(float* x, const float* delta, int S, int64_t delta_str
                           hipStream_t st) {
   if (R <= 0) return 0;
   if (y && (topk < 1 || topk > 64 || !pair_slot || !weights)) return TQ_ERR_BAD_ARG;
-  const int threads = 256;
+  // a row of 2,048 and more by 512 threads, so that each takes its four elements in one go and all of a row's loads
+  // are on their way at once (a function of H alone: a row's sums do not depend on what else the step holds)
+  const int threads = (H % 4 == 0 && H >= 2048) ? 512 : 256;
   const size_t shmem = (size_t)((H + 3) / 4 * 4 + threads / TQ_WAVE) * sizeof(float);
   if (shmem > 150 * 1024) return TQ_ERR_UNSUPPORTED;
   TQ_DISPATCH_W(wtype, {
