@@ -196,7 +196,8 @@ def test_a_gated_pair_of_a_few_hundred_rows_in_either_tile(ops, M, N):
 
 @pytest.mark.parametrize("act", ACTS)
 @pytest.mark.parametrize("M,N,K,bias", [(300, 200, 2200, True), (129, 130, 4104, False), (70, 64, 1000, False), (9, 40, 4096, True),
-                                        (40, 264, 8200, True), (64, 2048, 5632, False), (17, 72, 4096, False)])
+                                        (40, 264, 8200, True), (64, 2048, 5632, False), (17, 72, 4096, False), (33, 130, 2112, True),
+                                        (50, 96, 400, False), (32, 200, 4096, False)])
 def test_gemm_partial_sums(ops, act, M, N, K, bias):
     """A product may come back as partial sums over runs of k ([S, M, N], the bias in the first); however many the
     kernel makes, their sum is the product."""
@@ -206,21 +207,26 @@ def test_gemm_partial_sums(ops, act, M, N, K, bias):
     y = ops.gemm(a.to(DEV), w.to(DEV), act, bias=None if b is None else b.to(DEV), partial_sums=True).cpu()
     assert y.dim() == 3 and tuple(y.shape[1:]) == (M, N)
     if act == "bfloat16":
+        def tile_runs():    # tiles of 64 rows: up to 8 runs of at least 256 while the workgroups are few and the sums small
+            tiles, t = -(-M // 64) * -(-N // 128), 1
+            while t < 8 and tiles * t * 2 <= 512 and K // (t * 2) >= 256 and t * 2 * M * N * 4 <= 8 << 20:
+                t *= 2
+            while t > 1 and (t - 1) * (-(-(-(-K // 64)) // t) * 64) >= K:    # no run begins past the end
+                t //= 2
+            return t
+
         if M <= 16:
             runs = 1
+        elif 32 < M <= 64 and tile_runs() > 1:      # 33 to 64 rows take the tile kernel where it may split k
+            runs = tile_runs()
         elif M <= 64:       # few rows of a narrow matrix: runs of at least 128 of k for each of 8 waves, up to 4096 waves
             runs, waves = 1, -(-N // 32) * 8
             while runs < 8 and waves * runs < 4096 and K // (16 * runs) >= 128:
                 runs *= 2
         else:
             runs = 1 if K < 2048 else (2 if K < 4096 else 4)
-            if M <= 1024:   # tiles of 64 rows: up to 8 runs of at least 256 while the workgroups are few and the sums small
-                tiles, t = -(-M // 64) * -(-N // 128), 1
-                while t < 8 and tiles * t * 2 <= 512 and K // (t * 2) >= 256 and t * 2 * M * N * 4 <= 8 << 20:
-                    t *= 2
-                runs = max(runs, t)
-                while runs > 1 and (runs - 1) * (-(-(-(-K // 64)) // runs) * 64) >= K:    # no run begins past the end
-                    runs //= 2
+            if M <= 1024:
+                runs = max(runs, tile_runs())
         assert y.shape[0] == runs
     ref = ref_gemm(a, w, b, None)
     scale = ref.abs().max().item()

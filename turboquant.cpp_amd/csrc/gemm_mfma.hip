@@ -626,13 +626,38 @@ static bool gated_pair_in_tiles_of_64(int M, int N) {
 
 // Into how many runs of k a plain product of M rows may be split when its partial sums are wanted apart.  Many
 // rows: a product whose tiles do not fill the chip twice, and that has k enough, goes faster in 2 to 4 runs, each
-// at least 1024 long.  17 to 64 rows of a narrow matrix with a long k (the streaming kernel with at most 8 waves
-// over k): as many runs as bring about 4096 waves, each wave keeping 128 of k (64 rows by 2,048 x 2,048: 13.4 us in
-// two runs against 15.2 in one; by 2,048 x 5,632: 17.3 in four against 20.7 in two).  1 for up to 16 rows.
+// at least 1024 long, and up to 1,024 rows as tile_runs says.  17 to 64 rows of a narrow matrix with a long k in the
+// streaming kernel (at most 8 waves over k): as many runs as bring about 4096 waves, each wave keeping 128 of k
+// (64 rows by 2,048 x 2,048: 13.4 us in two runs against 15.2 in one; by 2,048 x 5,632: 17.3 in four against 20.7
+// in two); from 33 rows on the tile kernel with its runs instead, where it may split k.  1 for up to 16 rows.
+// Runs of k for a product that goes in tiles of 64 rows (up to 1,024 rows): a workgroup's time is its steps over k
+// (about 0.6 us each, whatever the memory does), so up to 8 runs, each at least 256 long, while the workgroups stay
+// within two to a compute unit and the partial sums within 8 MB, which the kernel behind has to read (128 rows by
+// 2,048 x 2,048: 8.7 us in eight runs against 14.6 in two; by 2,048 x 5,632: 13.7 against 19.3 in four).
+static int tile_runs(int M, int N, int K) {
+  const int64_t tiles64 = (int64_t)((M + 63) / 64) * ((N + TBN - 1) / TBN);
+  int t = 1;
+  while (t < 8 && tiles64 * t * 2 <= 512 && K / (t * 2) >= 256 && (int64_t)t * 2 * M * N * 4 <= (8 << 20)) t *= 2;
+  // every run must begin before the end of k (runs are whole tiles of 64)
+  while (t > 1 && (int64_t)(t - 1) * (((K + TBK - 1) / TBK + t - 1) / t * TBK) >= K) t /= 2;
+  return t;
+}
+
+// Whether partial sums of 33 to 64 rows come from the tile kernel rather than the streaming one: where the tile
+// kernel may split k at all.  Its one row tile then has up to eight runs of k to the streaming kernel's two to four
+// (64 rows by 2,048 x 2,048: 7.9 us against 13.1; by 2,048 x 5,632: 12.9 against 17.0; by 3,584 x 20,480: 46 against
+// 62).
+// From 17 to 32 rows it is level (2,048 x 2,048: 6.7 to 7.6 us against 7.8 to 8.7; 2,048 x 5,632: 11.9 to 12.7 against
+// 10.6 to 11.8), and the streaming kernel's fewer runs are less for the next kernel to add.
+static bool few_rows_in_tiles(int M, int N, int K) {
+  return M > 32 && M <= 64 && !wide_enough_for_tiles(N) && tile_runs(M, N, K) > 1;
+}
+
 TQ_API int tq_gemm_mfma_splits(int M, int N, int K) {
   if (M <= 16) return 1;
   if (M <= 64) {
     if (wide_enough_for_tiles(N)) return 1;
+    if (few_rows_in_tiles(M, N, K)) return tile_runs(M, N, K);
     const int64_t waves = (int64_t)((N + 31) / 32) * 8;
     int s = 1;
     while (s < 8 && waves * s < 4096 && K / (16 * s) >= 128) s *= 2;
@@ -641,17 +666,9 @@ TQ_API int tq_gemm_mfma_splits(int M, int N, int K) {
   const int64_t tiles = (int64_t)((M + 127) / 128) * ((N + TBN - 1) / TBN);
   int s = 1;
   while (s < 4 && tiles * s < 512 && K / (s * 2) >= 1024) s *= 2;
-  if (M <= 64 * 16) {
-    // Up to 1,024 rows go in tiles of 64 rows, and a workgroup's time is its steps over k (about 0.6 us each,
-    // whatever the memory does): up to 8 runs, each at least 256 long, while the workgroups stay within two to a
-    // compute unit and the partial sums within 8 MB, which the kernel behind has to read (128 rows by
-    // 2,048 x 2,048: 8.7 us in eight runs against 14.6 in two; by 2,048 x 5,632: 13.7 against 19.3 in four).
-    const int64_t tiles64 = (int64_t)((M + 63) / 64) * ((N + TBN - 1) / TBN);
-    int t = 1;
-    while (t < 8 && tiles64 * t * 2 <= 512 && K / (t * 2) >= 256 && (int64_t)t * 2 * M * N * 4 <= (8 << 20)) t *= 2;
+  if (M <= 64 * 16) {      // tiles of 64 rows: more and shorter runs
+    const int t = tile_runs(M, N, K);
     if (t > s) s = t;
-    // every run must begin before the end of k (runs are whole tiles of 64)
-    while (s > 1 && (int64_t)(s - 1) * (((K + TBK - 1) / TBK + s - 1) / s * TBK) >= K) s /= 2;
   }
   return s;
 }
@@ -711,6 +728,8 @@ TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gat
   } else if (M <= 16) {
     rc = launch_stream<1>(g, dual, out_act, 1, st);
   } else if (M <= 64 && wide_enough_for_tiles(N)) {
+    rc = launch_tile<64, 2, 4>(g, dual, out_act, splits, st);
+  } else if (M <= 64 && splits > 1 && few_rows_in_tiles(M, N, K)) {
     rc = launch_tile<64, 2, 4>(g, dual, out_act, splits, st);
   } else if (M <= 32) {
     rc = launch_stream<2>(g, dual, out_act, 1, st, splits);
