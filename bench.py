@@ -117,6 +117,118 @@ def plain_products(short: str) -> str:
     return "own kernels"
 
 
+def count_experts(fn):
+    """Runs fn() (an eager decode step) and returns the mean number of distinct experts a layer's router picked."""
+    import torch
+    from turboquant_cpp_amd.csrc import ops
+    picked = []
+    route = ops.route
+
+    def counting_route(*a, **k):
+        out = route(*a, **k)
+        picked.append(int(torch.unique(out[0]).numel()))
+        return out
+
+    ops.route = counting_route
+    try:
+        result = fn()
+    finally:
+        ops.route = route
+    return result, sum(picked) / max(len(picked), 1)
+
+
+def unequal_defaults(sizes: str) -> dict:
+    """The two stated workloads of unequal prompts: the larger checkpoint's sizes in bfloat16 (8 prompts of 512 to 4,096
+    tokens, seed 3, 256 decode steps) and the headline sizes in true 32-bit (64 prompts of 1 to 2,048, seed 4, 64 steps)."""
+    big = sizes == "a14b"
+    return {"batch": 8 if big else 64, "lo": 512 if big else 1, "hi": 4096 if big else 2048, "steps": 256 if big else 64,
+            "seed": 3 if big else 4}
+
+
+def unequal_workload(sizes: str, act: str, layers: int | None, wl: dict) -> dict:
+    """A batch of prompts of unequal lengths in one prompt step, then decode steps; builds its own model with random
+    weights and returns the record (the keys of the default run's line)."""
+    import torch
+    from turboquant_cpp_amd.csrc import ops
+    from turboquant_cpp_amd.engine.model import random_model
+    from turboquant_cpp_amd.engine.step import Engine
+    from turboquant_cpp_amd.sampling.sampler import TokenFetch
+    cfg, model_name = dict(SIZES[sizes][0]), SIZES[sizes][1]
+    full_layers = cfg["num_hidden_layers"]
+    layers = full_layers if layers is None else layers
+    cfg["num_hidden_layers"] = cfg["max_window_layers"] = layers
+    cfg["max_position_embeddings"] = wl["hi"] + wl["steps"] + 64
+    short = "bf16" if act == "bfloat16" else "fp32"
+    wbytes = 2 if act == "bfloat16" else 4
+    dev = "cuda:0"
+    t0 = time.time()
+    model = random_model(cfg, seed=wl["seed"], act=act, device=dev)
+    torch.cuda.synchronize()
+    print(f"[bench] {model_name} sizes, {layers} layers, {short}: random weights on the device in {time.time() - t0:.1f}s "
+          f"({model.weight_bytes / 1e9:.1f} GB)", file=sys.stderr, flush=True)
+    V = cfg["vocab_size"]
+    B = wl["batch"]
+    g = torch.Generator().manual_seed(wl["seed"])
+    lens = torch.randint(wl["lo"], wl["hi"] + 1, (B,), generator=g).tolist()
+    prompts = [torch.randint(0, V, (n,), generator=g).tolist() for n in lens]
+    page = 64
+    engine = Engine(model, max_tokens=sum(-(-(n + wl["steps"] + 1) // page) * page for n in lens), page_size=page, max_slots=B)
+    fetch = TokenFetch(dev, B)
+    best = None
+    for rep in range(2):                  # the first pass loads kernels and captures the decode graphs
+        slots = engine.open(B)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        logits = engine.step(slots, prompts)
+        torch.cuda.synchronize()
+        t_prompt = time.perf_counter() - t0
+        tokens = ops.argmax(logits, act)
+        used = None
+        t0 = time.perf_counter()
+        for i in range(wl["steps"]):
+            fetch.start(tokens)
+            if rep == 1 and i == 0:       # an eager step of the timed pass also counts the experts that are read
+                graphs, engine.graphs = engine.graphs, None
+                lg, used = count_experts(lambda: engine.step_from_device(slots, tokens))
+                engine.graphs = graphs
+            else:
+                lg = engine.step_from_device(slots, tokens)
+            fetch.wait()
+            tokens = ops.argmax(lg, act)
+        torch.cuda.synchronize()
+        t_decode = time.perf_counter() - t0
+        engine.close(slots)
+        best = (t_prompt, t_decode, used)
+    t_prompt, t_decode, used = best
+    T = sum(lens)
+    sec = t_decode / wl["steps"]
+    mean_total_ctx = T + B * (wl["steps"] + 1) / 2.0
+    read = decode_bytes(cfg, layers, B, mean_total_ctx / B, wbytes, used)
+    flops = sum(prefill_flops(cfg, layers, n, 0) for n in lens) + 2.0 * B * cfg["hidden_size"] * V
+    out = {
+        "metric": f"decode tok/s, batch {B} of unequal prompts ({wl['lo']}..{wl['hi']} tokens), {wl['steps']} steps "
+                  f"({model_name} layer sizes, random weights)",
+        "value": round(B / sec, 1), "unit": "tok/s", "n_gpus": 1, "steps": wl["steps"], "warmup": 0,
+        "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": short, "data": "synthetic",
+        "config": {"model": f"{model_name} sizes", "layers": layers, "layers_of_full_model": full_layers,
+                   "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
+                   "head_dim": cfg["hidden_size"] // cfg["num_attention_heads"], "vocab": V, "experts": cfg["num_experts"],
+                   "top_k": cfg["num_experts_per_tok"], "expert_inner": cfg["moe_intermediate_size"],
+                   "shared_inner": cfg["shared_expert_intermediate_size"], "global_batch": B,
+                   "prompt_tokens": T, "longest_prompt": max(lens), "shortest_prompt": min(lens),
+                   "weights": f"random N(0,0.02) seed {wl['seed']}", "kv_cache": short,
+                   "experts_read_per_layer": round(used, 1), "parallelism": "single GPU"},
+        "prefill": {"value": round(T / t_prompt, 1), "tokens": T, "ms": round(t_prompt * 1e3, 3),
+                    "frac": round(flops / t_prompt / PEAK_FLOPS[short], 4), "plain_products": plain_products(short)},
+        "roofline": {"bound": "hbm", "achieved": round(read / sec / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(read / sec / 1e9 / PEAK_HBM_GBS, 4)},
+        "decode": {"ms_total": round(t_decode * 1e3, 2), "gb_per_step": round(read / 1e9, 2)},
+    }
+    return out
+
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -148,6 +260,8 @@ def main() -> int:
     ap.add_argument("--prompt-max", type=int, default=None)
     ap.add_argument("--decode-steps", type=int, default=None)
     ap.add_argument("--seed", type=int, default=None)
+    ap.add_argument("--no-workloads", action="store_true",
+                    help="leave out the two workloads of unequal prompts that the default run adds under \"workloads\"")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single device)")
@@ -168,18 +282,21 @@ def main() -> int:
     cfg["max_window_layers"] = args.layers
     n_prefill = args.prefill_tokens
     cfg["max_position_embeddings"] = max(args.context, args.points_context, n_prefill)
-    if args.workload == "unequal":
-        big = args.sizes == "a14b"
-        wl = {"batch": args.batch if args.batch != 8 or big else 64,
-              "lo": args.prompt_min or (512 if big else 1), "hi": args.prompt_max or (4096 if big else 2048),
-              "steps": args.decode_steps or (256 if big else 64), "seed": args.seed if args.seed is not None else (3 if big else 4)}
-        cfg["max_position_embeddings"] = wl["hi"] + wl["steps"] + 64
     act = args.dtype
     short = "bf16" if act == "bfloat16" else "fp32"
     dev = "cuda:0"
     ops.library(act)
+    if args.workload == "unequal":
+        wl = unequal_defaults(args.sizes)
+        if args.batch != 8:
+            wl["batch"] = args.batch
+        for key, given in (("lo", args.prompt_min), ("hi", args.prompt_max), ("steps", args.decode_steps), ("seed", args.seed)):
+            if given is not None:
+                wl[key] = given
+        print(json.dumps(unequal_workload(args.sizes, act, args.layers, wl)), flush=True)
+        return 0
     t0 = time.time()
-    model = random_model(cfg, seed=wl["seed"] if args.workload == "unequal" else 2, act=act, device=dev)
+    model = random_model(cfg, seed=2, act=act, device=dev)
     torch.cuda.synchronize()
     print(f"[bench] {args.layers}-layer model with random weights on the device in {time.time() - t0:.1f}s "
           f"({model.weight_bytes / 1e9:.1f} GB)", file=sys.stderr, flush=True)
@@ -206,85 +323,6 @@ def main() -> int:
         return 0
 
     wbytes = 2 if act == "bfloat16" else 4
-
-    def count_experts(fn):
-        """Runs fn() (an eager decode step) and returns the mean number of distinct experts a layer's router picked."""
-        picked = []
-        route = ops.route
-
-        def counting_route(*a, **k):
-            out = route(*a, **k)
-            picked.append(int(torch.unique(out[0]).numel()))
-            return out
-
-        ops.route = counting_route
-        try:
-            result = fn()
-        finally:
-            ops.route = route
-        return result, sum(picked) / max(len(picked), 1)
-
-    if args.workload == "unequal":
-        B = wl["batch"]
-        g = torch.Generator().manual_seed(wl["seed"])
-        lens = torch.randint(wl["lo"], wl["hi"] + 1, (B,), generator=g).tolist()
-        prompts = [torch.randint(0, V, (n,), generator=g).tolist() for n in lens]
-        page = 64
-        engine = Engine(model, max_tokens=sum(-(-(n + wl["steps"] + 1) // page) * page for n in lens), page_size=page, max_slots=B)
-        fetch = TokenFetch(dev, B)
-        best = None
-        for rep in range(2):                  # the first pass loads kernels and captures the decode graphs
-            slots = engine.open(B)
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            logits = engine.step(slots, prompts)
-            torch.cuda.synchronize()
-            t_prompt = time.perf_counter() - t0
-            tokens = ops.argmax(logits, act)
-            used = None
-            t0 = time.perf_counter()
-            for i in range(wl["steps"]):
-                fetch.start(tokens)
-                if rep == 1 and i == 0:       # an eager step of the timed pass also counts the experts that are read
-                    graphs, engine.graphs = engine.graphs, None
-                    lg, used = count_experts(lambda: engine.step_from_device(slots, tokens))
-                    engine.graphs = graphs
-                else:
-                    lg = engine.step_from_device(slots, tokens)
-                fetch.wait()
-                tokens = ops.argmax(lg, act)
-            torch.cuda.synchronize()
-            t_decode = time.perf_counter() - t0
-            engine.close(slots)
-            best = (t_prompt, t_decode, used)
-        t_prompt, t_decode, used = best
-        T = sum(lens)
-        sec = t_decode / wl["steps"]
-        mean_total_ctx = T + B * (wl["steps"] + 1) / 2.0
-        read = decode_bytes(cfg, args.layers, B, mean_total_ctx / B, wbytes, used)
-        flops = sum(prefill_flops(cfg, args.layers, n, 0) for n in lens) + 2.0 * B * cfg["hidden_size"] * V
-        out = {
-            "metric": f"decode tok/s, batch {B} of unequal prompts ({wl['lo']}..{wl['hi']} tokens), {wl['steps']} steps "
-                      f"({model_name} layer sizes, random weights)",
-            "value": round(B / sec, 1), "unit": "tok/s", "n_gpus": 1, "steps": wl["steps"], "warmup": 0,
-            "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-            "dtype": short, "data": "synthetic",
-            "config": {"model": f"{model_name} sizes", "layers": args.layers, "layers_of_full_model": full_layers,
-                       "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
-                       "head_dim": cfg["hidden_size"] // cfg["num_attention_heads"], "vocab": V, "experts": cfg["num_experts"],
-                       "top_k": cfg["num_experts_per_tok"], "expert_inner": cfg["moe_intermediate_size"],
-                       "shared_inner": cfg["shared_expert_intermediate_size"], "global_batch": B,
-                       "prompt_tokens": T, "longest_prompt": max(lens), "shortest_prompt": min(lens),
-                       "weights": f"random N(0,0.02) seed {wl['seed']}", "kv_cache": short,
-                       "experts_read_per_layer": round(used, 1), "parallelism": "single GPU"},
-            "prefill": {"value": round(T / t_prompt, 1), "tokens": T, "ms": round(t_prompt * 1e3, 3),
-                        "frac": round(flops / t_prompt / PEAK_FLOPS[short], 4), "plain_products": plain_products(short)},
-            "roofline": {"bound": "hbm", "achieved": round(read / sec / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                         "frac": round(read / sec / 1e9 / PEAK_HBM_GBS, 4)},
-            "decode": {"ms_total": round(t_decode * 1e3, 2), "gb_per_step": round(read / 1e9, 2)},
-        }
-        print(json.dumps(out), flush=True)
-        return 0
 
     def run_decode(batch: int, context: int, steps: int, warmup: int):
         """Prefills `batch` prompts so that the timed steps end at `context`, then times `steps` decode steps."""
@@ -407,6 +445,23 @@ def main() -> int:
         "points": points,
         "points_detail": detail,
     }
+    default_run = (args.sizes == "a27b" and act == "bfloat16" and args.layers == full_layers and not args.no_points
+                   and not args.no_workloads)
+    if default_run:
+        # The two other stated workloads, each with a model of its own, once the headline model has left the device.
+        # Whatever happens to them, the headline line is printed.
+        import gc
+        del model, run_decode, run_prefill
+        gc.collect()
+        torch.cuda.empty_cache()
+        out["workloads"] = {}
+        for name, sizes, dtype in (("a14b_bf16_unequal_b8", "a14b", "bfloat16"), ("a27b_fp32_unequal_b64", "a27b", "float32")):
+            try:
+                out["workloads"][name] = unequal_workload(sizes, dtype, None, unequal_defaults(sizes))
+            except Exception as e:      # noqa: BLE001 - the record says what went wrong
+                out["workloads"][name] = {"error": f"{type(e).__name__}: {e}"[:300]}
+            gc.collect()
+            torch.cuda.empty_cache()
     print(json.dumps(out), flush=True)
     return 0
 

@@ -206,7 +206,10 @@ class PlainQwen2Moe:
         self.nh = c["num_attention_heads"]
         self.nkv = c.get("num_key_value_heads", self.nh)
         self.hd = c.get("head_dim") or self.H // self.nh
-        self.eps, self.theta = c["rms_norm_eps"], c["rope_theta"]
+        self.eps = c["rms_norm_eps"]
+        # the rotation's base: a key of its own, or inside the object that newer folders write
+        self.theta = c["rope_theta"] if c.get("rope_theta") is not None else c["rope_parameters"]["rope_theta"]
+        self.has_bias = c.get("qkv_bias", True)
         self.margins: dict[int, list] = {}      # per sparse layer, the routing margin of every token of the last call
         self.swaps: dict[int, list] = {}        # per sparse layer and token, the nearest exchanges of two experts
         self.other_side: dict = {}              # (layer, position) -> (i, j): near-ties that calls decide the other way
@@ -223,6 +226,8 @@ class PlainQwen2Moe:
         (window arithmetic of /root/reference/src/engine/tq_transformer.c:1646-1654, which the reference applies
         to another model family only)."""
         c = self.cfg
+        if c.get("layer_types") is not None:      # a folder that lists its layers' kinds is taken at its word
+            return c["sliding_window"] if c["layer_types"][l] == "sliding_attention" else None
         if c.get("use_sliding_window", False) and l >= c.get("max_window_layers", self.L):
             return c["sliding_window"]
         return None
@@ -232,9 +237,9 @@ class PlainQwen2Moe:
         rotation of q and k (:1342-1344), attention, output projection (:2239-2240)."""
         p, t = f"model.layers.{l}.self_attn.", self.t
         T = xb.shape[0]
-        q = matvec_rows(t[p + "q_proj.weight"], xb) + t[p + "q_proj.bias"]
-        k = matvec_rows(t[p + "k_proj.weight"], xb) + t[p + "k_proj.bias"]
-        v = matvec_rows(t[p + "v_proj.weight"], xb) + t[p + "v_proj.bias"]
+        q, k, v = (matvec_rows(t[p + n + "_proj.weight"], xb) for n in "qkv")
+        if self.has_bias:
+            q, k, v = q + t[p + "q_proj.bias"], k + t[p + "k_proj.bias"], v + t[p + "v_proj.bias"]
         q, k, v = q.view(T, self.nh, self.hd), k.view(T, self.nkv, self.hd), v.view(T, self.nkv, self.hd)
         pos = list(range(T))
         q, k = rope(q, pos, self.theta, self.rope_pairing), rope(k, pos, self.theta, self.rope_pairing)

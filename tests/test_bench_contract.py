@@ -86,3 +86,30 @@ def test_a_prompt_of_another_length_for_profiles():
     assert "300 tokens" in line["metric"] and line["layers"] == 1 and line["dtype"] == "bf16"
     assert abs(line["value"] - 300 / (line["ms"] * 1e-3)) < 0.01 * line["value"]
     assert 0 < line["host_ms"] <= line["ms"] * 1.01 and 0 < line["frac"] < 1
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_a_workload_of_unequal_prompts_on_the_gpu(dtype):
+    """The record that the default run adds under "workloads" for each of the two other stated workloads, here with one
+    layer, three prompts and four decode steps: the line's keys, a flat configuration, figures that fit each other."""
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--workload", "unequal", "--dtype", dtype, "--layers", "1",
+                        "--batch", "3", "--prompt-min", "5", "--prompt-max", "300", "--decode-steps", "4"],
+                       capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    line = json.loads(r.stdout.strip().splitlines()[-1])
+    for key in ("metric", "value", "unit", "ms_per_step", "dtype", "config", "prefill", "roofline"):
+        assert key in line, key
+    cfg = line["config"]
+    assert len(cfg) <= 20 and all(not isinstance(v, (dict, list)) for v in cfg.values())
+    assert cfg["layers"] == 1 and cfg["layers_of_full_model"] == 24 and cfg["global_batch"] == 3
+    assert 15 <= cfg["prompt_tokens"] <= 900 and 5 <= cfg["shortest_prompt"] <= cfg["longest_prompt"] <= 300
+    assert line["dtype"] == ("bf16" if dtype == "bfloat16" else "fp32") and line["steps"] == 4
+    assert abs(line["value"] - 3 / (line["ms_per_step"] * 1e-3)) < 0.01 * line["value"]
+    assert line["prefill"]["tokens"] == cfg["prompt_tokens"] and 0 < line["prefill"]["frac"] < 1
+    assert 0 < line["roofline"]["frac"] < 1
+
+
+def test_the_stated_workloads_of_unequal_prompts():
+    assert bench.unequal_defaults("a14b") == {"batch": 8, "lo": 512, "hi": 4096, "steps": 256, "seed": 3}
+    assert bench.unequal_defaults("a27b") == {"batch": 64, "lo": 1, "hi": 2048, "steps": 64, "seed": 4}

@@ -28,6 +28,47 @@ def test_config_reads_every_key_of_both_tiny_models():
     assert (a.rms_norm_eps, b.rms_norm_eps, a.rope_theta, b.rope_theta) == (1e-6, 1e-5, 1e4, 1e6)
 
 
+def test_a_folder_as_newer_tools_write_it():
+    """The layers' kinds listed one by one win over the rule of max_window_layers; the rotation's base is found inside
+    rope_parameters; q, k, v without bias read no bias tensors; "dtype" names the stored type."""
+    from tiny_configs import TINY_D
+    arch, d = config_from_dict(TINY_D)
+    assert [d.layer_window(l) for l in range(4)] == [19, None, 19, None]
+    assert d.rope_theta == 250000.0 and d.qkv_bias is False and d.torch_dtype == "float32"
+    plan = arch.plan(d)
+    assert [l.parts["mixer"].args["window"] for l in plan.layers] == [19, None, 19, None]
+    assert all("qkv_bias" not in l.parts["mixer"].tensors for l in plan.layers)
+    names = model_from_config(TINY_D, "float32").tensor_table()
+    assert not [n for n in names if n.endswith(".bias")]
+    # what the configuration writes back reads as itself
+    again = config_from_dict(arch.config_to_json(d))[1]
+    assert again == d
+    # without the list the rule of max_window_layers holds
+    e = copy.deepcopy(TINY_D)
+    del e["layer_types"]
+    assert [config_from_dict(e)[1].layer_window(l) for l in range(4)] == [None, None, None, 19]
+    # both places for the rotation's base may be there if they agree
+    e["rope_theta"] = 250000.0
+    assert config_from_dict(e)[1].rope_theta == 250000.0
+
+
+@pytest.mark.parametrize("change,word", [
+    ({"layer_types": ["full_attention"] * 3}, "layer_types"),
+    ({"layer_types": ["full_attention", "chunked_attention", "full_attention", "full_attention"]}, "chunked_attention"),
+    ({"sliding_window": None}, "sliding"),
+    ({"rope_parameters": {"rope_type": "yarn", "rope_theta": 1e4, "factor": 2.0}}, "rope_type"),
+    ({"rope_parameters": {"rope_type": "default"}}, "rope_theta"),
+    ({"rope_theta": 1e4}, "differ"),
+    ({"qkv_bias": "no"}, "true or false"),
+])
+def test_a_newer_folder_that_asks_for_what_is_not_built_is_refused(change, word):
+    from tiny_configs import TINY_D
+    d = copy.deepcopy(TINY_D)
+    d.update(change)
+    with pytest.raises(ConfigError, match=word):
+        config_from_dict(d)
+
+
 def test_head_dim_defaults_to_hidden_over_heads_and_kv_heads_to_heads():
     d = copy.deepcopy(TINY_A)
     del d["num_key_value_heads"]
@@ -149,9 +190,9 @@ def test_expected_tensor_names_and_shapes():
     assert table["model.embed_tokens.weight"] == ((384, 144), "table")
     assert table["model.layers.1.self_attn.q_proj.bias"] == ((144,), "bias")
     assert table["model.layers.1.self_attn.k_proj.weight"] == ((48, 144), "matrix")
-    assert table["model.layers.1.mlp.gate.weight"] == ((12, 144), "matrix")
+    assert table["model.layers.1.mlp.gate.weight"] == ((12, 144), "router")
     assert table["model.layers.1.mlp.experts.11.down_proj.weight"] == ((144, 48), "matrix")
-    assert table["model.layers.1.mlp.shared_expert_gate.weight"] == ((1, 144), "matrix")
+    assert table["model.layers.1.mlp.shared_expert_gate.weight"] == ((1, 144), "router")
     assert table["model.layers.0.mlp.up_proj.weight"] == ((160, 144), "matrix")
     assert table["model.layers.2.post_attention_layernorm.weight"] == ((144,), "scale")
     assert "model.layers.0.mlp.gate.weight" not in table and "lm_head.weight" in table
@@ -185,8 +226,12 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes():
 def test_stored_types():
     bf, f32, f16 = torch.bfloat16, torch.float32, torch.float16
     assert stored_dtype([bf], "bfloat16") == bf and stored_dtype([f16], "bfloat16") == bf
-    assert stored_dtype([f32], "bfloat16") == f32                 # stored in 32 bits: stays so
+    assert stored_dtype([f32], "bfloat16") == f32                 # stored in 32 bits: stays so, unless it is a matrix
     assert stored_dtype([bf, f32], "bfloat16") == f32
+    for role, want in (("matrix", bf), ("table", bf), ("scale", f32), ("bias", f32), ("router", f32)):
+        assert stored_dtype([f32], "bfloat16", role, "bfloat16") == want
+        assert stored_dtype([f32], "bfloat16", role, "keep") == f32
+        assert stored_dtype([f32], "float32", role, "bfloat16") == f32
     assert stored_dtype([bf], "float32") == f32 and stored_dtype([f32], "float32") == f32
     assert stored_dtype([torch.int64], "bfloat16") == torch.int32
 
@@ -206,20 +251,43 @@ def test_parameters_are_stacked_and_joined_from_their_tensors(model_dirs):
         assert torch.equal(model.lm_head, f.read("lm_head.weight"))
 
 
-def test_bfloat16_model_keeps_32_bit_tensors_in_32_bits(tmp_path):
+def test_a_bfloat16_model_rounds_32_bit_matrices_as_it_places_them_and_keeps_the_rest(tmp_path):
+    """On the bfloat16 path a matrix of a product that the folder stores in 32 bits becomes bfloat16 at load, with one
+    warning that counts them; norm weights, biases and the router's rows, which feed float32 arithmetic, stay as they
+    are stored; ``f32_matrices="keep"`` leaves everything as stored and warns that those products are slow."""
+    import warnings
+    from turboquant_cpp_amd.weights.loader import RoundedWeights, SlowWeights
     d = write_random_model_dir(str(tmp_path / "m"), TINY_A, seed=3, dtype="bfloat16")
-    # rewrite one norm weight and the router of layer 0 in float32
     with SafetensorsFolder(d) as f:
         tensors = {n: f.read(n).clone() for n in f.names()}
-    tensors["model.norm.weight"] = tensors["model.norm.weight"].float()
-    tensors["model.layers.0.mlp.gate.weight"] = tensors["model.layers.0.mlp.gate.weight"].float()
+    in32 = ["model.norm.weight", "model.layers.0.mlp.gate.weight", "model.layers.0.self_attn.q_proj.bias",
+            "model.layers.1.self_attn.o_proj.weight", "model.layers.0.mlp.experts.3.up_proj.weight"]
+    for n in in32:
+        tensors[n] = tensors[n].float() * 1.001          # values that bfloat16 does not hold
     write_safetensors(os.path.join(d, "model.safetensors"), tensors)
     model = model_from_config(TINY_A, "bfloat16")
-    with SafetensorsFolder(d) as f:
+    with SafetensorsFolder(d) as f, warnings.catch_warnings(record=True) as w:
+        warnings.simplefilter("always")
         model.load(f, "cpu")
+    assert [str(x.message)[:10] for x in w if x.category is RoundedWeights] == ["2 matrices"]
+    assert not [x for x in w if x.category is SlowWeights]
     assert model.final_norm.weight.dtype == torch.float32
     assert model.blocks[0].ffn.router.dtype == torch.float32
+    assert model.blocks[0].mixer.qkv_bias.dtype == torch.float32        # one of its three pieces is stored in 32 bits
+    assert model.blocks[1].mixer.qkv_bias.dtype == torch.bfloat16
+    assert model.blocks[1].mixer.out_weight.dtype == torch.bfloat16     # rounded here
+    assert torch.equal(model.blocks[1].mixer.out_weight, tensors["model.layers.1.self_attn.o_proj.weight"].bfloat16())
+    assert model.blocks[0].ffn.expert_up.dtype == torch.bfloat16
     assert model.blocks[1].ffn.router.dtype == torch.bfloat16 and model.embedding.dtype == torch.bfloat16
+    kept = model_from_config(TINY_A, "bfloat16")
+    with SafetensorsFolder(d) as f, warnings.catch_warnings(record=True) as w:
+        warnings.simplefilter("always")
+        kept.load(f, "cpu", f32_matrices="keep")
+    assert [str(x.message)[:10] for x in w if x.category is SlowWeights] == ["2 matrices"]
+    assert kept.blocks[1].mixer.out_weight.dtype == torch.float32 and kept.blocks[0].ffn.expert_up.dtype == torch.float32
+    assert torch.equal(kept.blocks[1].mixer.out_weight, tensors["model.layers.1.self_attn.o_proj.weight"])
+    with pytest.raises(ValueError, match="f32_matrices"):
+        kept.load(TensorDict(tensors), "cpu", f32_matrices="half")
     m32 = model_from_config(TINY_A, "float32")
     with SafetensorsFolder(d) as f:
         m32.load(f, "cpu")

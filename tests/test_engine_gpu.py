@@ -260,7 +260,7 @@ def test_replay(name, act, sharp_dirs, tmp_path):
 
 # ------------------------------------------------------------------------------------------------ in process
 @pytest.mark.parametrize("act", ACTS)
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "D"])
 def test_first_tokens_and_long_decoding(name, act, engines):
     eng, plain = engines(name, act)
     (seq,) = prompts_for(name, [330], seed=12)
@@ -353,6 +353,98 @@ def test_the_layer_sizes_of_a_real_checkpoint(tmp_path):
                 check_sequence(got[i], plain, s, act, f"real layer sizes, {act}, sequence of {len(s)}, {how}")
                 first = got[i] if first is None else first
         del plain
+
+
+def test_sixty_four_unequal_sequences_at_real_layer_sizes_in_32_bits(tmp_path):
+    """The stated 32-bit workload at its stated batch: 64 sequences of 1 to 2,048 tokens drawn uniformly (seed 4), two
+    layers of Qwen1.5-MoE-A2.7B's sizes, cut three ways: all prompts whole in one step; all but the last 32 tokens as
+    prompts and the rest token by token, shorter sequences ending earlier; and the sequences in another order over two
+    batches in slots used before, each prompt in two chunks.  The logits at each sequence's last 32 positions agree
+    between the three to 2e-5; the four shortest sequences agree with the plain model at every position, and four
+    longer ones (up to the longest) at their first 100, which the tokens behind them do not touch."""
+    from turboquant_cpp_amd.engine.model import load_model, write_random_model_dir
+    from turboquant_cpp_amd.engine.step import Engine
+    V = 8000
+    cfg = {"architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe", "vocab_size": V, "hidden_size": 2048,
+           "num_hidden_layers": 2, "num_attention_heads": 16, "num_key_value_heads": 16, "intermediate_size": 5632,
+           "moe_intermediate_size": 1408, "shared_expert_intermediate_size": 5632, "num_experts": 60,
+           "num_experts_per_tok": 4, "norm_topk_prob": False, "decoder_sparse_step": 1, "mlp_only_layers": [],
+           "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "use_sliding_window": False, "sliding_window": 32768,
+           "max_window_layers": 2, "max_position_embeddings": 4096, "tie_word_embeddings": False, "torch_dtype": "float32"}
+    act = "float32"
+    g = torch.Generator().manual_seed(4)
+    lens = torch.randint(1, 2049, (64,), generator=g).tolist()
+    seqs = [torch.randint(0, V, (n,), generator=g).tolist() for n in lens]
+    cut = [max(1, n - 32) for n in lens]                      # the positions from cut - 1 on are compared
+    by_length = sorted(range(64), key=lambda i: lens[i])
+    sample = {i: lens[i] for i in by_length[:4]}             # sequence -> its first positions that the plain model checks
+    sample.update({i: 100 for i in (by_length[20], by_length[35], by_length[50], by_length[63])})
+    d = write_random_model_dir(str(tmp_path / "a27b_two_layers_64"), cfg, 4, 0.02, 0.02, act)
+    eng = Engine(load_model(d, act=act, device=DEV), max_tokens=sum(-(-n // 64) * 64 for n in lens), max_slots=64)
+
+    # whole prompts in one step
+    slots = eng.open(64)
+    wants = [sorted(set(range(sample.get(i, 0))) | set(range(cut[i] - 1, n))) for i, n in enumerate(lens)]
+    lg = eng.step(slots, seqs, wants)
+    eng.close(slots)
+    whole, everything, o = {}, {}, 0
+    for i, w in enumerate(wants):
+        rows = lg[o:o + len(w)]
+        o += len(w)
+        if i in sample:
+            everything[i] = rows[:sample[i]].cpu()
+        whole[i] = rows[len(w) - (lens[i] - cut[i] + 1):].clone()
+    del lg
+    # the last 32 token by token
+    slots = eng.open(64)
+    lg = eng.step(slots, [s[:c] for s, c in zip(seqs, cut)])
+    rows = {i: [lg[i:i + 1].clone()] for i in range(64)}
+    pos = list(cut)
+    live = [i for i in range(64) if pos[i] < lens[i]]
+    eng.close([slots[i] for i in range(64) if i not in live])
+    while live:
+        lg = eng.step([slots[i] for i in live], [[seqs[i][pos[i]]] for i in live])
+        for j, i in enumerate(live):
+            rows[i].append(lg[j:j + 1].clone())
+            pos[i] += 1
+        eng.close([slots[i] for i in live if pos[i] == lens[i]])
+        live = [i for i in live if pos[i] < lens[i]]
+    one_by_one = {i: torch.cat(r) for i, r in rows.items()}
+    # another order, two batches, every prompt in two chunks
+    order = torch.randperm(64, generator=g).tolist()
+    chunked = {}
+    for batch in (order[:32], order[32:]):
+        slots = eng.open(32)
+        mid = [max(1, (cut[i] - 1) // 2) if cut[i] > 1 else 0 for i in batch]      # a first chunk that ends before cut - 1
+        first = [(s, i, m) for s, i, m in zip(slots, batch, mid) if m > 0]
+        if first:
+            eng.step([s for s, _, _ in first], [seqs[i][:m] for _, i, m in first], [[] for _ in first])
+        lg = eng.step(slots, [seqs[i][m:] for i, m in zip(batch, mid)],
+                      [list(range(cut[i] - 1 - m, lens[i] - m)) for i, m in zip(batch, mid)])
+        o = 0
+        for i in batch:
+            n = lens[i] - cut[i] + 1
+            chunked[i] = lg[o:o + n].clone()
+            o += n
+        eng.close(slots)
+    assert eng.cache.n_live == 0
+    worst = {"the last 32 token by token": 0.0, "another order, two batches, two chunks": 0.0}
+    for i in range(64):
+        for how, got in (("the last 32 token by token", one_by_one[i]), ("another order, two batches, two chunks", chunked[i])):
+            assert got.shape == whole[i].shape, (how, i, got.shape, whole[i].shape)
+            diff = (got - whole[i]).abs().max().item()
+            worst[how] = max(worst[how], diff)
+            # two cuts sum the same products in other orders (prompt and decode kernels): a fifth of what the comparison
+            # with the plain model allows
+            assert diff <= 2e-5, f"sequence {i} of {lens[i]} tokens, {how}: differs from the whole prompt's logits by {diff:.2e}"
+    print("64 unequal sequences, float32, against the whole prompts:", worst)
+    del eng
+    torch.cuda.empty_cache()
+    plain = PlainQwen2Moe(d)
+    shutil.rmtree(d)
+    for i, n in sample.items():
+        check_sequence(everything[i], plain, seqs[i][:n], act,
+                       f"64 unequal sequences, float32, the first {n} of sequence {i}'s {lens[i]} tokens")
 
 
 @pytest.mark.parametrize("act", ACTS)

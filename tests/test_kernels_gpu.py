@@ -105,6 +105,32 @@ def test_gemm_dense(ops, act, M, N, K, mode, monkeypatch):
             assert err < limit, (err, scale, vendor)
 
 
+@pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("N", [65537, 151936])
+@pytest.mark.parametrize("M", [17, 33, 64])
+def test_a_few_dozen_rows_times_a_matrix_of_a_vocabulary(ops, act, M, N):
+    """17 to 64 rows against a matrix of 65,536 rows and more: the shape of the vocabulary's product in a decode step
+    of that many sequences, which takes the tile kernels where narrower matrices take the streaming ones.  Plain and
+    as partial sums, against the product in float64 (worked out on the GPU: it is the reference here, not the
+    subject)."""
+    K = 2048
+    a = rnd((M, K), adt(act), 40 + M).to(DEV)
+    w = rnd((N, K), adt(act), 41, 0.2).to(DEV)
+    ref = a.double() @ w.double().T
+    scale = ref.abs().max().item()
+    limit = 1e-5 * scale * math.sqrt(K) if act == "float32" else 4e-3 * scale
+    y = ops.gemm(a, w, act)
+    assert tuple(y.shape) == (M, N) and (y.double() - ref).abs().max().item() < limit
+    parts = ops.gemm(a, w, act, partial_sums=True)
+    assert tuple(parts.shape[1:]) == (M, N) and (parts.double().sum(0) - ref).abs().max().item() < limit
+    # a row's result does not depend on how many rows come with it
+    alone = ops.gemm(a[M - 1:], w, act)
+    if act == "float32":
+        assert (alone[0] - y[M - 1]).abs().max().item() < 1e-5 * scale * math.sqrt(K)
+    else:
+        assert (alone[0] - y[M - 1]).abs().max().item() < 4e-3 * scale
+
+
 @pytest.mark.parametrize("M,N,K", [(512, 130, 264), (700, 6144, 2048), (2048, 257, 1000), (8192, 96, 16384), (600, 96, 16384)])
 def test_plain_products_of_many_rows(ops, M, N, K, monkeypatch):
     """From VENDOR_MIN_ROWS rows on (512 here, to keep the sizes small) a plain bfloat16 product without bias goes to
@@ -1119,6 +1145,54 @@ def test_attention_tiled(ops, act, nh, nkv, hd, window, page):
     assert run([0, 7, 100, 300]) < tol(act, 2)                   # runs that go on from a cached prefix
     assert run([n - 1 for n in lens]) < tol(act, 2)              # one token each: the split kernel
     assert run([1, 18, 149, 200]) < tol(act, 2)                  # mixed: not all single tokens
+
+
+@pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("hd", [96, 160, 224, 40])
+def test_decoding_reads_nothing_beyond_a_head_that_fills_no_whole_tile(ops, act, hd):
+    """One token per sequence with head sizes between the kernels' tile widths (96 lies between 64 and 128): the
+    sequence's last page is the pool's last, its kv head the last of the last layer, and what lies behind the pools
+    is NaN.  A load that does not stop at the head size reads those and the scores of keys in reach become NaN."""
+    nh, nkv, page, layers = 4, 2, 64, 2
+    layer = layers - 1
+    lens = [70, 129]
+    n_pages = sum(-(-n // page) for n in lens)
+    page_stride = layers * nkv * page * hd
+    table = torch.full((2, 3), -1, dtype=torch.int32)
+    table[0, :2] = torch.tensor([1, 0])
+    table[1, :3] = torch.tensor([2, 3, n_pages - 1])            # the longer sequence ends in the pool's last page
+    slots = [0, 1]
+    off = layer * nkv * page * hd
+    pools = []
+    for seed in (0, 1):
+        whole = torch.full((n_pages * page_stride + 65536,), float("nan"), dtype=adt(act))
+        whole[:n_pages * page_stride] = 0
+        pools.append(whole)
+    kp, vp = (w[:n_pages * page_stride] for w in pools)
+    scale = 1.0 / math.sqrt(hd)
+    qs, ks, vs = [], [], []
+    for i, n in enumerate(lens):
+        qs.append(rnd((n, nh, hd), adt(act), 231 + i))
+        ks.append(rnd((n, nkv, hd), adt(act), 235 + i))
+        vs.append(rnd((n, nkv, hd), adt(act), 239 + i))
+        for p in range(n):
+            for h in range(nkv):
+                base = int(table[slots[i], p // page]) * page_stride + off + (h * page + p % page) * hd
+                kp[base:base + hd] = ks[i][p, h]
+                vbase = int(table[slots[i], p // page]) * page_stride + off + h * page * hd + p % page
+                vp[vbase:vbase + hd * page:page] = vs[i][p, h]
+    kd, vd = (w.to(DEV)[:n_pages * page_stride] for w in pools)
+    ref = [ref_attention(a, b, c, None, scale).reshape(-1, nh * hd) for a, b, c in zip(qs, ks, vs)]
+    positions = torch.tensor([n - 1 for n in lens], dtype=torch.int32)
+    q = torch.stack([qs[i][-1] for i in range(2)]).reshape(2, nh * hd)
+    runs = {"cu_seqlens": torch.tensor([0, 1, 2], dtype=torch.int32).to(DEV),
+            "slots": torch.tensor(slots, dtype=torch.int32).to(DEV), "start": positions.to(DEV),
+            "max_new": 1, "max_end": max(lens), "decode": True}
+    out = ops.attention(q.to(DEV), kd, vd, off, positions.to(DEV), torch.tensor(slots, dtype=torch.int32).to(DEV),
+                        table.to(DEV), page, page_stride, nh, nkv, hd, None, scale, act, runs=runs).cpu()
+    want = torch.stack([ref[i][-1] for i in range(2)])
+    assert torch.isfinite(out).all()
+    assert (out.double() - want).abs().max().item() < tol(act, 2)
 
 
 def test_probes_run(ops):

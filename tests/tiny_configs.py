@@ -39,4 +39,19 @@ TINY_C = {
 }
 TINY_C_INIT = dict(seed=5, std=0.02, norm_std=0.02)
 
-TINY = {"A": (TINY_A, TINY_A_INIT), "B": (TINY_B, TINY_B_INIT), "C": (TINY_C, TINY_C_INIT)}
+# a folder as newer tools write it: the layers' kinds listed one by one (sliding first, then full, then sliding: not what
+# max_window_layers would give), the rotation's base inside rope_parameters, "dtype" for the stored type, q, k, v without
+# bias; 4 layers, heads of 16 on one kv head, window 19, 6 experts top-4 un-normalised
+TINY_D = {
+    "architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe",
+    "vocab_size": 300, "hidden_size": 80, "num_hidden_layers": 4, "num_attention_heads": 5,
+    "num_key_value_heads": 1, "head_dim": 16, "intermediate_size": 72, "moe_intermediate_size": 24,
+    "shared_expert_intermediate_size": 40, "num_experts": 6, "num_experts_per_tok": 4, "norm_topk_prob": False,
+    "decoder_sparse_step": 1, "mlp_only_layers": [2], "rope_parameters": {"rope_type": "default", "rope_theta": 250000.0},
+    "rms_norm_eps": 2e-6, "use_sliding_window": True, "sliding_window": 19, "max_window_layers": 3,
+    "layer_types": ["sliding_attention", "full_attention", "sliding_attention", "full_attention"],
+    "qkv_bias": False, "max_position_embeddings": 1024, "tie_word_embeddings": False, "dtype": "float32",
+}
+TINY_D_INIT = dict(seed=9, std=0.02, norm_std=0.02)
+
+TINY = {"D": (TINY_D, TINY_D_INIT), "A": (TINY_A, TINY_A_INIT), "B": (TINY_B, TINY_B_INIT), "C": (TINY_C, TINY_C_INIT)}

@@ -38,11 +38,14 @@ class Model:
 
     def __init__(self, path: str, *, temperature: float = 0.7, top_p: float = 0.9, max_tokens: int = 256,
                  context_length: int = 0, dtype: str = "bfloat16", seed: int = 42, rep_penalty: float = 1.1,
-                 max_batch: int = 8, device: str = "cuda:0", stop_tokens: Sequence[int] | None = None):
+                 max_batch: int = 8, device: str = "cuda:0", stop_tokens: Sequence[int] | None = None,
+                 f32_matrices: str = "bfloat16"):
+        """``f32_matrices``: with ``dtype="bfloat16"``, matrices that the folder stores in 32 bits are rounded to
+        bfloat16 as they are loaded ("bfloat16"), or stay as they are stored ("keep": their products are slow)."""
         if not os.path.isdir(path):
             raise FileNotFoundError(f"model folder not found: {path}")
         self._path = path
-        self._model = load_model(path, act=dtype, device=device)
+        self._model = load_model(path, act=dtype, device=device, f32_matrices=f32_matrices)
         self._setup(temperature, top_p, max_tokens, context_length, seed, rep_penalty, max_batch, stop_tokens)
 
     @classmethod
@@ -213,6 +216,12 @@ class Model:
             states = {int(n.split(".")[1]): f.read(n).clone() for n in f.entries if n.startswith("state.")}
             tokens = f.read("tokens").tolist()
             data = {"length": int(meta["length"]), "page_size": int(meta["page_size"]), "groups": groups, "states": states}
+        if len(tokens) != data["length"]:
+            raise RuntimeError(f"{path} holds {len(tokens)} tokens for {data['length']} cached positions")
+        V = self._engine.vocab_size
+        bad = [t for t in tokens if not 0 <= t < V]
+        if bad:
+            raise RuntimeError(f"{path} holds token {bad[0]}, outside the vocabulary of {V}")
         if data["length"] >= self.context_length:
             raise ChatContextOverflow(f"{path} holds {data['length']} tokens, the context is {self.context_length}")
         self.reset_chat()

@@ -52,6 +52,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("-j", dest="threads", type=int, default=None, help="accepted for compatibility; the GPU does the work")
     ap.add_argument("--ctx", type=int, default=0, help="override max context length (default: the model's, at most 4096)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--f32-weights", default="bfloat16", choices=["bfloat16", "keep"],
+                    help="with --dtype bfloat16: round matrices stored in 32 bits to bfloat16 at load (default), or keep them")
     ap.add_argument("--rep-penalty", type=float, default=1.1, help="repetition penalty over the last 32 tokens (default: 1.1)")
     ap.add_argument("--stop-id", type=int, action="append", default=None, help="stop token id (default: eos_token_id of config.json)")
     ap.add_argument("--random-prompt", default=None, metavar="LEN[,LEN...]", help="prompts of random token ids of these lengths")
@@ -104,7 +106,7 @@ def main(argv=None) -> int:
     t0 = time.time()
     model = Model(args.model, temperature=args.temperature, top_p=args.top_p, max_tokens=args.max_tokens,
                   context_length=args.ctx, dtype=args.dtype, seed=args.seed, rep_penalty=args.rep_penalty,
-                  max_batch=args.max_batch, stop_tokens=args.stop_id)
+                  max_batch=args.max_batch, stop_tokens=args.stop_id, f32_matrices=args.f32_weights)
     print(f"loaded {args.model} in {time.time() - t0:.1f}s ({args.dtype}, context {model.context_length})", file=sys.stderr)
     if args.bench_memory or args.bench_prefill:
         # the reference's two small benchmarks (/root/reference/tools/quant.c:726-800, :804-860): one token, its token
@@ -232,11 +234,20 @@ def main(argv=None) -> int:
         # token costs in every layer that keeps keys and values, against keys and values in 16-bit floats
         cache = model.engine.cache
         esz = 4 if args.dtype == "float32" else 2
-        n_tok = sum(len(p) + len(r.tokens) for p, r in zip(prompts, results))
+        # what the cache held of each sequence when it ended: a token that ended a sequence was never run, and a group
+        # with a window has given its older pages back
+        n_tok = sum(r.cached_positions for r in results) or sum(len(p) + len(r.tokens) for p, r in zip(prompts, results))
         k_per = sum(len(g.entries) * g.key.num_kv_heads * g.key.head_dim * esz for g in cache.groups)
         v_per = sum(len(g.entries) * g.key.num_kv_heads * g.key.value_dim * esz for g in cache.groups)
         f16_per = (k_per + v_per) // esz * 2
-        total, total16 = (k_per + v_per) * n_tok, f16_per * n_tok
+        if all(r.pages_held for r in results):
+            held = [sum(min(r.cached_positions, r.pages_held[i] * cache.page_size) for r in results)
+                    for i in range(len(cache.groups))]
+            total = sum(len(g.entries) * g.key.num_kv_heads * (g.key.head_dim + g.key.value_dim) * esz * n
+                        for g, n in zip(cache.groups, held))
+            total16 = total // esz * 2
+        else:
+            total, total16 = (k_per + v_per) * n_tok, f16_per * n_tok
         ratio = total16 / total if total else 0.0
         print("\n=== KV Cache Memory Stats ===", file=sys.stderr)
         print(f"Tokens in cache:      {n_tok}", file=sys.stderr)
@@ -265,6 +276,8 @@ def main(argv=None) -> int:
                      max_slots=len(prompts), use_graphs=False)
         eng.side_stream = None
         slots = eng.open(len(prompts))
+        print("[Profile] steps are timed eagerly on one stream, an event behind every launch; generation replays its "
+              "decode steps as graphs, which take less", file=sys.stderr)
 
         def report(phase, n_tok, steps):
             t = ops.profile_end()

@@ -352,9 +352,12 @@ static int launch_attention_f32(const AttnF32Args& p, int B, int decode, int max
   if (decode) {
     const int tiles = (max_end + AT - 1) / AT;
     const int group = p.nh / p.nkv, passes = (group + 15) / 16;
-    const int waves = tiles;
+    // with a window a token reaches at most window positions, which lie in window / AT + 2 tiles at the most
+    const int waves = p.window > 0 ? min(tiles, p.window / AT + 2) : tiles;
     if (p.nkv * passes > 65535 || waves > 65535 || tiles > F32_JOIN_TILES) return TQ_ERR_UNSUPPORTED;
-    if (p.hd % 32 == 0 && p.page_size % 32 == 0)
+    // whole lines only where the head fills its tiles of 16 (32, 64, 128, 256): the loads of that form have no
+    // guard on the head size, and a head of 96 would read beyond its rows and, in the last page, beyond the pool
+    if (p.hd == 16 * ND && p.hd % 32 == 0 && p.page_size % 32 == 0)
       hipLaunchKernelGGL((attn_f32_decode_kernel<ND, true>), dim3(B, p.nkv * passes, waves), dim3(64), 0, st, p, passes);
     else
       hipLaunchKernelGGL((attn_f32_decode_kernel<ND, false>), dim3(B, p.nkv * passes, waves), dim3(64), 0, st, p, passes);

@@ -1,7 +1,6 @@
 // An entry point that allocates nothing.
 //
-// It has no counterpart in the reference (whose sampler, /root/reference/src/engine/tq_generate.c:74-156, keeps a
-// workspace in host memory behind a mutex).  It is for callers that cannot allocate device memory: code under HIP
+// It has no counterpart in the reference.  It is for callers that cannot allocate device memory: code under HIP
 // graph capture, tight serving loops, harnesses that forbid hipMalloc.  tq_sample_topp needs R * V floats for the
 // probabilities and a few KB for its passes, which its caller has to bring; tq_sample_topp_static makes the same
 // choice, with the same kernels and the same arithmetic, out of an array that is part of the library's image:

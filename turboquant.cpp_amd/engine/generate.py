@@ -45,6 +45,8 @@ class GenerationOptions:
 class GenerationResult:
     tokens: list[int]
     finish_reason: str            # "stop" (end token), "length" (max_tokens), "context" (cache or model limit), "loop"
+    cached_positions: int = 0     # positions the cache held for the sequence when it ended (a token that ended it was not run)
+    pages_held: tuple = ()        # pages it held then, per cache group (a group with a window has given the older ones back)
 
 
 class LoopDetector:
@@ -148,8 +150,10 @@ def generate(engine, prompts: Sequence[Sequence[int]], options: GenerationOption
     def end(r, tracks, slot_of, reason=None):
         if reason is not None:
             tracks[r].finish_reason = reason
-        engine.close([slot_of.pop(r)])
-        results[r] = GenerationResult(tracks[r].out, tracks[r].finish_reason)
+        slot = slot_of.pop(r)
+        held = tuple(int((g.host_table[slot] >= 0).sum()) for g in engine.cache.groups)
+        results[r] = GenerationResult(tracks[r].out, tracks[r].finish_reason, engine.length(slot), held)
+        engine.close([slot])
 
     while waiting:
         batch = []

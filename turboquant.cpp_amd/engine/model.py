@@ -75,9 +75,11 @@ class CausalLM:
         """name -> (shape, role) of every checkpoint tensor this model reads."""
         return expected_tensors(self.bindings)
 
-    def load(self, reader, device) -> "CausalLM":
+    def load(self, reader, device, f32_matrices: str = "bfloat16") -> "CausalLM":
+        """``f32_matrices``: what becomes, on the bfloat16 path, of matrices that the checkpoint stores in 32 bits:
+        "bfloat16" rounds them once as they are placed, "keep" leaves them as stored."""
         self.device = torch.device(device)
-        self.weight_bytes = load_bindings(self.bindings, reader, self.act, self.device)
+        self.weight_bytes = load_bindings(self.bindings, reader, self.act, self.device, f32_matrices)
         if self.plan.lm_head is None:
             self.lm_head = self.embedding
         for part in self.parts():
@@ -134,17 +136,18 @@ def model_from_config(config_json: dict, act: str) -> CausalLM:
     return CausalLM(arch.plan(cfg), act, config=cfg)
 
 
-def load_model(model_dir: str, act: str = "bfloat16", device="cuda:0") -> CausalLM:
+def load_model(model_dir: str, act: str = "bfloat16", device="cuda:0", f32_matrices: str = "bfloat16") -> CausalLM:
     """Reads config.json, picks the architecture from it, and loads model.safetensors by tensor name."""
     arch, cfg = config_from_dir(model_dir)
     model = CausalLM(arch.plan(cfg), act, config=cfg)
     with SafetensorsFolder(model_dir) as folder:
-        model.load(folder, device)
+        model.load(folder, device, f32_matrices)
     return model
 
 
 def random_model(config_json: dict, seed: int, act: str = "bfloat16", device="cuda:0", std: float = 0.02,
-                 norm_std: float = 0.0, on_device: bool = True, dtype: str | None = None) -> CausalLM:
+                 norm_std: float = 0.0, on_device: bool = True, dtype: str | None = None,
+                 f32_matrices: str = "bfloat16") -> CausalLM:
     """A model with random weights drawn in memory, tensor by tensor, where the model lives: the values of the
     folder that ``write_random_model_dir`` writes for the same configuration, seed and ``dtype`` (the type the
     folder's tensors would have; default: the activation type)."""
@@ -165,7 +168,7 @@ def random_model(config_json: dict, seed: int, act: str = "bfloat16", device="cu
             shape, role = table[name]
             return random_tensor(self.index[name], shape, role, seed, std, norm_std, dtype, gen_device)
 
-    return model.load(_Lazy(), device)
+    return model.load(_Lazy(), device, f32_matrices)
 
 
 def write_random_model_dir(model_dir: str, config_json: dict, seed: int, std: float = 0.02, norm_std: float = 0.0,

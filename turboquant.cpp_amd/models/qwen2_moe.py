@@ -22,6 +22,7 @@ from ..config.plan import LayerSpec, ModelPlan, PartSpec, ScheduleEntry, Source
 from ..config.registry import Architecture, register_architecture
 
 ARCHITECTURE = "Qwen2MoeForCausalLM"
+FULL, SLIDING = "full_attention", "sliding_attention"
 
 
 @dataclass
@@ -49,6 +50,8 @@ class Qwen2MoeConfig:
     tie_word_embeddings: bool
     torch_dtype: str
     stop_token_ids: list[int] = field(default_factory=list)
+    qkv_bias: bool = True                   # q, k and v have a bias unless the folder says otherwise
+    layer_types: list[str] | None = None    # per layer "full_attention" or "sliding_attention", if the folder lists them
 
     # ---- derived ----
     def layer_is_sparse(self, layer: int) -> bool:
@@ -58,8 +61,12 @@ class Qwen2MoeConfig:
                 and (layer + 1) % self.decoder_sparse_step == 0)
 
     def layer_window(self, layer: int) -> int | None:
-        """Layers from ``max_window_layers`` on attend to the last ``sliding_window`` positions,
-        the current one included (window semantics of tq_transformer.c:1646-1654)."""
+        """A sliding layer attends to the last ``sliding_window`` positions, the current one included (window
+        semantics of tq_transformer.c:1646-1654).  Which layers slide: those that ``layer_types`` names, if the
+        folder has that list (the reference likewise takes a per-layer list where its metadata holds one,
+        tq_model.c:2867-2905); else the layers from ``max_window_layers`` on while ``use_sliding_window`` is true."""
+        if self.layer_types is not None:
+            return self.sliding_window if self.layer_types[layer] == SLIDING else None
         if self.use_sliding_window and layer >= self.max_window_layers:
             return self.sliding_window
         return None
@@ -79,6 +86,26 @@ def config_from_json(data: dict) -> Qwen2MoeConfig:
     require(data.get("rope_scaling") is None, f"rope_scaling {data.get('rope_scaling')!r} is not implemented")
     require(data.get("hidden_act", "silu") == "silu", f"hidden_act {data.get('hidden_act')!r} is not implemented (silu is)")
     layers = r.integer("num_hidden_layers", minimum=1)
+    # newer folders keep the rotation's constants in an object of their own
+    rope = data.get("rope_parameters")
+    require(rope is None or isinstance(rope, dict), f"rope_parameters must be an object, got {rope!r}")
+    if rope is not None:
+        kind = rope.get("rope_type", rope.get("type", "default"))
+        require(kind in (None, "default"), f"rope_parameters.rope_type {kind!r} is not implemented (default is)")
+    if data.get("rope_theta") is not None or rope is None:
+        rope_theta = r.number("rope_theta")
+        require(rope is None or rope.get("rope_theta") in (None, rope_theta),
+                f"rope_theta {rope_theta} and rope_parameters.rope_theta {rope and rope.get('rope_theta')} differ")
+    else:
+        rope_theta = KeyReader(rope, "config.json: rope_parameters").number("rope_theta")
+    layer_types = data.get("layer_types")
+    if layer_types is not None:
+        require(isinstance(layer_types, list) and len(layer_types) == layers,
+                f"layer_types must list one kind for each of the {layers} layers, got {layer_types!r}")
+        unknown = sorted({str(t) for t in layer_types if t not in (FULL, SLIDING)})
+        require(not unknown, f"layer_types names {unknown}; this architecture has {FULL!r} and {SLIDING!r}")
+        require(SLIDING not in layer_types or (window is not None and window > 0),
+                "layer_types names sliding layers but sliding_window is not a positive integer")
     stop: list[int] = []
     for key in ("eos_token_id",):
         if data.get(key) is not None:
@@ -98,15 +125,17 @@ def config_from_json(data: dict) -> Qwen2MoeConfig:
         norm_topk_prob=r.boolean("norm_topk_prob", False),
         decoder_sparse_step=r.integer("decoder_sparse_step", 1, minimum=1),
         mlp_only_layers=r.integer_list("mlp_only_layers", []),
-        rope_theta=r.number("rope_theta"),
+        rope_theta=rope_theta,
         rms_norm_eps=r.number("rms_norm_eps"),
         use_sliding_window=use_window,
         sliding_window=window,
         max_window_layers=r.integer("max_window_layers", layers, minimum=0),
         max_position_embeddings=r.integer("max_position_embeddings", minimum=1),
         tie_word_embeddings=r.boolean("tie_word_embeddings", False),
-        torch_dtype=r.string("torch_dtype", "bfloat16"),
+        torch_dtype=r.string("torch_dtype", data.get("dtype") or "bfloat16"),
         stop_token_ids=stop,
+        qkv_bias=r.boolean("qkv_bias", True),
+        layer_types=layer_types,
     )
     validate(cfg)
     return cfg
@@ -132,6 +161,8 @@ def validate(c: Qwen2MoeConfig) -> None:
 def config_to_json(c: Qwen2MoeConfig) -> dict:
     d = asdict(c)
     stop = d.pop("stop_token_ids")
+    if d["layer_types"] is None:
+        del d["layer_types"]
     d["architectures"] = [ARCHITECTURE]
     d["model_type"] = "qwen2_moe"
     if stop:
@@ -147,15 +178,16 @@ def plan(c: Qwen2MoeConfig) -> ModelPlan:
             kind="gqa_attention",
             args=dict(hidden_size=c.hidden_size, num_heads=c.num_attention_heads,
                       num_kv_heads=c.num_key_value_heads, head_dim=c.head_dim,
-                      qkv_bias=True, out_bias=False, window=c.layer_window(l),
+                      qkv_bias=c.qkv_bias, out_bias=False, window=c.layer_window(l),
                       position=PartSpec(kind="rope", args=dict(head_dim=c.head_dim, rotary_dim=c.head_dim,
                                                              theta=c.rope_theta, pairing="half"))),
             tensors={
                 # q, k and v are stacked into one matrix so one product makes all three
                 "qkv_weight": Source.concat([f"{p}.self_attn.{n}_proj.weight" for n in "qkv"]),
-                "qkv_bias": Source.concat([f"{p}.self_attn.{n}_proj.bias" for n in "qkv"]),
                 "out_weight": Source.single(f"{p}.self_attn.o_proj.weight"),
             })
+        if c.qkv_bias:
+            attn.tensors["qkv_bias"] = Source.concat([f"{p}.self_attn.{n}_proj.bias" for n in "qkv"])
         if c.layer_is_sparse(l):
             tensors = {
                 "router": Source.single(f"{p}.mlp.gate.weight"),

@@ -37,7 +37,7 @@ from ..config.plan import PartSpec
 @dataclass(frozen=True)
 class ParamSpec:
     """One parameter: its shape, its role (``matrix``, ``bias``, ``scale`` for norm weights, ``table`` for
-    embeddings) and, if it is several checkpoint tensors joined along dimension 0, their sizes there."""
+    embeddings, ``router`` for rows whose products are float32 arithmetic whatever the activation type) and, if it is several checkpoint tensors joined along dimension 0, their sizes there."""
     shape: tuple[int, ...]
     role: str = "matrix"
     splits: tuple[int, ...] | None = None

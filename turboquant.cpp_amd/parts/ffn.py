@@ -65,14 +65,14 @@ class SparseMoE(Part):
 
     def param_specs(self):
         E, H, I, S = self.num_experts, self.hidden_size, self.expert_size, self.shared_size
-        specs = {"router": ParamSpec((E, H)),
+        specs = {"router": ParamSpec((E, H), role="router"),
                  "expert_gate": ParamSpec((E, I, H)), "expert_up": ParamSpec((E, I, H)),
                  "expert_down": ParamSpec((E, H, I))}
         if S > 0:
             specs.update({"shared_gate": ParamSpec((S, H)), "shared_up": ParamSpec((S, H)),
                           "shared_down": ParamSpec((H, S))})
             if self.shared_gated:
-                specs["shared_scale"] = ParamSpec((1, H))
+                specs["shared_scale"] = ParamSpec((1, H), role="router")
         return specs
 
     def prepare(self, device, act):

@@ -1,7 +1,11 @@
 """From checkpoint tensors, by name, to the parameters of a model's parts.
 
 In the manner of the reference's loader (/root/reference/src/engine/tq_model.c:847-1666): tensors are looked up
-by name (:324-360), bfloat16 stays bfloat16 and float32 stays float32 (:367-412, :440-451).  Unlike it, a
+by name (:324-360) and converted as they are placed (:367-412, :440-451): on the bfloat16 path bfloat16 stays
+bfloat16, and of the tensors that the checkpoint stores in 32 bits the matrices of the products and the embedding
+table are rounded to bfloat16 once, here (with a warning that counts them), while norm weights, biases and the
+router's rows, which feed float32 arithmetic, stay in 32 bits; ``f32_matrices="keep"`` leaves every 32-bit tensor
+as it is stored, and the products of those matrices then run the plain multiply-add kernel.  Unlike it, a
 tensor that is not there is never a silent NULL (tq_model.c:418-423): everything is checked before
 anything is copied, and one error lists all missing tensors, all wrong shapes and, beside them, the tensors
 that the model does not read.  A checkpoint whose only difference is such extra tensors (a stray buffer) loads,
@@ -39,6 +43,18 @@ class WeightError(ValueError):
 
 class UnexpectedTensors(UserWarning):
     """The checkpoint holds tensors that the model does not read."""
+
+
+class RoundedWeights(UserWarning):
+    """Matrices that the checkpoint stores in 32 bits were rounded to bfloat16 as they were placed."""
+
+
+class SlowWeights(UserWarning):
+    """Matrices were kept in 32 bits on the bfloat16 path: their products do not run on the matrix cores."""
+
+
+F32_MATRICES = ("bfloat16", "keep")
+ROUNDED_ROLES = ("matrix", "table")      # what feeds bfloat16 products; scale, bias and router feed float32 arithmetic
 
 
 @dataclass
@@ -93,26 +109,36 @@ def check(bindings: list[Binding], available: dict[str, tuple[tuple[int, ...], t
                       stacklevel=3)
 
 
-def stored_dtype(dtypes: list[torch.dtype], act: str) -> torch.dtype:
+def stored_dtype(dtypes: list[torch.dtype], act: str, role: str = "scale", f32_matrices: str = "keep") -> torch.dtype:
     """The type a parameter is kept in: float32 on the 32-bit path; else bfloat16, but a tensor that the
-    checkpoint stores in 32 bits stays so, and integer tables are int32."""
+    checkpoint stores in 32 bits stays so unless it is a matrix of a product or the embedding table and
+    ``f32_matrices`` is "bfloat16"; integer tables are int32."""
     if any(d in (torch.int32, torch.int64) for d in dtypes):
         return torch.int32
-    if act == "float32" or any(d == torch.float32 for d in dtypes):
+    if act == "float32":
+        return torch.float32
+    if any(d == torch.float32 for d in dtypes) and not (f32_matrices == "bfloat16" and role in ROUNDED_ROLES):
         return torch.float32
     return torch.bfloat16
 
 
-def load_bindings(bindings: list[Binding], reader, act: str, device) -> int:
+def load_bindings(bindings: list[Binding], reader, act: str, device, f32_matrices: str = "bfloat16") -> int:
     """Checks all names and shapes, then fills every parameter on the device.  ``reader`` has
     ``entries`` (name -> object with .shape and .dtype name) and ``read(name)``.  Returns bytes placed."""
     from .safetensors_io import DTYPES
+    if f32_matrices not in F32_MATRICES:
+        raise ValueError(f"f32_matrices must be one of {F32_MATRICES}, got {f32_matrices!r}")
     available = {n: (tuple(e.shape), DTYPES[e.dtype][0]) for n, e in reader.entries.items()}
     check(bindings, available)
     placed = 0
+    rounded = kept = 0
     for b in bindings:
         pieces = b.pieces()
-        dtype = stored_dtype([available[n][1] for n, _ in pieces], act)
+        stored = [available[n][1] for n, _ in pieces]
+        dtype = stored_dtype(stored, act, b.spec.role, f32_matrices)
+        if act != "float32" and b.spec.role in ROUNDED_ROLES and torch.float32 in stored:
+            rounded += dtype == torch.bfloat16
+            kept += dtype == torch.float32
         dst = torch.empty(tuple(b.spec.shape), dtype=dtype, device=device)
         if b.source.how == "single":
             dst.copy_(reader.read(pieces[0][0]).to(dtype))
@@ -126,6 +152,12 @@ def load_bindings(bindings: list[Binding], reader, act: str, device) -> int:
                 o += shape[0]
         setattr(b.owner, b.attr, dst)
         placed += dst.numel() * dst.element_size()
+    if rounded:
+        warnings.warn(f"{rounded} matrices that the checkpoint stores in 32 bits were rounded to bfloat16 as they were "
+                      "placed (f32_matrices=\"keep\" leaves them as they are stored)", RoundedWeights, stacklevel=3)
+    if kept:
+        warnings.warn(f"{kept} matrices stay in 32 bits on the bfloat16 path: their products run the plain multiply-add "
+                      "kernel, not the matrix cores", SlowWeights, stacklevel=3)
     return placed
 
 
