@@ -117,8 +117,9 @@ def plain_products(short: str) -> str:
     return "own kernels"
 
 
-def count_experts(fn):
-    """Runs fn() (an eager decode step) and returns the mean number of distinct experts a layer's router picked."""
+def count_experts(fn, engine):
+    """Runs fn() (an eager decode step, part by part so that the routing can be watched) and returns the mean number of
+    distinct experts a layer's router picked."""
     import torch
     from turboquant_cpp_amd.csrc import ops
     picked = []
@@ -130,10 +131,12 @@ def count_experts(fn):
         return out
 
     ops.route = counting_route
+    executor, engine.native = engine.native, None
     try:
         result = fn()
     finally:
         ops.route = route
+        engine.native = executor
     return result, sum(picked) / max(len(picked), 1)
 
 
@@ -189,7 +192,7 @@ def unequal_workload(sizes: str, act: str, layers: int | None, wl: dict) -> dict
             fetch.start(tokens)
             if rep == 1 and i == 0:       # an eager step of the timed pass also counts the experts that are read
                 graphs, engine.graphs = engine.graphs, None
-                lg, used = count_experts(lambda: engine.step_from_device(slots, tokens))
+                lg, used = count_experts(lambda: engine.step_from_device(slots, tokens), engine)
                 engine.graphs = graphs
             else:
                 lg = engine.step_from_device(slots, tokens)
@@ -354,7 +357,7 @@ def main() -> int:
             return ops.argmax(lg, act)
 
         # the first warm-up step (which runs eagerly) also counts the distinct experts that each layer's router picks
-        tokens, experts_used = count_experts(lambda: one_step(tokens))
+        tokens, experts_used = count_experts(lambda: one_step(tokens), engine)
         for _ in range(warmup - 1):
             tokens = one_step(tokens)
         torch.cuda.synchronize()

@@ -133,6 +133,33 @@ def test_window_group_gives_back_pages_that_no_later_token_reaches():
     held(c)
 
 
+def test_a_group_with_a_window_has_pages_for_its_windows_only():
+    """With few slots, the pool of a group that keeps a window holds what the windows and one step's new positions
+    need (window 100 + 128 new positions: 4 pages of 64, and two for where they begin and end) and no more; the
+    group that keeps everything has all pages.  Sequences that grow in steps of that length never find it empty."""
+    c = two_group_cache(max_tokens=64 * 200, max_slots=3, window_step=128)
+    full, win = c.groups
+    assert full.pool.n_pages == 200 and win.pool.n_pages == 3 * (4 + 2) and c.step_limit == 128
+    slots = [c.open() for _ in range(3)]
+    for step in range(30):
+        for s in slots:
+            c.reserve(s, 128 if step % 3 else 1)
+        for s in slots:
+            c.commit(s)
+        held(c)
+    assert all(c.length(s) == 20 * 128 + 10 for s in slots)
+    # a step of more positions is for the caller to cut: the whole of it has room or not, before anything runs
+    c.room_for(slots, [1000, 1000, 1000])
+    with pytest.raises(CacheFull):
+        c.room_for(slots, [5000, 3000, 3000])
+    for s in slots:
+        c.close(s)
+    held(c)
+    # with many slots the windows would take more than every page there is: the pool is no smaller then, no limit
+    many = two_group_cache(max_tokens=64 * 20)
+    assert many.step_limit is None and all(g.pool.n_pages == 20 for g in many.groups)
+
+
 def test_a_sequence_that_outgrows_the_cache_is_refused_and_nothing_leaks():
     c = two_group_cache(max_tokens=64 * 3)
     s, t = c.open(), c.open()
@@ -253,6 +280,32 @@ def test_step_logits_equal_the_plain_model_whole_split_and_batched(cpu_engine, m
                 if pos[i] == len(prompts[i]):
                     eng.close([slots[i]])
         assert eng.cache.n_live == 0 and all(g.pool.n_free == g.pool.n_pages for g in eng.cache.groups)
+
+
+def test_a_long_prompt_runs_in_cuts_where_a_window_has_few_pages(cpu_engine, model_dirs):
+    """Configuration B keeps a window of 24 on two layers.  With three slots their group has pages for three windows and
+    a step of 64 positions, so prompts of 150 and 70 tokens go through in cuts of 64; the logits, asked for in an
+    order of their own, are the plain model's.  A step that the other group has no room for is refused whole."""
+    from plain_qwen2moe import PlainQwen2Moe
+    eng = cpu_engine("B", max_tokens=64 * 20, max_slots=3, window_step=64)
+    win = [g for g in eng.cache.groups if g.key.window is not None][0]
+    assert eng.cache.step_limit == 64 and win.pool.n_pages == 3 * (2 + 2) and eng.cache.n_pages == 20
+    plain = PlainQwen2Moe(model_dirs("B"))
+    g = torch.Generator().manual_seed(9)
+    prompts = [torch.randint(0, 384, (n,), generator=g).tolist() for n in (150, 20, 70)]
+    wants = [[149, 0, 64, 63, 100], [], [69, 5]]
+    slots = eng.open(3)
+    lg = eng.step(slots, prompts, wants)
+    ref = torch.cat([plain.logits(p).float()[w] for p, w in zip(prompts, wants) if w])
+    assert lg.shape == ref.shape and (lg - ref).abs().max() < 1e-4
+    assert [eng.length(s) for s in slots] == [150, 20, 70]
+    # one more position each, then a step that does not fit: nothing of it has run
+    eng.step(slots, [[1], [2], [3]])
+    with pytest.raises(CacheFull):
+        eng.step(slots, [[1] * 600, [2] * 600, [3] * 600])
+    assert [eng.length(s) for s in slots] == [151, 21, 71]
+    eng.close(slots)
+    assert all(g.pool.n_free == g.pool.n_pages for g in eng.cache.groups)
 
 
 def test_step_refuses_bad_input(cpu_engine):

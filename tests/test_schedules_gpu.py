@@ -78,6 +78,35 @@ def test_a_window_gives_pages_back_and_a_second_sequence_uses_them(act, sharp):
     check_sequence(out[True][1], plain, second, act, f"C {act} windowed decoding, second sequence")
 
 
+@pytest.mark.parametrize("act", ACTS)
+def test_a_window_with_few_pages_takes_long_prompts_in_cuts(act, sharp):
+    """Three slots, and the layers with a window of 40 have pages for three windows and a step of 128 positions (15
+    pages where the other layers have 40): prompts of 700, 300 and 50 tokens go through in cuts of 128, decoding goes
+    on behind them, and every position agrees with the plain model."""
+    from turboquant_cpp_amd.engine.step import Engine
+    d, plain, model = sharp("C", act)
+    eng = Engine(model, max_tokens=64 * 40, max_slots=3, window_step=128)
+    full, win = eng.cache.groups if eng.cache.groups[0].key.window is None else eng.cache.groups[::-1]
+    assert win.pool.n_pages == 3 * (3 + 2) and full.pool.n_pages == 40 and eng.cache.step_limit == 128
+    assert win.k_pages.numel() * 40 == full.k_pages.numel() * 15 * len(win.entries) // len(full.entries)
+    seqs = prompts_for("C", [700 + 6, 300 + 6, 50 + 6], seed=27)
+    slots = eng.open(3)
+    rows = eng.step(slots, [s[:-6] for s in seqs], [list(range(len(s) - 6)) for s in seqs])
+    per_seq, o = [], 0
+    for s in seqs:
+        per_seq.append([rows[o:o + len(s) - 6]])
+        o += len(s) - 6
+    for t in range(6, 0, -1):
+        lg = eng.step(slots, [[s[-t]] for s in seqs]).clone()
+        for i in range(3):
+            per_seq[i].append(lg[i:i + 1])
+    assert (win.host_table >= 0).sum() <= 3 * 2
+    eng.close(slots)
+    assert all(g.pool.n_free == g.pool.n_pages for g in eng.cache.groups)
+    for i, s in enumerate(seqs):
+        check_sequence(torch.cat(per_seq[i]), plain, s, act, f"C {act} prompt of {len(s) - 6} tokens in cuts of 128")
+
+
 # ------------------------------------------------------------------------------------------------ many sequences
 @pytest.mark.parametrize("act", ACTS)
 @pytest.mark.parametrize("name,n_seqs", [("A", 40), ("B", 17), ("C", 64), ("B", 530)])
@@ -101,16 +130,19 @@ def test_decode_steps_of_many_sequences(name, n_seqs, act, sharp, monkeypatch):
     out = {}
     for graphs in (True, False):
         eng = Engine(model, max_tokens=64 * n_seqs, max_slots=n_seqs, use_graphs=graphs)
+        # the step executor calls the vendor's library itself and counts; a step run part by part goes through torch.mm
+        vendor_products = lambda: len(calls) + (eng.native.vendor_products if eng.native is not None else 0)
         slots = eng.open(n_seqs)
         first = eng.step(slots, [s[:n] for s, n in zip(seqs, lens)], [list(range(n)) for n in lens])
-        assert bool(calls) == (act == "bfloat16" and sum(lens) >= 512)
-        del calls[:]
+        assert bool(vendor_products()) == (act == "bfloat16" and sum(lens) >= 512)
+        before = vendor_products()
         rows = []
         for t in range(n_dec):
             rows.append(eng.step(slots, [[s[n + t]] for s, n in zip(seqs, lens)]).clone())
             if t == 3:
                 torch.cuda.synchronize()
-        assert not calls
+        assert vendor_products() == before
+        del calls[:]
         eng.close(slots)
         if graphs:
             assert len(eng.graphs.graphs) == 1
@@ -311,15 +343,24 @@ def test_a_long_prompt_takes_the_taller_expert_tiles(sharp, monkeypatch):
 
     monkeypatch.setattr(ops, "route", spy)
     eng = Engine(model, max_tokens=64 * 40, page_size=64)
+    executor = eng.native
+    assert executor is not None
     for n, unit in ((1400, 128), (700, 64), (1400, 256)):
         monkeypatch.setattr(ops, "EXPERT_256_FROM", 256 if unit == 256 else 1024)
         (prompt,) = prompts_for("C", [n], seed=29)
         del units[:]
+        eng.native = None                   # part by part, where the spy sees the unit
         slots = eng.open(1)
         got = eng.step(slots, [prompt], [list(range(n))])
         eng.close(slots)
         assert units and all(u == unit for u in units), (n, units)
         check_sequence(got, plain, prompt, "bfloat16", f"C bfloat16 {n} tokens at once")
+        eng.native = executor               # and through the step executor, which takes the same unit: the same bits
+        del units[:]
+        slots = eng.open(1)
+        same = eng.step(slots, [prompt], [list(range(n))])
+        eng.close(slots)
+        assert not units and torch.equal(same, got), (n, (same - got).abs().max().item())
 
 
 # ------------------------------------------------------------------------------------------------ whose product it is
@@ -339,17 +380,25 @@ def test_a_long_prompt_whole_cut_and_with_every_product_in_own_kernels(name, sha
     real = torch.mm
     monkeypatch.setattr(torch, "mm", lambda *x, **kw: (calls.append(1), real(*x, **kw))[1])
     eng = Engine(model, max_tokens=64 * 24, page_size=64)
-    for vendor, cuts, label in ((True, [700], "whole"), (False, [700], "whole, own products"), (True, [250, 250, 200], "cut")):
-        monkeypatch.setattr(ops, "_VENDOR", vendor)
-        del calls[:]
-        slots = eng.open(1)
-        rows, at = [], 0
-        for n in cuts:
-            rows.append(eng.step(slots, [prompt[at:at + n]], [list(range(n))]).clone())
-            at += n
-        eng.close(slots)
-        assert bool(calls) == (vendor and cuts == [700]), (label, len(calls))
-        check_sequence(torch.cat(rows), plain, prompt, "bfloat16", f"{name} bfloat16 700 tokens {label}")
+    executor = eng.native
+    assert executor is not None
+    for by_executor in (True, False):           # the step executor calls the library itself; the parts go through torch.mm
+        eng.native = executor if by_executor else None
+        for vendor, cuts, label in ((True, [700], "whole"), (False, [700], "whole, own products"), (True, [250, 250, 200], "cut")):
+            monkeypatch.setattr(ops, "_VENDOR", vendor)
+            del calls[:]
+            before = executor.vendor_products
+            slots = eng.open(1)
+            rows, at = [], 0
+            for n in cuts:
+                rows.append(eng.step(slots, [prompt[at:at + n]], [list(range(n))]).clone())
+                at += n
+            eng.close(slots)
+            taken = executor.vendor_products - before if by_executor else len(calls)
+            assert bool(taken) == (vendor and cuts == [700]), (label, by_executor, taken)
+            assert by_executor or executor.vendor_products == before
+            check_sequence(torch.cat(rows), plain, prompt, "bfloat16",
+                           f"{name} bfloat16 700 tokens {label}, {'executor' if by_executor else 'part by part'}")
 
 
 # ------------------------------------------------------------------------------------------------ entry points

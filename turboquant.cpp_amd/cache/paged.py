@@ -11,7 +11,8 @@ blocks on demand with create / append / seq_len / free calls and status checks
   Slots are opened when a batch starts, closed when its sequence ends, and handed out again.
 * Keys and values live in *pages* of ``page_size`` positions.  Layers whose needs agree (kv heads,
   width of a key row, width of a value row, window) form a *group* with storage of its own: one pool of
-  pages, each page holding the rows of all the group's layers for ``page_size`` positions of one sequence:
+  pages (a group that keeps a window has a pool for its windows only: what every sequence's window, and the
+  ``window_step`` positions that one step may add to it, can hold), each page holding the rows of all the group's layers for ``page_size`` positions of one sequence:
   keys laid out ``[layer][kv head][row][head_dim]``, values transposed, ``[layer][kv head][value_dim][row]``
   (both as the attention kernels' operands want them).  Keys and values have pools of their own, so their
   rows may differ in width, and a group whose layers keep one row per position only (``value_dim`` 0) has no
@@ -175,9 +176,12 @@ class PagedCache:
     """
 
     def __init__(self, needs, max_tokens: int, dtype: torch.dtype, device, page_size: int = 64,
-                 max_slots: int | None = None, max_positions: int | None = None):
-        if page_size < 1 or max_tokens < 1:
-            raise CacheError("page_size and max_tokens must be positive")
+                 max_slots: int | None = None, max_positions: int | None = None, window_step: int = 2048):
+        """``window_step``: the most positions that one step adds to a sequence where a group keeps a window; such a
+        group's pool is sized for ``max_slots`` windows of that reach, and whoever runs longer steps cuts them
+        (``step_limit`` says so: None where no pool is smaller for it)."""
+        if page_size < 1 or max_tokens < 1 or window_step < 1:
+            raise CacheError("page_size, max_tokens and window_step must be positive")
         self.page_size = page_size
         self.n_pages = -(-max_tokens // page_size)
         self.max_slots = min(self.n_pages, 4096) if max_slots is None else max_slots
@@ -194,9 +198,18 @@ class PagedCache:
             if cache_need is not None and cache_of is None:
                 by_key.setdefault(GroupKey(cache_need.num_kv_heads, cache_need.head_dim, cache_need.value_width,
                                            cache_need.window), []).append(e)
-        self.groups: list[CacheGroup] = [
-            CacheGroup(key, entries, self.n_pages, page_size, self.max_slots, per_seq, dtype, device)
-            for key, entries in by_key.items()]
+        # A sequence holds, of a group with a window, the pages that its last `window` positions touch, and during a
+        # step those of the step's new positions too, until the step is committed: window + window_step positions
+        # lie in at most that many pages plus two.
+        self.step_limit: int | None = None
+        self.groups: list[CacheGroup] = []
+        for key, entries in by_key.items():
+            pages = self.n_pages
+            if key.window is not None:
+                for_windows = self.max_slots * (-(-(key.window + window_step) // page_size) + 2)
+                if for_windows < pages:
+                    pages, self.step_limit = for_windows, window_step
+            self.groups.append(CacheGroup(key, entries, pages, page_size, self.max_slots, per_seq, dtype, device))
         self._v_offset: dict[int, int] = {}
         for g in self.groups:
             for e in g.entries:
@@ -281,6 +294,21 @@ class PagedCache:
                 g.dirty.add(slot)
         s.reserved = n_new
         return s.length
+
+    def room_for(self, slots, counts) -> None:
+        """Raises CacheFull if the groups that keep every position (and each sequence's own bound) have no room for
+        ``counts[i]`` more positions in ``slots[i]``, all together; takes nothing.  For a step that is run in cuts:
+        the groups with a window have room for every cut by the size of their pools."""
+        need = 0
+        for slot, n in zip(slots, counts):
+            s = self._live(slot)
+            if s.length + n > self.max_positions:
+                raise CacheFull(f"sequence in slot {slot} would reach {s.length + n} positions, the cache holds {self.max_positions} per sequence")
+            held = (s.length + self.page_size - 1) // self.page_size
+            need += (s.length + n + self.page_size - 1) // self.page_size - held
+        for g in self.groups:
+            if g.key.window is None and need > g.pool.n_free:
+                raise CacheFull(f"cache needs {need} more pages, {g.pool.n_free} of {g.pool.n_pages} are free")
 
     def needs_page(self, slot: int, n_new: int = 1) -> bool:
         """Whether ``n_new`` more positions would take a page that the sequence does not hold yet."""

@@ -17,12 +17,15 @@ import time
 CSRC = os.path.dirname(os.path.abspath(__file__))
 
 # sources per activation type: each has matrix-core kernels of its own
-COMMON_SOURCES = ["elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "moe.hip", "sampling.hip"]
+# (host/: the step executor and its way into the vendor's matrix library, host code that calls the kernels' entry points)
+COMMON_SOURCES = ["elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "moe.hip", "sampling.hip",
+                  "host/engine.cpp", "host/vendor.cpp"]
 SOURCES = {
     "float32": COMMON_SOURCES + ["gemm_f32.hip", "attention_f32.hip"],
     "bfloat16": COMMON_SOURCES + ["gemm_mfma.hip", "attention_mfma.hip", "probe.hip"],
 }
-HEADERS = ["common.h", "no_alloc.h", "gemm_mfma.h"]
+HEADERS = ["common.h", "no_alloc.h", "gemm_mfma.h", "turboquant_kernels.h", "host/engine.h", "host/vendor.h",
+           "host/host_common.h"]
 DEFINES = {"float32": "-DTQ_ACT_F32", "bfloat16": "-DTQ_ACT_BF16"}
 FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-fno-gpu-rdc",
          # keep the compiler from forming packed 32-bit float instructions
@@ -106,7 +109,7 @@ def build(dtype: str, force: bool = False, verbose: bool = True) -> str:
     t0 = time.time()
     procs = []
     for src in sources:
-        obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
+        obj = os.path.join(obj_dir, os.path.splitext(os.path.basename(src))[0] + ".o")
         cmd = [hipcc, *FLAGS, DEFINES[dtype], "-c", os.path.join(CSRC, src), "-o", obj]
         # what the compiler prints goes to a file: a pipe that nobody reads while the compilers run together
         # would block the one that fills it
@@ -136,7 +139,7 @@ def build(dtype: str, force: bool = False, verbose: bool = True) -> str:
                 say(f"  still compiling: {', '.join(s for s, _, _, _ in pending)} ({time.time() - t0:.0f}s)")
                 last = time.time()
     tmp = target + f".tmp{os.getpid()}"
-    link = subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *sorted(objs), "-o", tmp],
+    link = subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *sorted(objs), "-ldl", "-o", tmp],
                           stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if link.returncode != 0:
         raise BuildError(f"hipcc failed to link {target}:\n{link.stdout}")

@@ -21,6 +21,7 @@ namespace {
 
 thread_local char g_error[512] = "";
 thread_local int64_t g_launches = 0;
+thread_local int64_t g_vendor_products = 0;
 
 int fail(int code, const char* fmt, ...) {
   va_list ap;
@@ -114,6 +115,7 @@ struct Product {
   int tile_rows = 0;
   int gate = 0;
   bool partial = false;
+  void* dest = nullptr;      // where the result goes, if not into the arena (never with partial sums)
 };
 
 bool vendor_product(const Ctx& c, const Product& p) {
@@ -133,18 +135,20 @@ int product(Ctx& c, const Product& p, void** out, int* splits, int side = 0) {
   const size_t esz = p.out_act ? TQ_ACT_BYTES : 4;
   const int tile_rows = p.tile_rows ? p.tile_rows : (p.M <= 32 ? 16 : 64);
   *splits = 1;
+  auto result = [&](size_t bytes) { return p.dest ? p.dest : c.arena.take(bytes); };
   if (!grouped && !p.a_rows && !p.bias.ptr && vendor_product(c, p)) {
     if (!p.w2) {
-      *out = c.arena.take((size_t)p.M * p.N * esz);
+      *out = result((size_t)p.M * p.N * esz);
       RUN(c, "vendor product",
           tq_vendor_product(p.a, p.lda, p.w.ptr, *out, p.out_act, p.M, p.N, p.K, c.vendor_ws[side], c.stream));
+      if (!c.dry) ++g_vendor_products;
       return 0;
     }
     const bool behind = (const char*)p.w2 == (const char*)p.w.ptr + (size_t)p.N * p.K * 2;
     if (p.out_act && behind) {
       // f(a w^T) * (a w2^T) with w2 behind w: one product over both matrices into float, some thousand rows at a
       // time, and the gate's activation in a pass of its own
-      *out = c.arena.take((size_t)p.M * p.N * esz);
+      *out = result((size_t)p.M * p.N * esz);
       const int64_t chunk = c.s->vendor_gated_rows > 0 ? c.s->vendor_gated_rows : 4096;
       float* gu = (float*)c.arena.take((size_t)(p.M < chunk ? p.M : chunk) * 2 * p.N * 4);
       for (int64_t r = 0; r < p.M; r += chunk) {
@@ -152,6 +156,7 @@ int product(Ctx& c, const Product& p, void** out, int* splits, int side = 0) {
         RUN(c, "vendor product",
             tq_vendor_product((const char*)p.a + r * p.lda * 2, p.lda, p.w.ptr, gu, 0, rows, 2 * p.N, p.K,
                               c.vendor_ws[side], c.stream));
+        if (!c.dry) ++g_vendor_products;
         if (int rc = gated_act(c, gu, 2 * p.N, (char*)*out + r * p.N * TQ_ACT_BYTES, rows, p.N, p.gate)) return rc;
       }
       return 0;
@@ -160,7 +165,7 @@ int product(Ctx& c, const Product& p, void** out, int* splits, int side = 0) {
 #if defined(TQ_ACT_BF16)
   if (use_mfma(p.w, p.K)) {
     if (p.partial) *splits = tq_gemm_mfma_splits(p.M, p.N, p.K);
-    *out = c.arena.take((size_t)*splits * p.M * p.N * esz);
+    *out = result((size_t)*splits * p.M * p.N * esz);
     RUN(c, "gemm_mfma",
         tq_gemm_mfma(p.a, p.lda, p.a_rows, p.gather, p.w.ptr, p.w2, p.gstride, p.tile_group, p.n_tiles, p.bias.ptr,
                      (int)p.bias.wtype, *out, p.N, p.out_act, p.M, p.N, p.K, tile_rows, *splits, p.gate, c.stream));
@@ -171,7 +176,7 @@ int product(Ctx& c, const Product& p, void** out, int* splits, int side = 0) {
       ((uintptr_t)p.w2 & 15) == 0 && (tile_rows == 16 || tile_rows == 64)) {
     const int runs = tq_gemm_f32_runs(p.M, p.N, p.K, grouped || p.a_rows != nullptr);
     if (p.partial) *splits = runs;
-    *out = c.arena.take((size_t)*splits * p.M * p.N * 4);
+    *out = result((size_t)*splits * p.M * p.N * 4);
     void* scratch = nullptr;
     if (runs > 1 && !p.partial) scratch = c.arena.take((size_t)runs * (p.w2 ? 2 : 1) * p.M * p.N * 4);
     RUN(c, "gemm_f32",
@@ -181,7 +186,7 @@ int product(Ctx& c, const Product& p, void** out, int* splits, int side = 0) {
     return 0;
   }
 #endif
-  *out = c.arena.take((size_t)p.M * p.N * esz);
+  *out = result((size_t)p.M * p.N * esz);
   RUN(c, "gemm",
       tq_gemm_generic(p.a, p.lda, p.a_rows, p.gather, p.w.ptr, p.w2, (int)p.w.wtype, p.gstride, p.tile_group, p.n_tiles,
                       p.bias.ptr, (int)p.bias.wtype, *out, p.N, p.out_act, p.M, p.N, p.K, tile_rows, p.gate, c.stream));
@@ -511,54 +516,12 @@ int walk(Ctx& c, size_t* entry_bytes) {
     void* normed;
     float* normed32;
     if (int rc = norm(c, m.final_norm, x, pending, s.want_rows, (int)s.n_want, &normed, &normed32, false)) return rc;
-    // the vocabulary's product writes the caller's logits; it is a plain product into float
+    // the vocabulary's product: a plain product into float that writes the caller's logits
     Product p;
-    p.a = normed, p.lda = H, p.w = m.lm_head, p.M = (int)s.n_want, p.N = (int)m.vocab, p.K = H;
-    void* out = s.logits;
-    const size_t before = c.arena.used;
-    // the product's result goes straight to s.logits: take nothing from the arena for it
-    struct Direct {
-      Ctx& c;
-      void* keep;
-    };
-    Arena saved = c.arena;
+    p.a = normed, p.lda = H, p.w = m.lm_head, p.M = (int)s.n_want, p.N = (int)m.vocab, p.K = H, p.dest = s.logits;
+    void* got;
     int one;
-    // run the dispatch with an arena whose first take yields the caller's buffer
-    Arena direct;
-    direct.dry = c.dry;
-    direct.base = (char*)s.logits;
-    direct.cap = c.dry ? 0 : (size_t)s.n_want * m.vocab * 4 + 256;
-    // scratch that a product may need beside its result still comes from the entry's half: the result is the first take
-    (void)before;
-    (void)out;
-    c.arena = direct;
-    void* got = nullptr;
-    // products that take scratch after their result (the float path's runs of k) would take it behind the logits:
-    // give the float path its scratch from the half instead
-    int rc = 0;
-#if defined(TQ_ACT_F32)
-    {
-      const bool f32 = p.w.wtype == TQ_F32 && p.K % 4 == 0 && ((uintptr_t)p.w.ptr & 15) == 0;
-      const int runs = f32 ? tq_gemm_f32_runs(p.M, p.N, p.K, 0) : 1;
-      c.arena = saved;
-      if (f32 && runs > 1) {
-        void* scratch = c.arena.take((size_t)runs * p.M * p.N * 4);
-        RUN(c, "gemm_f32",
-            tq_gemm_f32(p.a, p.lda, nullptr, 1, p.w.ptr, nullptr, 0, nullptr, nullptr, nullptr, 0, s.logits, p.N, p.M, p.N,
-                        p.K, p.M <= 32 ? 16 : 64, 0, scratch, 0, c.stream));
-        got = s.logits;
-      } else {
-        saved = c.arena;
-        c.arena = direct;
-        rc = product(c, p, &got, &one);
-      }
-    }
-#else
-    rc = product(c, p, &got, &one);
-#endif
-    if (c.arena.base == direct.base) c.arena = saved;
-    if (rc) return rc;
-    if (!c.dry && got != s.logits) return fail(TQ_ERR_BAD_ARG, "the vocabulary's product did not write the caller's logits");
+    if (int rc = product(c, p, &got, &one)) return rc;
     if (m.logit_softcap > 0) RUN(c, "softcap", tq_softcap(s.logits, (int64_t)s.n_want * m.vocab, (float)m.logit_softcap, c.stream));
   }
   if (c.arena.peak > most) most = c.arena.peak;
@@ -593,6 +556,7 @@ int run(const tq_model_desc* m, const tq_step_desc* s, bool launch, int64_t* byt
   if (s->side_stream)
     if (int rc = events_for_device(r)) return rc;
   g_launches = 0;
+  g_vendor_products = 0;
   return walk(r, &entry_bytes);
 }
 
@@ -611,6 +575,8 @@ int tq_step_forward(const tq_model_desc* model, const tq_step_desc* step) { retu
 const char* tq_engine_last_error(void) { return g_error; }
 
 int64_t tq_engine_last_launches(void) { return g_launches; }
+
+int64_t tq_engine_last_vendor_products(void) { return g_vendor_products; }
 
 void tq_engine_struct_sizes(int64_t* out) {
   out[0] = sizeof(tq_weight), out[1] = sizeof(tq_norm_desc), out[2] = sizeof(tq_attention_desc);

@@ -5,7 +5,7 @@
 // /root/reference/src/engine/tq_transformer.c:2281-3029) over a model structure that its loader filled
 // (/root/reference/include/turboquant/tq_engine.h).  Here the model structure is the set of descriptors below, which
 // say, layer by layer, which part runs with which sizes, constants and weights; a host in any language fills them
-// (the Python package does, from the model's plan and its loaded parameters; quant_main.cpp does, from a folder) and
+// (the Python package does, from the model's plan and its loaded parameters) and
 // hands them to tq_step_forward together with the step's packed tokens.  The executor knows the parts (norm,
 // attention, dense and sparse feed-forward, the pre-norm arrangement) and nothing of any architecture.
 //
@@ -138,6 +138,8 @@ const char* tq_engine_last_error(void);
 void tq_engine_struct_sizes(int64_t* out9);
 // How many kernels the last tq_step_forward of this thread launched (vendor products included).
 int64_t tq_engine_last_launches(void);
+// How many of them were products of the vendor's matrix library.
+int64_t tq_engine_last_vendor_products(void);
 
 #ifdef __cplusplus
 }

@@ -20,6 +20,7 @@ class StepContext:
     # called with (schedule entry, the residual stream behind that entry [T, H] float32, the batch), for whoever wants
     # to look at activations layer by layer (the reference prints them under TQ_DEBUG, tq_transformer.c:2340-2344)
     layer_hook: "object | None" = None
+    native: "object | None" = None      # the model's form for the step executor (engine/native.py), if it has one
 
     def kv(self, entry: int) -> KVView:
         """Keys and values of the schedule entry (or of the entry whose cache it reads)."""

@@ -72,7 +72,7 @@ class DecodeGraph:
         self.fill(slots, starts, tokens)
         e = self.engine
         ctx = StepContext(batch=self.batch(slots, starts), cache=e.cache, act=e.model.act, device=e.device,
-                          side_stream=e.side_stream, capturing=True)
+                          side_stream=e.side_stream, capturing=True, native=e.native)
         torch.cuda.synchronize()
         # Nothing may be destroyed on the device while the stream is capturing: an older graph that the garbage
         # collector happens to find in the middle of the capture would end the process.  So the collector rests

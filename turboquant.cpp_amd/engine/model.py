@@ -104,16 +104,21 @@ class CausalLM:
         return needs
 
     def new_cache(self, max_tokens: int, page_size: int = 64, max_slots: int | None = None,
-                  max_positions: int | None = None) -> PagedCache:
+                  max_positions: int | None = None, window_step: int = 2048) -> PagedCache:
         """``max_positions``: the most positions a sequence may reach, if that is to be fewer than the model allows."""
         limit = self.plan.max_positions if max_positions is None else min(max_positions, self.plan.max_positions)
         return PagedCache(self.cache_needs(), max_tokens, self.act_dtype, self.device, page_size=page_size,
-                          max_slots=max_slots, max_positions=limit)
+                          max_slots=max_slots, max_positions=limit, window_step=window_step)
 
     # ------------------------------------------------------------ forward
     def forward(self, ctx: StepContext) -> torch.Tensor:
         """Runs the step's tokens through the schedule; returns float32 logits [wanted rows, vocab]."""
         b = ctx.batch
+        if ctx.native is not None and ctx.layer_hook is None and ops._PROFILE is None:
+            # one call into the library's step executor issues every launch of the step; what follows here is the
+            # same step part by part, for models with parts that the executor does not know, for whoever looks at
+            # the layers (layer_hook) and for the profile, which puts an event behind every launch
+            return ctx.native.forward(ctx)
         x = ops.embed(b.tokens, self.embedding, self.act, scale=self.plan.embedding_scale)
         pending = None
         for entry, e in enumerate(self.schedule):

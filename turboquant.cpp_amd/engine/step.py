@@ -17,6 +17,7 @@ from .batch import pack_step
 from .context import StepContext
 from .graph import DecodeGraphs
 from .model import CausalLM
+from .native import NativeModel
 
 
 class StepError(ValueError):
@@ -28,10 +29,13 @@ class Engine:
     each sequence rounded up to whole pages of ``page_size``."""
 
     def __init__(self, model: CausalLM, max_tokens: int, page_size: int = 64, max_slots: int | None = None,
-                 use_graphs: bool = True, max_positions: int | None = None):
-        """``max_positions``: the most positions one sequence may reach (default and upper bound: the model's)."""
+                 use_graphs: bool = True, max_positions: int | None = None, window_step: int = 2048):
+        """``max_positions``: the most positions one sequence may reach (default and upper bound: the model's).
+        ``window_step``: layers that keep a window have pages for their windows and for this many new positions per
+        sequence; a step that brings a sequence more is run in cuts of that length."""
         self.model = model
-        self.cache = model.new_cache(max_tokens, page_size=page_size, max_slots=max_slots, max_positions=max_positions)
+        self.cache = model.new_cache(max_tokens, page_size=page_size, max_slots=max_slots, max_positions=max_positions,
+                                     window_step=window_step)
         self.device = model.device
         self.vocab_size = model.plan.vocab_size
         # decode steps are replayed as HIP graphs where a GPU runs them
@@ -40,6 +44,8 @@ class Engine:
         # (which shapes of step are replayed is the parts' word, asked shape by shape: Part.replayable)
         self.graphs = DecodeGraphs(self) if use_graphs and on_gpu else None
         self.layer_hook = None      # see StepContext.layer_hook; while it is set, steps run eagerly
+        # the model and this cache as the library's step executor takes them (None: steps run part by part from here)
+        self.native = NativeModel.build(model, self.cache) if on_gpu else None
 
     # ------------------------------------------------------------ sequences
     def open(self, n: int = 1) -> list[int]:
@@ -86,6 +92,9 @@ class Engine:
             bad = [w for w in want if not 0 <= w < len(toks)]
             if bad:
                 raise StepError(f"wanted place {bad[0]} is outside the {len(toks)} tokens that sequence {i} brings")
+        limit = self.cache.step_limit
+        if limit is not None and max(len(t) for t in token_lists) > limit:
+            return self._step_in_cuts(slots, token_lists, wants, limit)
         starts = self._reserve(slots, [len(t) for t in token_lists])
         try:
             logits = None
@@ -104,6 +113,33 @@ class Engine:
         for slot in slots:
             self.cache.commit(slot)
         return logits
+
+    def _step_in_cuts(self, slots, token_lists, wants, limit: int) -> torch.Tensor:
+        """A step whose sequences bring more tokens than a group with a window has room for at once: cuts of
+        ``limit`` tokens per sequence, one after the other (the logits at a position do not depend on how its
+        sequence was cut).  Whether the whole step has room is looked at before the first cut runs."""
+        self.cache.room_for(slots, [len(t) for t in token_lists])
+        pieces, where = [], {}          # (sequence, place in its wants) -> (cut, row of that cut's logits)
+        for cut in range(-(-max(len(t) for t in token_lists) // limit)):
+            lo = cut * limit
+            live = [i for i, t in enumerate(token_lists) if len(t) > lo]
+            cut_wants, row = [], 0
+            for i in live:
+                mine = [(j, w - lo) for j, w in enumerate(wants[i]) if lo <= w < lo + limit]
+                for j, _ in mine:
+                    where[(i, j)] = (cut, row)
+                    row += 1
+                cut_wants.append([w for _, w in mine])
+            pieces.append(self.step([slots[i] for i in live], [token_lists[i][lo:lo + limit] for i in live], cut_wants))
+        order = [where[(i, j)] for i in range(len(slots)) for j in range(len(wants[i]))]
+        if not order:
+            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
+        offsets, total = [], 0
+        for p in pieces:
+            offsets.append(total)
+            total += p.shape[0]
+        rows = torch.tensor([offsets[c] + r for c, r in order], dtype=torch.int64, device=self.device)
+        return torch.cat(pieces)[rows]
 
     def step_from_device(self, slots: list[int], tokens: torch.Tensor) -> torch.Tensor:
         """A decode step whose tokens are already on the device: ``tokens`` int32 [len(slots)], one for each
@@ -152,6 +188,6 @@ class Engine:
     def _eager(self, batch) -> torch.Tensor:
         # a second stream for what does not depend on the main line (the parts decide what they put there)
         ctx = StepContext(batch=batch, cache=self.cache, act=self.model.act, device=self.device,
-                          side_stream=self.side_stream, layer_hook=self.layer_hook)
+                          side_stream=self.side_stream, layer_hook=self.layer_hook, native=self.native)
         with ops.own_products(max(batch.n_new) == 1):      # a decode step runs the kernels that its replay runs
             return self.model.forward(ctx)

@@ -12,6 +12,8 @@ from __future__ import annotations
 
 import math
 
+import torch
+
 from ..config.plan import PartSpec
 from ..csrc import ops
 from .base import CacheNeed, ParamSpec, Part, build_part, register_part
@@ -67,6 +69,18 @@ class GroupedQueryAttention(Part):
 
     def state_need(self):
         return None
+
+    def native(self):
+        from ..csrc import host_api
+        if self.qk_norm_eps is not None:        # the executor has no form with a norm of the heads
+            return None
+        table = self.position.table(self.qkv_weight.device)
+        if table.dtype != torch.float32 or not table.is_contiguous() or table.numel() * 2 != self.position.rotary_dim:
+            return None
+        return host_api.AttentionDesc(self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim, self.window or 0,
+                                      self.position.pairing_code, self.position.rotary_dim, self.scale,
+                                      host_api.weight(self.qkv_weight), host_api.weight(self.qkv_bias),
+                                      host_api.weight(self.out_weight), host_api.weight(self.out_bias), table.data_ptr())
 
     def forward(self, normed, ctx, entry):
         b, kv = ctx.batch, ctx.kv(entry)

@@ -92,6 +92,12 @@ class Part:
     def prepare(self, device, act: str) -> None:
         """Called once after the parameters are on the device."""
 
+    def native(self):
+        """The part's description for the step executor (a structure of ``csrc.host_api``: its sizes, constants and the
+        addresses of its parameters), or None if the executor has no form of this part.  A model whose layers all have
+        one is stepped by one call into the executor; any other is stepped part by part through ``forward``."""
+        return None
+
 
 _REGISTRIES: dict[str, dict[str, Callable[..., Part]]] = {
     "norm": {}, "mixer": {}, "ffn": {}, "position": {}, "block": {},

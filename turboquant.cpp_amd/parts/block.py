@@ -28,6 +28,20 @@ class PreNormBlock(Part):
     def state_need(self):
         return self.mixer.state_need()
 
+    def native(self):
+        from ..csrc import host_api
+        norm1, mixer, norm2, ffn = (p.native() for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn))
+        if not (isinstance(norm1, host_api.NormDesc) and isinstance(mixer, host_api.AttentionDesc)
+                and isinstance(norm2, host_api.NormDesc) and isinstance(ffn, (host_api.DenseFfnDesc, host_api.MoeFfnDesc))):
+            return None
+        layer = host_api.LayerDesc()
+        layer.mixer_norm, layer.attention, layer.ffn_norm = norm1, mixer, norm2
+        if isinstance(ffn, host_api.DenseFfnDesc):
+            layer.ffn_kind, layer.dense = host_api.FFN_DENSE, ffn
+        else:
+            layer.ffn_kind, layer.moe = host_api.FFN_MOE, ffn
+        return layer
+
     def forward(self, x, pending, ctx, entry):
         normed, _ = self.mixer_norm.forward(x, pending, ctx)
         pending = self.mixer.forward(normed, ctx, entry)

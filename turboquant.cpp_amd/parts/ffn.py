@@ -40,6 +40,11 @@ class DenseSwiGLU(Part):
         # gate and up side by side: a long prompt's pair may then go out as one product over both
         self.gate, self.up = ops.side_by_side(self.gate, self.up)
 
+    def native(self):
+        from ..csrc import host_api
+        return host_api.DenseFfnDesc(self.hidden_size, self.inner_size, ops.GATES[self.activation], host_api.weight(self.gate),
+                                     host_api.weight(self.up), host_api.weight(self.down))
+
     def forward(self, normed, normed32, ctx):
         h = ops.gemm(normed, self.gate, ctx.act, w2=self.up, out_act=True, activation=self.activation)
         return ops.gemm(h, self.down, ctx.act, partial_sums=True)
@@ -78,6 +83,14 @@ class SparseMoE(Part):
     def prepare(self, device, act):
         if self.shared_size > 0:     # as in the dense part; the experts' products never leave this library's kernels
             self.shared_gate, self.shared_up = ops.side_by_side(self.shared_gate, self.shared_up)
+
+    def native(self):
+        from ..csrc import host_api
+        w = host_api.weight
+        return host_api.MoeFfnDesc(self.hidden_size, self.num_experts, self.top_k, self.expert_size, self.shared_size,
+                                   int(self.renormalize), ops.GATES[self.activation], w(self.router),
+                                   w(self.shared_scale if self.shared_gated else None), w(self.expert_gate), w(self.expert_up),
+                                   w(self.expert_down), w(self.shared_gate), w(self.shared_up), w(self.shared_down))
 
     def forward(self, normed, normed32, ctx):
         T = normed.shape[0]

@@ -19,6 +19,10 @@ class RMSNorm(Part):
     def param_specs(self):
         return {"weight": ParamSpec((self.size,), role="scale")}
 
+    def native(self):
+        from ..csrc import host_api
+        return host_api.NormDesc(host_api.weight(self.weight), self.eps)
+
     def forward(self, x, delta, ctx, rows=None, want_act=True, want_f32=False):
         return ops.add_rmsnorm(x, delta, self.weight, self.eps, ctx.act, rows=rows, want_act=want_act,
                                want_f32=want_f32)
