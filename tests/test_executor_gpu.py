@@ -162,3 +162,62 @@ def test_a_model_with_a_part_that_the_executor_does_not_know_runs_part_by_part(m
         outs.append(e.step(slot, [p], [list(range(20))]))
         e.close(slot)
     assert torch.equal(outs[0], outs[1])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_the_host_program_without_python_generates_what_the_library_does(name, act, tmp_path):
+    """``bin/quant_c``: the host program in C++ (csrc/host/quant_main.cpp) reads the plan that the package writes from
+    config.json, loads model.safetensors by tensor name, keeps a cache of its own and drives the step executor; its
+    greedy tokens are those of the Python entry point, which runs the same kernels (unequal prompts, of which the
+    shorter ones end earlier; B stops on its end tokens 7 and 11 if they come)."""
+    import os
+    import subprocess
+    import sys
+    from test_engine_gpu import ROOT
+    from turboquant_cpp_amd import Model
+    from turboquant_cpp_amd.engine.model import write_random_model_dir
+    cfg, init = TINY[name]
+    d = write_random_model_dir(str(tmp_path / "m"), cfg, init["seed"], SHARP, init["norm_std"], act)
+    prompts = prompts_for(name, [5, 70, 1, 23], seed=64)
+    text = ";".join(",".join(str(t) for t in p) for p in prompts)
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "quant_c"), d, "-p", text, "-n", "9", "--dtype", act],
+                         capture_output=True, text=True, timeout=600)
+    assert run.returncode == 0, run.stderr[-2000:]
+    got = []
+    for line in run.stdout.splitlines():
+        head, reason = line.rsplit("(", 1)
+        got.append(([int(t) for t in head.split("]")[1].split()], reason.rstrip(")")))
+    with Model(d, dtype=act, temperature=0.0, rep_penalty=1.0, max_tokens=9, max_batch=4) as m:
+        want = m.generate_detailed(prompts, loop_detection=False)
+    assert got == [(r.tokens, r.finish_reason) for r in want]
+    # a folder that does not fit the model is refused with the list of what is missing
+    os.rename(os.path.join(d, "model.safetensors"), os.path.join(d, "kept"))
+    from turboquant_cpp_amd.weights import SafetensorsFolder, write_safetensors
+    with SafetensorsFolder(d, files=[os.path.join(d, "kept")]) as f:
+        tensors = {n: f.read(n).clone() for n in f.names() if not n.endswith("model.norm.weight")}
+    write_safetensors(os.path.join(d, "model.safetensors"), tensors)
+    bad = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "quant_c"), d, "-p", "1,2", "--dtype", act],
+                         capture_output=True, text=True, timeout=600)
+    assert bad.returncode != 0 and "missing tensors (1): model.norm.weight" in bad.stderr
+
+
+def test_the_plan_file_names_every_part_and_tensor():
+    """No GPU: the plan that a host without Python reads lists every layer's parts with their constants, every
+    parameter with the checkpoint tensors behind it, the table of rotation angles and the schedule."""
+    from turboquant_cpp_amd.engine.model import model_from_config
+    from turboquant_cpp_amd.engine.plan_file import plan_text
+    model = model_from_config(TINY["B"][0], "bfloat16")
+    text = plan_text(model)
+    lines = text.splitlines()
+    assert lines[0] == "tqplan 1" and lines[1].startswith("model Qwen2MoeForCausalLM act=bfloat16 vocab=384 hidden=144 n_layers=3")
+    assert "stop 2 7 11" in lines
+    assert [l for l in lines if l.startswith("entry ")] == [f"entry {i} layer={i} cache_of=-1" for i in range(3)]
+    assert sum(l.startswith("part ") and " moe_swiglu " in l for l in lines) == 1
+    assert any(l.startswith("part 1 mixer gqa_attention") and "window=24" in l for l in lines)
+    assert any(l.startswith("part 0 mixer gqa_attention") and "window=" not in l for l in lines)
+    named = {w for l in lines if l.startswith("param ") for w in l.split() if w.startswith("model.") or w.startswith("lm_head.")}
+    assert named == set(model.tensor_table())
+    table = [l for l in lines if l.startswith("table 0 mixer inv_freq 12 ")][0].split()[5:]
+    assert len(table) == 12 and table[0] == "3f800000"

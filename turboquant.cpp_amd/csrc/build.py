@@ -159,8 +159,53 @@ def build(dtype: str, force: bool = False, verbose: bool = True) -> str:
     return target
 
 
+RUNNER_SOURCES = ["host/quant_main.cpp", "host/engine.h"]
+
+
+def runner_name() -> str:
+    h = hashlib.sha256()
+    for name in RUNNER_SOURCES:
+        with open(os.path.join(CSRC, name), "rb") as f:
+            h.update(f.read())
+    return f"tq_run-{h.hexdigest()[:12]}"
+
+
+def find_runner() -> str | None:
+    for d in _build_dirs():
+        p = os.path.join(d, runner_name())
+        if os.path.isfile(p):
+            return p
+    return None
+
+
+def build_runner(force: bool = False, verbose: bool = True) -> str:
+    """Compiles the host program without Python (host/quant_main.cpp) and returns its path.  It loads a kernel
+    library at run time and is linked against the HIP runtime only."""
+    if not force:
+        found = find_runner()
+        if found:
+            return found
+    hipcc = _hipcc()
+    target = os.path.join(_writable_dir(), runner_name())
+    tmp = target + f".tmp{os.getpid()}"
+    if verbose:
+        print(f"[turboquant] compiling the host program into {target}", file=sys.stderr, flush=True)
+    run = subprocess.run([hipcc, "-O2", "-std=c++17", os.path.join(CSRC, "host", "quant_main.cpp"), "-ldl", "-o", tmp],
+                         stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if run.returncode != 0:
+        raise BuildError(f"hipcc failed on host/quant_main.cpp:\n{run.stdout}")
+    os.replace(tmp, target)
+    for old in os.listdir(os.path.dirname(target)):
+        if old.startswith("tq_run-") and old != os.path.basename(target) and ".tmp" not in old:
+            try:
+                os.remove(os.path.join(os.path.dirname(target), old))
+            except OSError:
+                pass
+    return target
+
+
 def build_all(force: bool = True, verbose: bool = True) -> list[str]:
-    return [build(d, force=force, verbose=verbose) for d in SOURCES]
+    return [build(d, force=force, verbose=verbose) for d in SOURCES] + [build_runner(force=force, verbose=verbose)]
 
 
 if __name__ == "__main__":

@@ -28,8 +28,6 @@ struct MfmaGemmArgs {
   int64_t split_stride;
   int gate;                 // activation of the gated pair
   int group_ratio;          // tile kernel: row tiles per entry of tile_group and unit of n_tiles (0 or 1: one)
-  int pair64;               // tile kernel of 128 rows over a row order in units of 64: a workgroup takes two units of
-                            // one expert, or the expert's last one alone
 };
 
 // For bytes that are read once (a matrix streamed past a few rows): a load that tells the caches so.  Measured on

@@ -320,47 +320,6 @@ __global__ __launch_bounds__(512) void qkv_rope_write_kernel(MfmaGemmArgs g, Rop
 // 128 bytes per clock; XOR with bits 0..2 at 107, no swizzle at 31.
 __device__ __forceinline__ int swz(int row, int chunk) { return row * TBK + ((chunk ^ ((row >> 1) & 7)) << 3); }
 
-// Which tile a workgroup takes (false: none).  Workgroups are dealt to the chip's 8 dies in turn (id % 8), and each die
-// has its own L2: so the tiles are numbered such that one die gets a contiguous run of them.  One matrix: a
-// run goes through bands of 8 row tiles, down a band's column of row tiles first, so that workgroups that run
-// at the same time on a die share their tiles of `a` and of `w` in that die's L2.  A matrix per expert: a run
-// goes expert by expert, so that an expert's matrix is read by one die (by two where a run ends), and within an
-// expert column by column with the expert's row tiles side by side (measured against row tile by row tile: 6 to
-// 12 % faster, the more the more row tiles an expert has); only the row tiles in use are dealt.
-__device__ __forceinline__ bool tile_of_workgroup(const MfmaGemmArgs& g, int& tile_m, int& tile_n, int* run_end = nullptr,
-                                                  int* run_begin = nullptr) {
-  // an entry of tile_group (and a unit of n_tiles) stands for `ratio` row tiles of this kernel where the row
-  // order was padded to a multiple of the tile's height
-  const int ratio = g.group_ratio > 1 ? g.group_ratio : 1;
-  const int gx = g.tile_group && g.n_tiles ? min(g.n_tiles[0] * ratio, (int)gridDim.x) : (int)gridDim.x;
-  const int gy = gridDim.y, total = gx * gy;
-  const int id = blockIdx.y * gridDim.x + blockIdx.x;
-  const int die = id % 8, q = total / 8, rem = total % 8;
-  if (id / 8 >= q + (die < rem ? 1 : 0)) return false;
-  const int logical = die * q + min(die, rem) + id / 8;
-  if (g.tile_group) {
-    // the expert whose row tiles [lo, hi) hold row tile logical / gy; within it column by column, the expert's
-    // row tiles of a column one after the other, so that they read that column's rows of w at the same time
-    const int u = logical / gy / ratio, e = g.tile_group[u], gu = gx / ratio;
-    int lo = u, hi = u + 1;
-    while (lo > 0 && g.tile_group[lo - 1] == e) --lo;
-    while (hi < gu && g.tile_group[hi] == e) ++hi;
-    lo *= ratio;
-    hi *= ratio;
-    const int local = logical - lo * gy, n_e = hi - lo;
-    tile_n = local / n_e;
-    tile_m = lo + local % n_e;
-    if (run_end) *run_end = hi;
-    if (run_begin) *run_begin = lo;
-  } else {
-    const int band = logical / (8 * gy), in_band = logical % (8 * gy);
-    const int bh = min(8, gx - band * 8);
-    tile_m = band * 8 + in_band % bh;
-    tile_n = in_band / bh;
-  }
-  return true;
-}
-
 template <int BM, int WM, int WN, bool DUAL, bool OUT_ACT, int BN = TBN>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g) {
   constexpr int NT = 64 * WM * WN;
@@ -375,24 +334,51 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g)
   bf16_t* As = (bf16_t*)smem;
   bf16_t* Ws = As + BM * TBK;
   bf16_t* Vs = Ws + BN * TBK;
-  int tile_m, tile_n, run_end = 0, run_begin = 0;
-  if (!tile_of_workgroup(g, tile_m, tile_n, &run_end, &run_begin)) return;
+  // Which tile this workgroup takes.  Workgroups are dealt to the chip's 8 dies in turn (id % 8), and each die
+  // has its own L2: so the tiles are numbered such that one die gets a contiguous run of them.  One matrix: a
+  // run goes through bands of 8 row tiles, down a band's column of row tiles first, so that workgroups that run
+  // at the same time on a die share their tiles of `a` and of `w` in that die's L2.  A matrix per expert: a run
+  // goes expert by expert, so that an expert's matrix is read by one die (by two where a run ends), and within an
+  // expert column by column with the expert's row tiles side by side (measured against row tile by row tile: 6 to
+  // 12 % faster, the more the more row tiles an expert has); only the row tiles in use are dealt.
+  int tile_m, tile_n;
+  {
+    // an entry of tile_group (and a unit of n_tiles) stands for `ratio` row tiles of this kernel where the row
+    // order was padded to a multiple of the tile's height
+    const int ratio = g.group_ratio > 1 ? g.group_ratio : 1;
+    const int gx = g.tile_group && g.n_tiles ? min(g.n_tiles[0] * ratio, (int)gridDim.x) : (int)gridDim.x;
+    const int gy = gridDim.y, total = gx * gy;
+    const int id = blockIdx.y * gridDim.x + blockIdx.x;
+    const int die = id % 8, q = total / 8, rem = total % 8;
+    if (id / 8 >= q + (die < rem ? 1 : 0)) return;
+    const int logical = die * q + min(die, rem) + id / 8;
+    if (g.tile_group) {
+      // the expert whose row tiles [lo, hi) hold row tile logical / gy; within it column by column, the expert's
+      // row tiles of a column one after the other, so that they read that column's rows of w at the same time
+      const int u = logical / gy / ratio, e = g.tile_group[u], gu = gx / ratio;
+      int lo = u, hi = u + 1;
+      while (lo > 0 && g.tile_group[lo - 1] == e) --lo;
+      while (hi < gu && g.tile_group[hi] == e) ++hi;
+      lo *= ratio;
+      hi *= ratio;
+      const int local = logical - lo * gy, n_e = hi - lo;
+      tile_n = local / n_e;
+      tile_m = lo + local % n_e;
+    } else {
+      const int band = logical / (8 * gy), in_band = logical % (8 * gy);
+      const int bh = min(8, gx - band * 8);
+      tile_m = band * 8 + in_band % bh;
+      tile_n = in_band / bh;
+    }
+  }
   const int group = g.tile_group ? g.tile_group[tile_m / (g.group_ratio > 1 ? g.group_ratio : 1)] : 0;
   const bf16_t* w = g.w + (size_t)group * g.group_stride;
   const bf16_t* w2 = DUAL ? g.w2 + (size_t)group * g.group_stride : nullptr;
-  // Units of 64 rows taken two at a time (pair64, BM = 128): the workgroup of an expert's first, third, ... unit takes
-  // that unit and the next one of the same expert, the others have nothing to do; an expert's last unit may stand
-  // alone, and then the waves of the tile's lower half only fetch.  So an expert's matrices pass once per 128 of
-  // its rows without any expert's rows being padded to more than 64.
-  const bool pairs = BM == 128 && g.pair64 && g.tile_group;
-  if (pairs && ((tile_m - run_begin) & 1)) return;
-  const int rows_here = pairs && tile_m + 1 >= run_end ? 64 : BM;
-  const int m0 = pairs ? tile_m * 64 : tile_m * BM, n0 = tile_n * BN;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
   // an expert's rows stand at the head of its units: a tile that begins with a row of padding holds nothing else
   if (g.tile_group && g.a_rows && g.a_rows[min(m0, g.M - 1)] < 0) return;
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int wm = wave / WN, wn = wave % WN;
-  const bool active = wm * (MI * 32) < rows_here;     // whether this wave's rows exist
   // this workgroup's run of k: k_lo .. k_lo + Kl (all of k unless the product is split), and where its sums go
   const int k_lo = blockIdx.z * g.k_per;
   const int Kl = min(g.K, k_lo + g.k_per) - k_lo;
@@ -410,8 +396,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g)
 #pragma unroll
   for (int i = 0; i < A_CH; ++i) {
     const int idx = tid + i * NT, row = idx / 8, ch = idx % 8;
-    // (rows of a half that is not there read the other half's rows once more: nothing new leaves the caches)
-    const int m = min(m0 + (row < rows_here ? row : row - 64), g.M - 1);
+    const int m = min(m0 + row, g.M - 1);
     int src = m;
     if (g.a_rows && g.a_gather) src = max(g.a_rows[m], 0);
     a_src[i] = g.a + (size_t)src * g.lda + k_lo + ch * 8;
@@ -487,7 +472,6 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g)
     const bf16_t* Ac = As + cur;
     const bf16_t* Wc = Ws + cur;
     const bf16_t* Vc = Vs + cur;
-    if (active)
 #pragma unroll
     for (int j = 0; j < TBK / 16; ++j) {
       bf16x8 af[MI], wf[NI], vf[DUAL ? NI : 1];
@@ -515,7 +499,6 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g)
 #undef TQ_FETCH
 #undef TQ_STAGE
 
-  if (!active) return;
 #pragma unroll
   for (int ni = 0; ni < NI; ++ni) {
     const int n = n0 + wn * (NI * 32) + ni * 32 + lr;
@@ -526,215 +509,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int m = m0 + wm * (MI * 32) + mi * 32 + 8 * (v / 4) + 4 * lc + (v % 4);
-        if (m >= g.M || m >= m0 + rows_here) continue;
+        if (m >= g.M) continue;
         if (g.a_rows && g.a_rows[m] < 0) continue;
         float o = acc[mi][ni][v] + b;
         if (DUAL) o = gate_fn(o, g.gate) * acc2[mi][ni][v];
-        store_out<OUT_ACT>(g, m, n, o);
-      }
-  }
-}
-
-// ------------------------------------------------------------------------------------------ rows in LDS, matrices past them
-// A product over experts in a long prompt: tiles of 64 rows by 16 * NT * 4 columns by four waves.  The tile of `a`
-// (64 rows x 64 of k) goes through LDS as in the kernel above, but the matrices do not: a wave owns NT tiles of 16
-// columns (of w, and of w2 in a gated pair) and streams their rows from memory straight into the operand registers
-// of v_mfma_f32_16x16x32_bf16, by whole lines with the exchange between pairs of lanes, two steps of k ahead of the
-// products.  No byte of a matrix is written to or read from LDS, and what a wave reads of `a` there (a kilobyte per
-// 16 rows and 32 of k) serves NT (2 NT in a gated pair) products: a quarter of a kilobyte per product where the
-// kernel above, whose waves own 32 x 32 outputs, reads one and a half.  grid as for gemm_tile_kernel with BM = 64.
-#define TQ_RS_BM 64
-template <int NT, bool DUAL, bool OUT_ACT>
-__global__ __launch_bounds__(256, 2) void gemm_rowstream_kernel(MfmaGemmArgs g) {
-  constexpr int MT = TQ_RS_BM / 16, BN = 16 * NT * 4, D = DUAL ? 2 : 1;
-  __shared__ __attribute__((aligned(16))) bf16_t As[3][TQ_RS_BM * TBK];
-  int tile_m, tile_n;
-  if (!tile_of_workgroup(g, tile_m, tile_n)) return;
-  const int group = g.tile_group ? g.tile_group[tile_m / (g.group_ratio > 1 ? g.group_ratio : 1)] : 0;
-  const bf16_t* w = g.w + (size_t)group * g.group_stride;
-  const bf16_t* w2 = DUAL ? g.w2 + (size_t)group * g.group_stride : nullptr;
-  const int m0 = tile_m * TQ_RS_BM, n0 = tile_n * BN;
-  if (g.tile_group && g.a_rows && g.a_rows[min(m0, g.M - 1)] < 0) return;     // a tile of padding only
-  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
-  const int r = lane % 16, c4 = lane / 16;
-  const int K = g.K, NC = (K + TBK - 1) / TBK;
-
-  // what this thread stages of the tile of `a`: two chunks of 16 bytes per step of 64 of k
-  const bf16_t* a_src[2];
-  int a_dst[2];
-#pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int idx = tid + i * 256, row = idx / 8, ch = idx % 8;
-    const int m = min(m0 + row, g.M - 1);
-    int src = m;
-    if (g.a_rows && g.a_gather) src = max(g.a_rows[m], 0);
-    a_src[i] = g.a + (size_t)src * g.lda + ch * 8;
-    a_dst[i] = swz(row, ch);
-  }
-  const int a_ch = tid % 8;
-  // what this lane fetches of the matrices: of each of the wave's column tiles, chunk q of rows r % 8 and 8 + r % 8
-  const int q = c4 + 4 * (r / 8);
-  const bf16_t *w_lo[NT], *w_hi[NT], *v_lo[DUAL ? NT : 1], *v_hi[DUAL ? NT : 1];
-#pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    const int n_a = n0 + (wave * NT + t) * 16 + r % 8, n_b = n_a + 8;
-    // columns past the end read row 0 instead: what they produce is never stored
-    w_lo[t] = w + (size_t)(n_a < g.N ? n_a : 0) * K + q * 8;
-    w_hi[t] = w + (size_t)(n_b < g.N ? n_b : 0) * K + q * 8;
-    if (DUAL) {
-      v_lo[t] = w2 + (size_t)(n_a < g.N ? n_a : 0) * K + q * 8;
-      v_hi[t] = w2 + (size_t)(n_b < g.N ? n_b : 0) * K + q * 8;
-    }
-  }
-  f32x4 acc[NT][MT], acc2[DUAL ? NT : 1][DUAL ? MT : 1];
-#pragma unroll
-  for (int t = 0; t < NT; ++t)
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      acc[t][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-      if (DUAL) acc2[t][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-    }
-  const u32x4 zero = {0u, 0u, 0u, 0u};
-  u32x4 pa[2];
-  u32x4 wq[3][NT][2], vq[DUAL ? 3 : 1][DUAL ? NT : 1][2];
-  // (macros, so that the register arrays are only ever indexed by constants)
-#define TQ_RS_FETCH_A(c)                                                                                   \
-  do {                                                                                                     \
-    const int k__ = (c) * TBK;                                                                             \
-    const bool ok__ = k__ + a_ch * 8 < K;                                                                  \
-    _Pragma("unroll") for (int i = 0; i < 2; ++i)                                                          \
-        pa[i] = ok__ ? *reinterpret_cast<const u32x4*>(a_src[i] + k__) : zero;                             \
-  } while (0)
-#define TQ_RS_STAGE_A(buf)                                                                                 \
-  do {                                                                                                     \
-    _Pragma("unroll") for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4*>(&As[buf][a_dst[i]]) = pa[i];   \
-  } while (0)
-#define TQ_RS_FETCH_W(c, set)                                                                              \
-  do {                                                                                                     \
-    const int k__ = (c) * TBK;                                                                             \
-    const bool ok__ = k__ + q * 8 < K;                                                                     \
-    _Pragma("unroll") for (int t = 0; t < NT; ++t) {                                                       \
-      wq[set][t][0] = ok__ ? *reinterpret_cast<const u32x4*>(w_lo[t] + k__) : zero;                        \
-      wq[set][t][1] = ok__ ? *reinterpret_cast<const u32x4*>(w_hi[t] + k__) : zero;                        \
-      if (DUAL) {                                                                                          \
-        vq[set][t][0] = ok__ ? *reinterpret_cast<const u32x4*>(v_lo[t] + k__) : zero;                      \
-        vq[set][t][1] = ok__ ? *reinterpret_cast<const u32x4*>(v_hi[t] + k__) : zero;                      \
-      }                                                                                                    \
-    }                                                                                                      \
-  } while (0)
-  // the same fetches without a condition, for steps that lie wholly inside k: conditions around loads make the
-  // compiler wait for everything in flight where the branches meet, and the two steps of lead would be lost
-#define TQ_RS_FETCH_A_IN(c)                                                                                \
-  do {                                                                                                     \
-    _Pragma("unroll") for (int i = 0; i < 2; ++i)                                                          \
-        pa[i] = *reinterpret_cast<const u32x4*>(a_src[i] + (c) * TBK);                                     \
-  } while (0)
-#define TQ_RS_FETCH_W_IN(c, set)                                                                           \
-  do {                                                                                                     \
-    const int k__ = (c) * TBK;                                                                             \
-    _Pragma("unroll") for (int t = 0; t < NT; ++t) {                                                       \
-      wq[set][t][0] = *reinterpret_cast<const u32x4*>(w_lo[t] + k__);                                      \
-      wq[set][t][1] = *reinterpret_cast<const u32x4*>(w_hi[t] + k__);                                      \
-      if (DUAL) {                                                                                          \
-        vq[set][t][0] = *reinterpret_cast<const u32x4*>(v_lo[t] + k__);                                    \
-        vq[set][t][1] = *reinterpret_cast<const u32x4*>(v_hi[t] + k__);                                    \
-      }                                                                                                    \
-    }                                                                                                      \
-  } while (0)
-  // the products of step c out of register set s and LDS buffer s
-#define TQ_RS_MULTIPLY(s)                                                                                  \
-  do {                                                                                                     \
-    _Pragma("unroll") for (int t = 0; t < NT; ++t) {                                                       \
-      to_own_row(wq[s][t][0], wq[s][t][1]);                                                                \
-      if (DUAL) to_own_row(vq[s][t][0], vq[s][t][1]);                                                      \
-    }                                                                                                      \
-    _Pragma("unroll") for (int kb = 0; kb < 2; ++kb) {                                                     \
-      bf16x8 af[MT];                                                                                       \
-      _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                                    \
-          af[mt] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&As[s][swz(mt * 16 + r, kb * 4 + c4)])); \
-      _Pragma("unroll") for (int t = 0; t < NT; ++t) {                                                     \
-        const bf16x8 wf = __builtin_bit_cast(bf16x8, wq[s][t][kb]);                                        \
-        _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                                  \
-            acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mt], wf, acc[t][mt], 0, 0, 0);         \
-        if (DUAL) {                                                                                        \
-          const bf16x8 vf = __builtin_bit_cast(bf16x8, vq[s][t][kb]);                                      \
-          _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                                \
-              acc2[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mt], vf, acc2[t][mt], 0, 0, 0);     \
-        }                                                                                                  \
-      }                                                                                                    \
-    }                                                                                                      \
-  } while (0)
-  int c0 = 0;
-  if ((c0 + 5) * TBK <= K) {
-    // Loads in the order in which the loop below leaves them behind (the matrices' rows of step c, the tile of `a` of
-    // step c + 1, the matrices' rows of step c + 1), so that the loop's first wait, for the tile of `a`, leaves the
-    // rows of step c + 1 on their way as every later one does.
-    TQ_RS_FETCH_A_IN(0);
-    TQ_RS_STAGE_A(0);
-    TQ_RS_FETCH_W_IN(0, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    TQ_RS_FETCH_A_IN(1);
-    __builtin_amdgcn_sched_barrier(0);
-    TQ_RS_FETCH_W_IN(1, 1);
-    __syncthreads();
-    // three steps at a time while all that they fetch (up to step c0 + 4) lies wholly inside k
-    for (; (c0 + 5) * TBK <= K; c0 += 3) {
-#pragma unroll
-      for (int s = 0; s < 3; ++s) {
-        TQ_RS_STAGE_A((s + 1) % 3);
-        __builtin_amdgcn_sched_barrier(0);
-        TQ_RS_FETCH_A_IN(c0 + s + 2);
-        __builtin_amdgcn_sched_barrier(0);
-        TQ_RS_FETCH_W_IN(c0 + s + 2, (s + 2) % 3);
-        __builtin_amdgcn_sched_barrier(0);
-        TQ_RS_MULTIPLY(s);
-        __syncthreads();
-      }
-    }
-  } else {
-    TQ_RS_FETCH_A(0);
-    TQ_RS_FETCH_W(0, 0);
-    if (NC > 1) TQ_RS_FETCH_W(1, 1);
-    TQ_RS_STAGE_A(0);
-    if (NC > 1) TQ_RS_FETCH_A(1);
-    __syncthreads();
-  }
-  for (; c0 < NC; c0 += 3) {
-#pragma unroll
-    for (int s = 0; s < 3; ++s) {
-      const int c = c0 + s;
-      if (c < NC) {        // (the same for every thread of the workgroup)
-        if (c + 1 < NC) TQ_RS_STAGE_A((s + 1) % 3);
-        if (c + 2 < NC) {
-          TQ_RS_FETCH_A(c + 2);
-          TQ_RS_FETCH_W(c + 2, (s + 2) % 3);
-        }
-        TQ_RS_MULTIPLY(s);
-        __syncthreads();
-      }
-    }
-  }
-#undef TQ_RS_FETCH_A_IN
-#undef TQ_RS_FETCH_W_IN
-#undef TQ_RS_MULTIPLY
-#undef TQ_RS_FETCH_A
-#undef TQ_RS_STAGE_A
-#undef TQ_RS_FETCH_W
-  // a lane holds column l % 16 and rows 4 * (l / 16) + v of each tile of 16 x 16
-#pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    const int n = n0 + (wave * NT + t) * 16 + r;
-    if (n >= g.N) continue;
-    const float b = bias_at(g, n);
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        const int m = m0 + mt * 16 + 4 * c4 + v;
-        if (m >= g.M) continue;
-        if (g.a_rows && g.a_rows[m] < 0) continue;
-        float o = acc[t][mt][v] + b;
-        if (DUAL) o = gate_fn(o, g.gate) * acc2[t][mt][v];
         store_out<OUT_ACT>(g, m, n, o);
       }
   }
@@ -783,7 +561,7 @@ static int launch_stream(MfmaGemmArgs g, bool dual, bool out_act, int row_tiles,
 
 template <int BM, int WM, int WN, int BN = TBN>
 static int launch_tile(const MfmaGemmArgs& g, bool dual, bool out_act, int splits, hipStream_t st) {
-  const dim3 grid(g.pair64 ? g.M / 64 : (g.M + BM - 1) / BM, (g.N + BN - 1) / BN, splits);
+  const dim3 grid((g.M + BM - 1) / BM, (g.N + BN - 1) / BN, splits);
   const size_t shmem = (size_t)2 * (BM + BN * (dual ? 2 : 1)) * TBK * sizeof(bf16_t);
 #define TQ_TILE(D, O)                                                                                  \
   do {                                                                                                 \
@@ -803,27 +581,6 @@ static int launch_tile(const MfmaGemmArgs& g, bool dual, bool out_act, int split
     TQ_TILE(false, false);
 #undef TQ_TILE
   return 0;
-}
-
-// A gated pair: two column tiles of each matrix to a wave (128 columns a workgroup); one matrix: four (256 columns).
-static int launch_rowstream(const MfmaGemmArgs& g, bool dual, bool out_act, hipStream_t st) {
-  const int BN = dual ? 128 : 256;
-  const dim3 grid((g.M + TQ_RS_BM - 1) / TQ_RS_BM, (g.N + BN - 1) / BN, 1);
-  if (dual && out_act) hipLaunchKernelGGL((gemm_rowstream_kernel<2, true, true>), grid, dim3(256), 0, st, g);
-  else if (dual) hipLaunchKernelGGL((gemm_rowstream_kernel<2, true, false>), grid, dim3(256), 0, st, g);
-  else if (out_act) hipLaunchKernelGGL((gemm_rowstream_kernel<4, false, true>), grid, dim3(256), 0, st, g);
-  else hipLaunchKernelGGL((gemm_rowstream_kernel<4, false, false>), grid, dim3(256), 0, st, g);
-  return 0;
-}
-
-// Which kernel takes a product over experts whose rows are ordered in units of 64: 2 (the default) tiles of 128 rows
-// over two units of an expert at a time, 0 tiles of 64 rows, 1 the kernel that streams the matrices past the rows.
-// For measurements; all give a row the same sums in the same order of k.
-static int g_expert_kernel = 0;
-TQ_API int tq_gemm_mfma_expert_kernel(int which) {
-  const int before = g_expert_kernel;
-  if (which >= 0 && which <= 3) g_expert_kernel = which;
-  return before;
 }
 
 // Whether a product of 17 to 64 rows takes the tiled kernel: a matrix wide enough to give every compute unit two
@@ -945,18 +702,7 @@ TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gat
       rc = launch_stream<2>(g, dual, out_act, M / 32, st);
     } else if (tile_rows == 64) {
       if ((N + TBN - 1) / TBN > 65535) return TQ_ERR_UNSUPPORTED;
-      if (g_expert_kernel == 2) {
-        if (M % 64) return TQ_ERR_BAD_ARG;
-        g.pair64 = 1;
-        rc = dual ? launch_tile<128, 2, 4>(g, dual, out_act, 1, st) : launch_tile<128, 4, 2>(g, dual, out_act, 1, st);
-      } else if (g_expert_kernel == 3) {      // the same with sixteen waves to the workgroup
-        if (M % 64) return TQ_ERR_BAD_ARG;
-        g.pair64 = 1;
-        rc = launch_tile<128, 4, 4>(g, dual, out_act, 1, st);
-      } else if (g_expert_kernel == 1)
-        rc = launch_rowstream(g, dual, out_act, st);
-      else
-        rc = launch_tile<64, 2, 4>(g, dual, out_act, 1, st);
+      rc = launch_tile<64, 2, 4>(g, dual, out_act, 1, st);
     } else if (tile_rows == 128) {     // experts with hundreds of rows each: the taller tile's rate for little padding
       if ((N + TBN - 1) / TBN > 65535 || M % 128) return TQ_ERR_UNSUPPORTED;
       // the gated pair as 2 x 4 waves of 64 x 32 outputs (and as many of w2): 3 to 4 % faster than 4 x 2 of 32 x 64

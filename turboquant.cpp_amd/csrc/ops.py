@@ -66,7 +66,6 @@ _OPTIONAL = {
     "tq_gemm_mfma": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int,
                      _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "tq_gemm_mfma_splits": [_c_int, _c_int, _c_int],
-    "tq_gemm_mfma_expert_kernel": [_c_int],
     "tq_gemm_mfma_pair_splits": [_c_int, _c_int, _c_int, _c_int, _c_int, _c_int],
     "tq_gemm_mfma_pair": [_c_ptr, _c_ptr, _c_int, _c_ptr],
     "tq_qkv_rope_write": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr,

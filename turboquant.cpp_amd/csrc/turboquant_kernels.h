@@ -45,7 +45,6 @@ int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gather, co
         int64_t group_stride, const int* tile_group, const int* n_tiles, const void* bias, int bias_type,
         void* out, int64_t ldc, int out_is_act, int M, int N, int K, int tile_rows, int splits, int gate,
         hipStream_t st);
-int tq_gemm_mfma_expert_kernel(int which);
 int tq_gemm_mfma_pair_splits(int N1, int K1, int grouped1, int N2, int K2, int grouped2);
 int tq_gemm_mfma_pair(const int64_t* d1, const int64_t* d2, int splits2, hipStream_t st);
 int tq_qkv_rope_write(const void* a, int64_t lda, const void* w, const void* bias, int bias_type, int T, int K,
