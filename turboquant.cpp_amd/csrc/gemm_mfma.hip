@@ -379,6 +379,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g)
   if (g.tile_group && g.a_rows && g.a_rows[min(m0, g.M - 1)] < 0) return;
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int wm = wave / WN, wn = wave % WN;
+  // A wave whose rows of an expert's tile are all padding (the expert's last tile is half empty on average) has
+  // nothing to multiply: it fetches and stages its share of the tile and waits at the barriers.
+  const int wave_m0 = m0 + wm * (MI * 32);
+  const bool active = !(g.tile_group && g.a_rows) || (wave_m0 < g.M && g.a_rows[wave_m0] >= 0);
   // this workgroup's run of k: k_lo .. k_lo + Kl (all of k unless the product is split), and where its sums go
   const int k_lo = blockIdx.z * g.k_per;
   const int Kl = min(g.K, k_lo + g.k_per) - k_lo;
@@ -472,6 +476,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g)
     const bf16_t* Ac = As + cur;
     const bf16_t* Wc = Ws + cur;
     const bf16_t* Vc = Vs + cur;
+    if (active)
 #pragma unroll
     for (int j = 0; j < TBK / 16; ++j) {
       bf16x8 af[MI], wf[NI], vf[DUAL ? NI : 1];
@@ -499,6 +504,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g)
 #undef TQ_FETCH
 #undef TQ_STAGE
 
+  if (!active) return;
 #pragma unroll
   for (int ni = 0; ni < NI; ++ni) {
     const int n = n0 + wn * (NI * 32) + ni * 32 + lr;
