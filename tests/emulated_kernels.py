@@ -239,9 +239,17 @@ def qkv_rope_write(a, qkv_weight, qkv_bias, positions, seq_of_token, block_table
                          layer_offset, page_size, page_stride, num_heads, num_kv_heads, head_dim, act, runs=runs)
 
 
+def gather_rows(src, index, act):
+    return src.index_select(0, index.long())
+
+
+def scatter_rows(dst, index, rows, act):
+    dst.index_copy_(0, index.long(), rows)
+
+
 def install(monkeypatch):
     """Puts the stand-ins in place of the kernels for one test."""
     from turboquant_cpp_amd.csrc import ops
     for name in ("embed", "add_rmsnorm", "rope_kv_write", "qkv_rope_write", "attention", "gemm", "router_topk", "moe_align", "route", "gemm_pair",
-                 "head_rmsnorm", "expert_tile_rows", "moe_combine", "argmax", "rep_penalty", "sample_topp", "softcap"):
+                 "head_rmsnorm", "expert_tile_rows", "moe_combine", "argmax", "rep_penalty", "sample_topp", "softcap", "gather_rows", "scatter_rows"):
         monkeypatch.setattr(ops, name, globals()[name])

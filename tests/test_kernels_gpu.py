@@ -47,6 +47,25 @@ def test_embed(ops, act, wdtype):
 
 
 @pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("shape,dtype", [((9, 3), torch.float32), ((40, 5, 130), torch.float32), ((7, 6), torch.bfloat16),
+                                         ((5, 4100), torch.int32)])
+def test_rows_by_index(ops, act, shape, dtype):
+    """Rows gathered out of and scattered into a tensor with a row per slot, as a step takes and puts back the
+    fixed-size state of its sequences: bit for bit what indexing gives."""
+    g = torch.Generator().manual_seed(5)
+    table = (torch.randn(shape, generator=g) * 100).to(dtype)
+    index = torch.randperm(shape[0], generator=g)[: max(1, shape[0] // 2)].to(torch.int32)
+    got = ops.gather_rows(table.to(DEV), index.to(DEV), act).cpu()
+    assert torch.equal(got, table[index.long()])
+    rows = (torch.randn((index.numel(), *shape[1:]), generator=g) * 100).to(dtype)
+    dev = table.to(DEV)
+    ops.scatter_rows(dev, index.to(DEV), rows.to(DEV), act)
+    want = table.clone()
+    want[index.long()] = rows
+    assert torch.equal(dev.cpu(), want)
+
+
+@pytest.mark.parametrize("act", ACTS)
 @pytest.mark.parametrize("H", [48, 200, 1000])
 def test_add_rmsnorm(ops, act, H):
     T, S, eps = 7, 3, 1e-5
@@ -1197,9 +1216,10 @@ def test_decoding_reads_nothing_beyond_a_head_that_fills_no_whole_tile(ops, act,
 
 def test_probes_run(ops):
     """The two kernels behind `bench.py --probe` (a plain read, the matrix instructions alone) do the work they are
-    timed for: the read of 256 MiB takes at least as long as the memory's published rate allows and no longer
-    than a tenth of it would, and the matrix loop stays below the published peak and above a tenth of it.  A
-    kernel whose loop the compiler had emptied, or that read a fraction of the buffer, would be too fast."""
+    timed for: the read of 256 MiB takes at least as long as the memory's published rate allows and no more than
+    twice what it took when measured (4.7 to 6.9 TB/s), and the matrix loop stays below the published peak and above
+    two thirds of what it reached (1.85 to 2.45 PFLOP/s).  A kernel whose loop the compiler had emptied, or that read
+    a fraction of the buffer, would be too fast; one that had lost its whole-line loads or its unrolling too slow."""
     def seconds(fn):
         fn()
         torch.cuda.synchronize()
@@ -1217,7 +1237,7 @@ def test_probes_run(ops):
     nbytes = buf.numel() * 4
     for once in (False, True):
         rate = nbytes / seconds(lambda: ops.probe_stream(buf, once))
-        assert 0.8e12 < rate < 8.0e12 * 1.05, (once, rate)
+        assert (3.4e12 if once else 2.4e12) < rate < 8.0e12 * 1.05, (once, rate)
     assert ops.probe_mfma(32, 4, 10, 1, DEV) == 4 * 8 * 10 * 196608.0
     for shape in (32, 16):
         flop = [0.0]
@@ -1226,4 +1246,4 @@ def test_probes_run(ops):
             flop[0] = ops.probe_mfma(shape, 512, 2000, 12345, DEV)
         t = seconds(run)
         rate = flop[0] / t
-        assert 0.25e15 < rate < 2.5e15 * 1.02, (shape, rate)
+        assert 1.2e15 < rate < 2.5e15 * 1.02, (shape, rate)

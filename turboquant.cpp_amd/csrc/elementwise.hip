@@ -42,6 +42,29 @@ TQ_API int tq_softcap(float* x, int64_t n, float cap, hipStream_t st) {
   return 0;
 }
 
+// ---------------------------------------------------------------- rows by index
+// The rows of a sequence's fixed-size state lie at its slot; a step works on the rows of its own sequences.
+// gather: dst[i] = src[idx[i]];  scatter: dst[idx[i]] = src[i];  rows of `words` 32-bit words.  grid (rows, chunks).
+__global__ void move_rows_kernel(const uint32_t* __restrict__ src, const int* __restrict__ idx, uint32_t* __restrict__ dst,
+                                 int64_t words, int scatter) {
+  const int64_t row = blockIdx.x, at = idx[row];
+  const uint32_t* from = src + (scatter ? row : at) * words;
+  uint32_t* to = dst + (scatter ? at : row) * words;
+  for (int64_t w = (int64_t)blockIdx.y * blockDim.x + threadIdx.x; w < words; w += (int64_t)gridDim.y * blockDim.x) to[w] = from[w];
+}
+
+// src, dst: rows of row_bytes bytes (a multiple of 4); idx [n]: for gather the row of src behind each row of dst, for
+// scatter the row of dst that each row of src goes to (every index once).
+TQ_API int tq_move_rows(const void* src, const int* idx, void* dst, int n, int64_t row_bytes, int scatter, hipStream_t st) {
+  if (n <= 0 || row_bytes <= 0) return 0;
+  if (row_bytes % 4 != 0 || n > 65535 * 32768) return TQ_ERR_UNSUPPORTED;
+  const int64_t words = row_bytes / 4;
+  const int chunks = (int)((words + 1023) / 1024 < 1024 ? (words + 1023) / 1024 : 1024);
+  hipLaunchKernelGGL(move_rows_kernel, dim3(n, chunks), dim3(256), 0, st, (const uint32_t*)src, idx, (uint32_t*)dst, words, scatter);
+  TQ_LAUNCH_CHECK();
+  return 0;
+}
+
 // ---------------------------------------------------------------- residual sum + RMS norm
 // For row r (token rows[r], or r itself when rows is null):
 //   v = x[row] + d[row]                         (the residual sum, in float)

@@ -118,10 +118,18 @@ struct Product {
   void* dest = nullptr;      // where the result goes, if not into the arena (never with partial sums)
 };
 
+// Whether a plain product goes to the vendor's library: the caller's bound on the rows, not under capture, and the
+// library has a kernel for the shapes that would be asked of it (the product itself, or a gated pair's product over
+// both matrices in chunks of rows); the same answer in the pass that counts and in the pass that launches.
 bool vendor_product(const Ctx& c, const Product& p) {
   const tq_step_desc& s = *c.s;
-  return bf16_path() && s.vendor_min_rows > 0 && p.M >= s.vendor_min_rows && (p.K < 16384 || p.M >= 8192) &&
-         p.w.wtype == TQ_BF16 && !s.capturing && !s.decode && tq_vendor_available();
+  if (!(bf16_path() && s.vendor_min_rows > 0 && p.M >= s.vendor_min_rows && (p.K < 16384 || p.M >= 8192) &&
+        p.w.wtype == TQ_BF16 && !s.capturing && !s.decode && tq_vendor_available()))
+    return false;
+  if (!p.w2) return tq_vendor_takes(p.M, p.N, p.K, p.lda, p.out_act) != 0;
+  const int64_t chunk = s.vendor_gated_rows > 0 ? s.vendor_gated_rows : 4096;
+  const int rows = (int)(p.M < chunk ? p.M : chunk), last = (int)(p.M % chunk);
+  return tq_vendor_takes(rows, 2 * p.N, p.K, p.lda, 0) != 0 && (last == 0 || tq_vendor_takes(last, 2 * p.N, p.K, p.lda, 0) != 0);
 }
 
 int gated_act(Ctx& c, const float* gu, int64_t ld, void* out, int M, int N, int gate) {

@@ -24,6 +24,9 @@ struct Api {
   decltype(&hipblasLtMatrixLayoutCreate) layout_create = nullptr;
   decltype(&hipblasLtMatmulPreferenceCreate) pref_create = nullptr;
   decltype(&hipblasLtMatmulPreferenceSetAttribute) pref_set = nullptr;
+  decltype(&hipblasLtMatmulPreferenceDestroy) pref_destroy = nullptr;
+  decltype(&hipblasLtMatmulDescDestroy) desc_destroy = nullptr;
+  decltype(&hipblasLtMatrixLayoutDestroy) layout_destroy = nullptr;
   decltype(&hipblasLtMatmulAlgoGetHeuristic) heuristic = nullptr;
   decltype(&hipblasLtMatmul) matmul = nullptr;
   bool ok = false;
@@ -34,6 +37,7 @@ struct Problem {        // what the library was asked once for a shape, kept for
   hipblasLtMatrixLayout_t a, b, d;
   hipblasLtMatmulAlgo_t algo;
   size_t workspace;
+  bool usable;
 };
 
 std::mutex g_lock;
@@ -41,6 +45,14 @@ Api g_api;
 bool g_tried = false;
 std::map<int, hipblasLtHandle_t> g_handles;                                   // by device
 std::map<std::tuple<int, int, int, int, int64_t, int>, Problem> g_problems;  // device, M, N, K, lda, out type
+constexpr size_t kMostProblems = 2048;     // shapes kept; a host that brings ever new row counts starts over beyond that
+
+void forget(Problem& p) {
+  if (p.desc) g_api.desc_destroy(p.desc);
+  for (hipblasLtMatrixLayout_t l : {p.a, p.b, p.d})
+    if (l) g_api.layout_destroy(l);
+  p = Problem{};
+}
 
 template <class F>
 bool sym(void* lib, const char* name, F& fn) {
@@ -70,6 +82,8 @@ void load_api() {
          sym(lib, "hipblasLtMatmulDescSetAttribute", a.desc_set) && sym(lib, "hipblasLtMatrixLayoutCreate", a.layout_create) &&
          sym(lib, "hipblasLtMatmulPreferenceCreate", a.pref_create) &&
          sym(lib, "hipblasLtMatmulPreferenceSetAttribute", a.pref_set) &&
+         sym(lib, "hipblasLtMatmulPreferenceDestroy", a.pref_destroy) && sym(lib, "hipblasLtMatmulDescDestroy", a.desc_destroy) &&
+         sym(lib, "hipblasLtMatrixLayoutDestroy", a.layout_destroy) &&
          sym(lib, "hipblasLtMatmulAlgoGetHeuristic", a.heuristic) && sym(lib, "hipblasLtMatmul", a.matmul);
 }
 
@@ -81,6 +95,83 @@ extern "C" int tq_vendor_available(void) {
   return g_api.ok ? 1 : 0;
 }
 
+namespace {
+
+// The library's plan for a shape (kept once made), or null: the library is absent or has no kernel for it.
+// code: 0, TQ_ERR_UNSUPPORTED or 1000 + the library's status.
+const Problem* problem_for(int M, int N, int K, int64_t lda, int out_is_bf16, hipblasLtHandle_t* handle, int* code) {
+  *code = TQ_ERR_UNSUPPORTED;
+  load_api();
+  if (!g_api.ok) return nullptr;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+  auto h = g_handles.find(dev);
+  if (h == g_handles.end()) {
+    hipblasLtHandle_t made = nullptr;
+    if (g_api.create(&made) != HIPBLAS_STATUS_SUCCESS) return nullptr;
+    h = g_handles.emplace(dev, made).first;
+  }
+  *handle = h->second;
+  const auto key = std::make_tuple(dev, M, N, K, lda, out_is_bf16);
+  auto p = g_problems.find(key);
+  if (p == g_problems.end()) {
+    if (g_problems.size() >= kMostProblems) {
+      for (auto& kept : g_problems) forget(kept.second);
+      g_problems.clear();
+    }
+    // Column-major as the library counts: out^T [N][M] = w [N][K] a^T, that is op(A) = A^T with A = w seen as
+    // [K][N] with leading size K, and B = a seen as [K][M] with leading size lda.
+    Problem pr{};
+    hipblasStatus_t s = g_api.desc_create(&pr.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F);
+    if (s != HIPBLAS_STATUS_SUCCESS) {
+      *code = 1000 + (int)s;
+      return nullptr;
+    }
+    const int32_t ta = HIPBLAS_OP_T, tb = HIPBLAS_OP_N;
+    g_api.desc_set(pr.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &ta, sizeof(ta));
+    g_api.desc_set(pr.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &tb, sizeof(tb));
+    const hipDataType out_type = out_is_bf16 ? HIP_R_16BF : HIP_R_32F;
+    hipblasLtMatmulPreference_t pref = nullptr;
+    if ((s = g_api.layout_create(&pr.a, HIP_R_16BF, K, N, K)) != HIPBLAS_STATUS_SUCCESS ||
+        (s = g_api.layout_create(&pr.b, HIP_R_16BF, K, M, lda)) != HIPBLAS_STATUS_SUCCESS ||
+        (s = g_api.layout_create(&pr.d, out_type, N, M, N)) != HIPBLAS_STATUS_SUCCESS ||
+        (s = g_api.pref_create(&pref)) != HIPBLAS_STATUS_SUCCESS) {
+      forget(pr);
+      *code = 1000 + (int)s;
+      return nullptr;
+    }
+    const uint64_t max_ws = TQ_VENDOR_WORKSPACE;
+    g_api.pref_set(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &max_ws, sizeof(max_ws));
+    hipblasLtMatmulHeuristicResult_t found[1];
+    int n_found = 0;
+    s = g_api.heuristic(h->second, pr.desc, pr.a, pr.b, pr.d, pr.d, pref, 1, found, &n_found);
+    g_api.pref_destroy(pref);
+    pr.usable = s == HIPBLAS_STATUS_SUCCESS && n_found >= 1 && found[0].workspaceSize <= TQ_VENDOR_WORKSPACE;
+    if (pr.usable) {
+      pr.algo = found[0].algo;
+      pr.workspace = found[0].workspaceSize;
+    } else {
+      forget(pr);          // what is kept says only that the library has nothing for this shape
+    }
+    p = g_problems.emplace(key, pr).first;
+  }
+  if (!p->second.usable) return nullptr;
+  *code = 0;
+  return &p->second;
+}
+
+}  // namespace
+
+// Whether tq_vendor_product would take this product (asked once per shape of the library, then remembered); a
+// caller decides with it before it plans its memory.
+extern "C" int tq_vendor_takes(int M, int N, int K, int64_t lda, int out_is_bf16) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  std::lock_guard<std::mutex> hold(g_lock);
+  hipblasLtHandle_t handle = nullptr;
+  int code = 0;
+  return problem_for(M, N, K, lda, out_is_bf16, &handle, &code) != nullptr;
+}
+
 // out[m][n] = sum_k a[m][k] * w[n][k]: a bfloat16 [M][K] with row stride lda, w bfloat16 [N][K], out [M][N] in float
 // (out_is_bf16 0) or bfloat16, sums in float.  workspace: TQ_VENDOR_WORKSPACE bytes that no other stream uses
 // meanwhile.  Returns 0, TQ_ERR_UNSUPPORTED (the library is absent or has no kernel for the shape: nothing was
@@ -89,46 +180,12 @@ extern "C" int tq_vendor_product(const void* a, int64_t lda, const void* w, void
                                  int K, void* workspace, hipStream_t st) {
   if (M <= 0 || N <= 0) return 0;
   std::lock_guard<std::mutex> hold(g_lock);
-  load_api();
-  if (!g_api.ok) return TQ_ERR_UNSUPPORTED;
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) return TQ_ERR_BAD_ARG;
-  auto h = g_handles.find(dev);
-  if (h == g_handles.end()) {
-    hipblasLtHandle_t handle = nullptr;
-    if (g_api.create(&handle) != HIPBLAS_STATUS_SUCCESS) return TQ_ERR_UNSUPPORTED;
-    h = g_handles.emplace(dev, handle).first;
-  }
-  const auto key = std::make_tuple(dev, M, N, K, lda, out_is_bf16);
-  auto p = g_problems.find(key);
-  if (p == g_problems.end()) {
-    // Column-major as the library counts: out^T [N][M] = w [N][K] a^T, that is op(A) = A^T with A = w seen as
-    // [K][N] with leading size K, and B = a seen as [K][M] with leading size lda.
-    Problem pr{};
-    hipblasStatus_t s = g_api.desc_create(&pr.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F);
-    if (s != HIPBLAS_STATUS_SUCCESS) return 1000 + (int)s;
-    const int32_t ta = HIPBLAS_OP_T, tb = HIPBLAS_OP_N;
-    g_api.desc_set(pr.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &ta, sizeof(ta));
-    g_api.desc_set(pr.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &tb, sizeof(tb));
-    const hipDataType out_type = out_is_bf16 ? HIP_R_16BF : HIP_R_32F;
-    if ((s = g_api.layout_create(&pr.a, HIP_R_16BF, K, N, K)) != HIPBLAS_STATUS_SUCCESS) return 1000 + (int)s;
-    if ((s = g_api.layout_create(&pr.b, HIP_R_16BF, K, M, lda)) != HIPBLAS_STATUS_SUCCESS) return 1000 + (int)s;
-    if ((s = g_api.layout_create(&pr.d, out_type, N, M, N)) != HIPBLAS_STATUS_SUCCESS) return 1000 + (int)s;
-    hipblasLtMatmulPreference_t pref = nullptr;
-    if ((s = g_api.pref_create(&pref)) != HIPBLAS_STATUS_SUCCESS) return 1000 + (int)s;
-    const uint64_t max_ws = TQ_VENDOR_WORKSPACE;
-    g_api.pref_set(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &max_ws, sizeof(max_ws));
-    hipblasLtMatmulHeuristicResult_t found[1];
-    int n_found = 0;
-    s = g_api.heuristic(h->second, pr.desc, pr.a, pr.b, pr.d, pr.d, pref, 1, found, &n_found);
-    if (s != HIPBLAS_STATUS_SUCCESS || n_found < 1 || found[0].workspaceSize > TQ_VENDOR_WORKSPACE) return TQ_ERR_UNSUPPORTED;
-    pr.algo = found[0].algo;
-    pr.workspace = found[0].workspaceSize;
-    p = g_problems.emplace(key, pr).first;
-  }
+  hipblasLtHandle_t handle = nullptr;
+  int code = 0;
+  const Problem* pr = problem_for(M, N, K, lda, out_is_bf16, &handle, &code);
+  if (!pr) return code;
   const float one = 1.0f, zero = 0.0f;
-  const Problem& pr = p->second;
-  hipblasStatus_t s = g_api.matmul(h->second, pr.desc, &one, w, pr.a, a, pr.b, &zero, out, pr.d, out, pr.d, &pr.algo,
-                                   workspace, pr.workspace ? TQ_VENDOR_WORKSPACE : 0, st);
+  hipblasStatus_t s = g_api.matmul(handle, pr->desc, &one, w, pr->a, a, pr->b, &zero, out, pr->d, out, pr->d, &pr->algo,
+                                   workspace, pr->workspace ? TQ_VENDOR_WORKSPACE : 0, st);
   return s == HIPBLAS_STATUS_SUCCESS ? 0 : 1000 + (int)s;
 }

@@ -9,6 +9,7 @@
 extern "C" {
 #endif
 int tq_vendor_available(void);
+int tq_vendor_takes(int M, int N, int K, int64_t lda, int out_is_bf16);
 int tq_vendor_product(const void* a, int64_t lda, const void* w, void* out, int out_is_bf16, int M, int N, int K,
                       void* workspace, hipStream_t st);
 #ifdef __cplusplus

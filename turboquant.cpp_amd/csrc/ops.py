@@ -31,6 +31,7 @@ _c_int, _c_i64, _c_f32, _c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, c
 _SIGNATURES = {
     "tq_embed": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_f32, _c_ptr],
     "tq_softcap": [_c_ptr, _c_i64, _c_f32, _c_ptr],
+    "tq_move_rows": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_ptr],
     "tq_gated_act": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "tq_head_rmsnorm": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_f32, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "tq_add_rmsnorm": [_c_ptr, _c_ptr, _c_int, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_f32,
@@ -227,6 +228,29 @@ def softcap(logits: torch.Tensor, cap: float, act) -> torch.Tensor:
     _need(cap > 0, k, "the cap must be positive")
     _run(k, library(act).tq_softcap(_ptr(logits), logits.numel(), float(cap), _stream()))
     return logits
+
+
+def gather_rows(src: torch.Tensor, index: torch.Tensor, act) -> torch.Tensor:
+    """``src[index]`` along the first dimension (``index`` int32 on the device): the rows of a step's sequences out of
+    a tensor that has a row per slot."""
+    k = "gather_rows"
+    _check(src, k, "src")
+    _check(index, k, "index", torch.int32)
+    _need(index.dim() == 1 and src.dim() >= 1, k, "index must be [n], src [rows, ...]")
+    row_bytes = (src.numel() // max(src.shape[0], 1)) * src.element_size()
+    out = torch.empty((index.numel(), *src.shape[1:]), dtype=src.dtype, device=src.device)
+    _run(k, library(act).tq_move_rows(_ptr(src), _ptr(index), _ptr(out), index.numel(), row_bytes, 0, _stream()))
+    return out
+
+
+def scatter_rows(dst: torch.Tensor, index: torch.Tensor, rows: torch.Tensor, act) -> None:
+    """``dst[index] = rows`` along the first dimension; every index at most once."""
+    k = "scatter_rows"
+    _check(dst, k, "dst")
+    _check(index, k, "index", torch.int32)
+    _check(rows, k, "rows", dst.dtype, (index.numel(), *dst.shape[1:]))
+    row_bytes = (dst.numel() // max(dst.shape[0], 1)) * dst.element_size()
+    _run(k, library(act).tq_move_rows(_ptr(rows), _ptr(index), _ptr(dst), index.numel(), row_bytes, 1, _stream()))
 
 
 @dataclasses.dataclass

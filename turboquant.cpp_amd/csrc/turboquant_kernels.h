@@ -21,6 +21,7 @@ extern "C" {
 // elementwise.hip: embedding, soft cap, residual sum + RMS norm, per-head norm, rotation + cache write, weighted sum of expert rows (both libraries)
 int tq_embed(const int* tokens, const void* table, int wtype, float* x, int T, int H, float scale, hipStream_t st);
 int tq_softcap(float* x, int64_t n, float cap, hipStream_t st);
+int tq_move_rows(const void* src, const int* idx, void* dst, int n, int64_t row_bytes, int scatter, hipStream_t st);
 int tq_add_rmsnorm(float* x, const float* delta, int S, int64_t delta_stride, const float* y, const int* pair_slot,
         const float* weights, int topk, const float* gate, const void* w, int wtype, float eps, const int* rows,
         int R, void* out, float* out32, int H, hipStream_t st);

@@ -45,8 +45,10 @@ class StepContext:
     def state_rows(self, entry: int) -> torch.Tensor:
         """The state of the step's sequences, [sequences, ...], in the step's order: gathered through the slots on
         the device, so a captured step replays it for other slots."""
-        return self.cache.state(entry).index_select(0, self.batch.slots_dev.long())
+        from ..csrc import ops
+        return ops.gather_rows(self.cache.state(entry), self.batch.slots_dev, self.act)
 
     def store_state_rows(self, entry: int, rows: torch.Tensor) -> None:
         """Puts the advanced state of the step's sequences back (the counterpart of ``state_rows``)."""
-        self.cache.state(entry).index_copy_(0, self.batch.slots_dev.long(), rows)
+        from ..csrc import ops
+        ops.scatter_rows(self.cache.state(entry), self.batch.slots_dev, rows.contiguous(), self.act)
