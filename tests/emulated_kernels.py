@@ -110,6 +110,7 @@ def gemm(a, w, act, bias=None, w2=None, out_act=False, a_rows=None, tile_group=N
             y = gate(y) * (src @ w2.float().T)
     else:
         P, N = a_rows.numel(), w.shape[1]
+        tile_rows %= 1024        # (units of 64 taken two at a time give what unit by unit gives)
         y = torch.full((P, N), float("nan"))
         for tile in range(int(n_tiles[0])):
             g = int(tile_group[tile])
@@ -156,8 +157,8 @@ def moe_align(ids, num_experts, unit, act):
     cap = (cap + unit - 1) // unit * unit
     sorted_token = torch.full((cap,), -1, dtype=torch.int32)
     pair_slot = torch.empty((T, topk), dtype=torch.int32)
-    tile_expert = torch.zeros((cap // unit,), dtype=torch.int32)
-    row = tile = 0
+    tile_expert = torch.zeros((2 * (cap // unit),), dtype=torch.int32)      # row tiles, then items of two row tiles
+    row = tile = item = 0
     for e in range(num_experts):
         mine = [i for i, x in enumerate(flat) if x == e]
         for j, i in enumerate(mine):
@@ -165,9 +166,12 @@ def moe_align(ids, num_experts, unit, act):
             pair_slot.view(-1)[i] = row + j
         nt = -(-len(mine) // unit)
         tile_expert[tile:tile + nt] = e
+        for first in range(tile, tile + nt, 2):
+            tile_expert[cap // unit + item] = first
+            item += 1
         tile += nt
         row += nt * unit
-    return sorted_token, pair_slot, tile_expert, torch.tensor([tile], dtype=torch.int32)
+    return sorted_token, pair_slot, tile_expert, torch.tensor([tile, item], dtype=torch.int32)
 
 
 def moe_combine(y, pair_slot, weights, shared, shared_gate, act):

@@ -83,12 +83,13 @@ def test_the_executor_gives_the_bits_of_the_parts(name, act, models):
 @pytest.mark.gpu
 @pytest.mark.parametrize("act", ACTS)
 def test_the_executor_at_the_layer_sizes_of_a_real_checkpoint(act, monkeypatch):
-    """Two layers of Qwen1.5-MoE-A2.7B's sizes: steps of 1, 8, 17, 64, 300 and 900 tokens (the pair of products in one
-    launch, the streaming and the tile kernels, units of 16 to 64 rows per expert, one and two streams), decode steps
+    """Two layers of Qwen1.5-MoE-A2.7B's sizes: steps of 1, 8, 17, 64, 300, 900 and 1,100 tokens (the pair of products in one
+    launch, the streaming and the tile kernels, units of 16 to 64 rows per expert and, in the longest, units of 64 two
+    at a time, one and two streams), decode steps
     eager and replayed.  A step of 900 tokens hands its plain bfloat16 products to the vendor's library; the executor
     calls that library itself where the parts go through torch, and the two may be served by different kernels of it:
     there both are compared with each other at the bound of a bfloat16 product, and with every product in this
-    library's kernels the bits agree again."""
+    library's kernels the bits agree again, also between the experts' units taken two at a time and one by one."""
     from turboquant_cpp_amd.csrc import ops
     from turboquant_cpp_amd.engine.model import random_model
     from turboquant_cpp_amd.engine.step import Engine
@@ -101,7 +102,7 @@ def test_the_executor_at_the_layer_sizes_of_a_real_checkpoint(act, monkeypatch):
            "max_window_layers": 2, "max_position_embeddings": 4096, "tie_word_embeddings": False, "torch_dtype": "float32"}
     model = random_model(cfg, seed=7, act=act, device=DEV)
     g = torch.Generator().manual_seed(62)
-    lens = [1, 8, 17, 64, 300, 900]
+    lens = [1, 8, 17, 64, 300, 900, 1100]
     prompts = [torch.randint(0, V, (n,), generator=g).tolist() for n in lens]
     engines = [Engine(model, max_tokens=64 * 40), Engine(model, max_tokens=64 * 40)]
     engines[1].native = None
@@ -124,7 +125,7 @@ def test_the_executor_at_the_layer_sizes_of_a_real_checkpoint(act, monkeypatch):
     a, b = run(engines[0]), run(engines[1])
     vendor = act == "bfloat16" and ops._VENDOR
     for key in a:
-        if key == 900 and vendor:
+        if key in (900, 1100) and vendor:
             scale = b[key].abs().max().item()
             assert (a[key] - b[key]).abs().max().item() < 0.04 * scale, key
         else:
@@ -133,14 +134,21 @@ def test_the_executor_at_the_layer_sizes_of_a_real_checkpoint(act, monkeypatch):
     assert all(2 * 8 + 3 <= launches[n] <= 2 * 14 + 3 for n in lens), launches
     if vendor:
         monkeypatch.setattr(ops, "_VENDOR", False)
-        own = []
+        for n in (900, 1100):
+            own = []
+            for eng in engines:
+                slot = eng.open(1)
+                own.append(eng.step(slot, [prompts[lens.index(n)]], [[0, n - 1]]).clone())
+                eng.close(slot)
+            assert torch.equal(own[0], own[1])
+            scale = own[0].abs().max().item()
+            assert (own[0] - a[n]).abs().max().item() < 0.04 * scale
+        # 1,100 tokens are 73 rows per expert: units of 64 two at a time; one by one they give the same bits
+        monkeypatch.setattr(ops, "EXPERT_PAIRS_FROM", 1 << 30)
         for eng in engines:
             slot = eng.open(1)
-            own.append(eng.step(slot, [prompts[-1]], [[0, 899]]).clone())
+            assert torch.equal(eng.step(slot, [prompts[-1]], [[0, 1099]]), own[0])
             eng.close(slot)
-        assert torch.equal(own[0], own[1])
-        scale = own[0].abs().max().item()
-        assert (own[0] - a[900]).abs().max().item() < 0.04 * scale
 
 
 @pytest.mark.gpu

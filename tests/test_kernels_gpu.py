@@ -318,9 +318,10 @@ def test_gemm_rows_do_not_depend_on_the_batch(ops, act):
         assert torch.equal(part, full[:m])
 
 
-def test_the_height_of_expert_tiles(ops):
-    """16 up to 5 pairs per expert and 32 up to 10 where the bfloat16 matrix-core product runs (else 16 up to 12), 128 from 256 rows per expert and 256 from 1,024 where the bfloat16 matrix-core product
-    runs, else 64."""
+def test_the_height_of_expert_tiles(ops, monkeypatch):
+    """16 up to 5 pairs per expert and 32 up to 10 where the bfloat16 matrix-core product runs (else 16 up to 12), 64
+    beyond, which the products take two at a time from 64 rows per expert on; 128 and 256 only where their borders
+    are lowered, and only for the bfloat16 matrix-core product."""
     a16, w16 = torch.zeros((1, 64), dtype=torch.bfloat16), torch.zeros((1, 8, 64), dtype=torch.bfloat16)
     a32, w32 = a16.float(), w16.float()
     assert ops.expert_tile_rows(60 * 5, 60, "bfloat16", a16, w16) == 16
@@ -329,6 +330,12 @@ def test_the_height_of_expert_tiles(ops):
     assert ops.expert_tile_rows(60 * 10 + 1, 60, "bfloat16", a16, w16) == 64
     assert ops.expert_tile_rows(60 * 12, 60, "float32", a32, w32) == 16
     assert ops.expert_tile_rows(60 * 12 + 1, 60, "float32", a32, w32) == 64
+    assert ops.expert_tile_rows(60 * 100000, 60, "bfloat16", a16, w16) == 64
+    assert ops.expert_product_rows(64, 60 * 64 - 1, 60) == 64
+    assert ops.expert_product_rows(64, 60 * 64, 60) == 64 + ops.TILE_PAIRS
+    assert ops.expert_product_rows(16, 60 * 64, 60) == 16 and ops.expert_product_rows(256, 60 * 2000, 60) == 256
+    monkeypatch.setattr(ops, "EXPERT_128_FROM", 256)
+    monkeypatch.setattr(ops, "EXPERT_256_FROM", 1024)
     assert ops.expert_tile_rows(60 * 256 - 1, 60, "bfloat16", a16, w16) == 64
     assert ops.expert_tile_rows(60 * 256, 60, "bfloat16", a16, w16) == 128
     assert ops.expert_tile_rows(60 * 1024 - 1, 60, "bfloat16", a16, w16) == 128
@@ -339,23 +346,26 @@ def test_the_height_of_expert_tiles(ops):
 
 
 @pytest.mark.parametrize("act", ACTS)
-@pytest.mark.parametrize("unit", [16, 32, 64, 128, 256])
-@pytest.mark.parametrize("T,E,k,H,I", [(1, 5, 2, 72, 40), (9, 7, 3, 136, 88), (150, 6, 2, 64, 200), (700, 3, 2, 64, 136)])
+@pytest.mark.parametrize("unit", [16, 32, 64, 128, 256, 64 + 1024])
+@pytest.mark.parametrize("T,E,k,H,I", [(1, 5, 2, 72, 40), (9, 7, 3, 136, 88), (150, 6, 2, 64, 200), (700, 3, 2, 64, 136),
+                                       (700, 3, 2, 128, 192), (260, 5, 3, 192, 320)])
 def test_expert_products(ops, act, unit, T, E, k, H, I):
     """Pairs ordered by expert, the gated product over gathered rows, the second product over rows in place.
     Units of 32, 128 and 256 rows are the bfloat16 matrix-core product's alone (32: the streaming kernel with two row
     tiles to a wave; with 256, the gated pair runs in tiles of
     256 rows and the second product in two tiles of 128 to a unit; 700 tokens give each expert a whole unit and
-    a part of one)."""
-    if unit not in (16, 64) and act != "bfloat16":
-        pytest.skip("tiles of 32, 128 and 256 rows are for the bfloat16 matrix-core product")
+    a part of one).  64 + 1024: units of 64 that the products take two at a time, by the items that the order lists
+    behind its row tiles (where k is no multiple of 64 they fall back to one unit at a time)."""
+    rows, unit = unit, unit % 1024
+    if rows not in (16, 64) and act != "bfloat16":
+        pytest.skip("tiles of 32, 128 and 256 rows and pairs of units are for the bfloat16 matrix-core product")
     g = torch.Generator().manual_seed(40)
     ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32)
     x = rnd((T, H), adt(act), 41)
     wg, wu = rnd((E, I, H), adt(act), 42, 0.2), rnd((E, I, H), adt(act), 43, 0.2)
     wd = rnd((E, H, I), adt(act), 44, 0.2)
     st, slot, tile_e, n_tiles = ops.moe_align(ids.to(DEV), E, unit, act)
-    st_c, slot_c, tile_c, nt = st.cpu(), slot.cpu(), tile_e.cpu(), int(n_tiles.cpu())
+    st_c, slot_c, tile_c, (nt, n_items) = st.cpu(), slot.cpu(), tile_e.cpu(), n_tiles.cpu().tolist()
     # the order: every pair has its row, rows of one expert are together and in order of token, tiles are whole
     assert sorted(slot_c.view(-1).tolist()) == [r for r in range(st_c.numel()) if st_c[r] >= 0]
     for t in range(T):
@@ -364,11 +374,18 @@ def test_expert_products(ops, act, unit, T, E, k, H, I):
             assert int(st_c[r]) == t and int(tile_c[r // unit]) == int(ids[t, j])
     assert nt == sum(-(-int((ids == e).sum()) // unit) for e in range(E))
     rows_by_expert = [[r for r in range(nt * unit) if st_c[r] >= 0 and tile_c[r // unit] == e] for e in range(E)]
-    for rows in rows_by_expert:
-        assert [int(st_c[r]) for r in rows] == sorted(int(st_c[r]) for r in rows)
+    for mine in rows_by_expert:
+        assert [int(st_c[r]) for r in mine] == sorted(int(st_c[r]) for r in mine)
+    # the items behind the row tiles: every expert's row tiles two at a time, its last one alone if their number is odd
+    items = tile_c[st_c.numel() // unit:][:n_items].tolist()
+    expected = []
+    for e in range(E):
+        mine = [t for t in range(nt) if tile_c[t] == e]
+        expected += mine[::2]
+    assert items == expected
     h = ops.gemm(x.to(DEV), wg.to(DEV), act, w2=wu.to(DEV), out_act=True, a_rows=st, tile_group=tile_e,
-                 n_tiles=n_tiles, tile_rows=unit)
-    y = ops.gemm(h, wd.to(DEV), act, a_rows=st, tile_group=tile_e, n_tiles=n_tiles, tile_rows=unit, gather=False).cpu()
+                 n_tiles=n_tiles, tile_rows=rows)
+    y = ops.gemm(h, wd.to(DEV), act, a_rows=st, tile_group=tile_e, n_tiles=n_tiles, tile_rows=rows, gather=False).cpu()
     hc = h.cpu()
     for t in range(T):
         for j in range(k):
@@ -565,9 +582,10 @@ def test_routing_in_one_call(ops, act, E, k, H, renorm, shared):
             assert torch.equal(got[0], ids_all[:T]) and torch.equal(got[1], w_all[:T])
             assert (got[2] is None) == (not shared) and (not shared or torch.equal(got[2], gate_all[:T]))
             want = ops.moe_align(ids_all[:T].contiguous(), E, unit, act)
-            n = int(want[3])          # tiles in use; the entries of tile_expert beyond them are not written
+            n, items = want[3].tolist()      # tiles and items in use; the entries beyond them are not written
+            half = want[2].numel() // 2
             assert torch.equal(got[3], want[0]) and torch.equal(got[4], want[1]) and torch.equal(got[6], want[3])
-            assert torch.equal(got[5][:n], want[2][:n])
+            assert torch.equal(got[5][:n], want[2][:n]) and torch.equal(got[5][half:half + items], want[2][half:half + items])
 
 
 # ------------------------------------------------------------------------------------------------ rope + cache + attention

@@ -327,10 +327,10 @@ def test_the_configurations_whose_bfloat16_logits_lay_furthest_off(run, case, tm
 
 # ------------------------------------------------------------------------------------------------ a long prompt's experts
 def test_a_long_prompt_takes_the_taller_expert_tiles(sharp, monkeypatch):
-    """From 256 rows per expert on, the bfloat16 products over experts take tiles of 128 rows: a prompt of 1,400 tokens
+    """Where the borders of the taller units are lowered (by default units of 64 stay, taken two at a time), the bfloat16
+    products over experts take tiles of 128 rows from 256 rows per expert on: a prompt of 1,400 tokens
     with one expert of five per token goes that way through the engine (and one of 700 does not), and every
-    position agrees with the plain model.  From 1,024 rows per expert on the row order's unit is 256 (here the
-    bound is lowered to 256 rows, since the configuration's positions end at 2,048)."""
+    position agrees with the plain model.  With the second border at 256 rows too the row order's unit is 256."""
     from turboquant_cpp_amd.csrc import ops
     from turboquant_cpp_amd.engine.step import Engine
     d, plain, model = sharp("C", "bfloat16")
@@ -346,6 +346,7 @@ def test_a_long_prompt_takes_the_taller_expert_tiles(sharp, monkeypatch):
     executor = eng.native
     assert executor is not None
     for n, unit in ((1400, 128), (700, 64), (1400, 256)):
+        monkeypatch.setattr(ops, "EXPERT_128_FROM", 256)
         monkeypatch.setattr(ops, "EXPERT_256_FROM", 256 if unit == 256 else 1024)
         (prompt,) = prompts_for("C", [n], seed=29)
         del units[:]

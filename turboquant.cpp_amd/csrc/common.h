@@ -14,6 +14,8 @@
 // error codes of the extern "C" entry points (0 = ok, > 0 = hipError_t)
 #define TQ_ERR_BAD_ARG (-1)
 #define TQ_ERR_UNSUPPORTED (-2)
+// added to a tile_rows of 64 of a product over experts: two units of one expert per workgroup (see tq_gemm_mfma)
+#define TQ_TILE_PAIRS 1024
 
 struct bf16_t {
   uint16_t bits;

@@ -524,6 +524,149 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tile_kernel(MfmaGemmArgs g)
   }
 }
 
+// ------------------------------------------------------------------------------------------ experts with many rows
+// A matrix per expert whose rows are ordered in units of 64: a workgroup of 16 waves takes an item of the row order,
+// two units of one expert (or the expert's last one alone), and 256 columns: 128 of each matrix of a gated pair, or
+// 256 of one matrix.  What binds such a product is the bytes that a compute unit has on their way: every tile of 64
+// rows asks for its expert's matrices again, and a tile's bytes travel for the time of a miss whoever holds them,
+// since a wave's loads come back in the order it asked.  With the tile kernel's loads, stores into LDS and products
+// taken out one at a time, 2,048 tokens over 60 experts of 1,408 x 2,048 took 215 us without the products, 225
+// without the reads from LDS, 155 without the loads (248 whole); reads that hit in a die's L2 alone run at 31 TB/s,
+// three times what the tile kernel moves.  So two units per workgroup, for which an expert's matrices pass two
+// thirds as often, and the tiles straight from memory into a ring of three LDS stages (global_load_lds_dwordx4: no
+// registers in between, no stores into LDS by the waves), two of them on their way while the third is multiplied
+// (with one on its way the tiles alone took 205 us, with two 153).  A load instruction of a wave fills eight rows
+// of 128 bytes in LDS, lane l the l-th chunk of 16 bytes: the XOR swizzle of the tile kernel is therefore applied
+// to what a lane asks for, not to where it lands.  The ring leaves one workgroup to a compute unit; its barrier
+// is a bare s_barrier behind a wait for the wave's own loads of the tile that is due (a __syncthreads would wait
+// for the loads of the later tiles too).  Tried and slower: all reads of a step from LDS before its first product
+// (230 us against 209), a ring of four stages for w with the tiles of a asked for by waves of their own one step
+// ahead (247), the same with the tiles of a through registers (the compiler waits for every load before each store).
+// The sums of an output run over k in the same order as in the tile kernel: same bits.
+#define RING_STAGES 3
+__device__ __forceinline__ void load_to_lds16(const bf16_t* src, bf16_t* wave_base) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                   (__attribute__((address_space(3))) void*)wave_base, 16, 0, 0);
+}
+
+template <bool DUAL, bool OUT_ACT>
+__global__ __launch_bounds__(1024) void gemm_ring_kernel(MfmaGemmArgs g) {
+  constexpr int BM = 128, BH = 128;                  // rows of a; columns per half of the tile of w
+  constexpr int STAGE = (BM + 2 * BH) * TBK;         // elements of one stage
+  constexpr int L = 3;                               // loads per thread and stage: its chunk of a, of either half of w
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  bf16_t* ring = (bf16_t*)smem;
+  const int units_all = g.M / 64;
+  const int* items = g.tile_group + units_all;
+  const int n_units = min(g.n_tiles[0], units_all);
+  const int n_items = min(g.n_tiles[1], units_all);
+  // the items are dealt to the dies as the tile kernel deals an expert's row tiles: a die gets a contiguous run,
+  // expert by expert, within an expert column by column with the expert's items of a column side by side
+  int item, tile_n;
+  {
+    const int gy = gridDim.y, total = n_items * gy;
+    const int id = blockIdx.y * gridDim.x + blockIdx.x;
+    const int die = id % 8, q = total / 8, rem = total % 8;
+    if (id / 8 >= q + (die < rem ? 1 : 0)) return;
+    const int logical = die * q + min(die, rem) + id / 8;
+    const int p = logical / gy, e = g.tile_group[items[p]];
+    int lo = p, hi = p + 1;
+    while (lo > 0 && g.tile_group[items[lo - 1]] == e) --lo;
+    while (hi < n_items && g.tile_group[items[hi]] == e) ++hi;
+    const int local = logical - lo * gy, n_e = hi - lo;
+    tile_n = local / n_e;
+    item = lo + local % n_e;
+  }
+  const int u0 = items[item];
+  const int units = (item + 1 < n_items ? items[item + 1] : n_units) - u0 >= 2 ? 2 : 1;
+  const int group = g.tile_group[u0];
+  const bf16_t* w = g.w + (size_t)group * g.group_stride;
+  const bf16_t* w2 = DUAL ? g.w2 + (size_t)group * g.group_stride : w;
+  const int m0 = u0 * 64;
+  const int n0 = tile_n * (DUAL ? BH : 2 * BH);      // first column of the first half
+  const int n1 = DUAL ? n0 : n0 + BH;                // and of the second (the other matrix's same columns, or the next 128)
+  const int tid = threadIdx.x, lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
+  const int wm = wave / 4, wn = wave % 4;            // 4 x 4 waves, each 32 rows x 32 columns of either half
+  const int wave_m0 = m0 + wm * 32;
+  const bool active = wm < 2 * units && wave_m0 < g.M && (!g.a_rows || g.a_rows[wave_m0] >= 0);
+
+  // What this thread asks for of each stage: the chunk that belongs at place tid % 8 of row tid / 8 of the tile of a
+  // and of either half of w.  Rows past the end, rows of padding and the second unit's rows of an item of one read
+  // some valid row instead: those outputs are never stored.
+  const int row = tid / 8;
+  const int chunk = (tid % 8) ^ ((row >> 1) & 7);
+  const bf16_t *a_src, *w_src, *v_src;
+  {
+    const int m = min(m0 + (units == 2 ? row : row % 64), g.M - 1);
+    int src = m;
+    if (g.a_rows && g.a_gather) src = max(g.a_rows[m], 0);
+    a_src = g.a + (size_t)src * g.lda + chunk * 8;
+    w_src = w + (size_t)min(n0 + row, g.N - 1) * g.K + chunk * 8;
+    v_src = w2 + (size_t)min(n1 + row, g.N - 1) * g.K + chunk * 8;
+  }
+  const int wave_off = wave * 8 * TBK;               // the eight rows that a load of this wave fills
+#define TQ_ISSUE(stage, k0)                                                  \
+  do {                                                                       \
+    bf16_t* base = ring + (stage) * STAGE + wave_off;                        \
+    load_to_lds16(a_src + (k0), base);                                       \
+    load_to_lds16(w_src + (k0), base + BM * TBK);                            \
+    load_to_lds16(v_src + (k0), base + (BM + BH) * TBK);                     \
+  } while (0)
+
+  f32x16 acc, acc2;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] = 0.f, acc2[v] = 0.f;
+  const int steps = g.K / TBK;
+  for (int s = 0; s < RING_STAGES - 1 && s < steps; ++s) TQ_ISSUE(s, s * TBK);
+  const int lr = lane % 32, lc = lane / 32;
+  int cur = 0;
+  for (int t = 0; t < steps; ++t) {
+    // tile t is in LDS once no more loads of this wave are on their way than those of the tiles behind it
+    // (s_waitcnt: vmcnt in bits 3..0, nothing asked of the other counters)
+    if (t + 1 < steps) __builtin_amdgcn_s_waitcnt(0x0F70 | L);
+    else __builtin_amdgcn_s_waitcnt(0x0F70);
+    // every wave's share of tile t has landed and every wave is through with tile t - 1, whose stage tile t + 2 takes
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (t + RING_STAGES - 1 < steps) {
+      int nxt = cur + RING_STAGES - 1;
+      if (nxt >= RING_STAGES) nxt -= RING_STAGES;
+      TQ_ISSUE(nxt, (t + RING_STAGES - 1) * TBK);
+    }
+    if (active) {
+      const bf16_t* Ac = ring + cur * STAGE;
+      const bf16_t* Wc = Ac + BM * TBK;
+      const bf16_t* Vc = Wc + BH * TBK;
+#pragma unroll
+      for (int j = 0; j < TBK / 16; ++j) {
+        const bf16x8 af = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(Ac + swz(wm * 32 + lr, 2 * j + lc)));
+        const bf16x8 wf = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(Wc + swz(wn * 32 + lr, 2 * j + lc)));
+        const bf16x8 vf = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(Vc + swz(wn * 32 + lr, 2 * j + lc)));
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, wf, acc, 0, 0, 0);
+        acc2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, vf, acc2, 0, 0, 0);
+      }
+    }
+    if (++cur == RING_STAGES) cur = 0;
+  }
+#undef TQ_ISSUE
+  if (!active) return;
+  const int na = n0 + wn * 32 + lr, nb = n1 + wn * 32 + lr;
+  const float ba = na < g.N ? bias_at(g, na) : 0.f, bb = !DUAL && nb < g.N ? bias_at(g, nb) : 0.f;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int m = m0 + wm * 32 + 8 * (v / 4) + 4 * lc + (v % 4);
+    if (m >= g.M) continue;
+    if (g.a_rows && g.a_rows[m] < 0) continue;
+    if (DUAL) {
+      if (na < g.N) store_out<OUT_ACT>(g, m, na, gate_fn(acc[v] + ba, g.gate) * acc2[v]);
+    } else {
+      if (na < g.N) store_out<OUT_ACT>(g, m, na, acc[v] + ba);
+      if (nb < g.N) store_out<OUT_ACT>(g, m, nb, acc2[v] + bb);
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------------ launch
 // Waves that split k in the streaming kernel: a power of two, enough for about 2048 waves on the chip when one
 // matrix is multiplied and for about 256 per matrix when there is one per expert, each wave keeping at least 256 of
@@ -586,6 +729,26 @@ static int launch_tile(const MfmaGemmArgs& g, bool dual, bool out_act, int split
   else
     TQ_TILE(false, false);
 #undef TQ_TILE
+  return 0;
+}
+
+// grid (units of 64 rows: at most so many items, tiles of 256 columns: 128 of a gated pair)
+static int launch_ring(const MfmaGemmArgs& g, bool dual, bool out_act, hipStream_t st) {
+  const int cols = dual ? 128 : 256;
+  const dim3 grid(g.M / 64, (g.N + cols - 1) / cols);
+  const size_t shmem = (size_t)RING_STAGES * (128 + 256) * TBK * sizeof(bf16_t);
+#define TQ_RING(D, O)                                                                                              \
+  do {                                                                                                             \
+    if (hipFuncSetAttribute((const void*)gemm_ring_kernel<D, O>, hipFuncAttributeMaxDynamicSharedMemorySize,       \
+                            (int)shmem) != hipSuccess)                                                             \
+      return TQ_ERR_UNSUPPORTED;                                                                                   \
+    hipLaunchKernelGGL((gemm_ring_kernel<D, O>), grid, dim3(1024), shmem, st, g);                                  \
+  } while (0)
+  if (dual && out_act) TQ_RING(true, true);
+  else if (dual) TQ_RING(true, false);
+  else if (out_act) TQ_RING(false, true);
+  else TQ_RING(false, false);
+#undef TQ_RING
   return 0;
 }
 
@@ -681,7 +844,8 @@ TQ_API int tq_gemm_mfma_splits(int M, int N, int K) {
 
 // a: bfloat16 [.., K] with row stride lda (a multiple of 8, as K must be); w, w2: bfloat16.
 // tile_rows: with tile_group set, the padding unit of the row order (16, 32, 64, 128 or 256); else a hint that is
-// ignored.
+// ignored.  64 + TQ_TILE_PAIRS: units of 64 taken two at a time, by the items that the row order lists behind its
+// row tiles (tile_group[M / 64 ..], n_tiles[1]).
 // splits > 1 (as tq_gemm_mfma_splits says, for a plain product into float): run z of k goes to out + z * M * ldc,
 // the bias to run 0; the sum over the runs is the caller's.
 TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gather, const void* w, const void* w2,
@@ -706,9 +870,12 @@ TQ_API int tq_gemm_mfma(const void* a, int64_t lda, const int* a_rows, int a_gat
     } else if (tile_rows == 32) {      // the streaming kernel with two row tiles and two column tiles to a wave
       if (M % 32) return TQ_ERR_BAD_ARG;
       rc = launch_stream<2>(g, dual, out_act, M / 32, st);
-    } else if (tile_rows == 64) {
-      if ((N + TBN - 1) / TBN > 65535) return TQ_ERR_UNSUPPORTED;
-      rc = launch_tile<64, 2, 4>(g, dual, out_act, 1, st);
+    } else if (tile_rows == 64 || tile_rows == 64 + TQ_TILE_PAIRS) {
+      if ((N + TBN - 1) / TBN > 65535 || M % 64) return TQ_ERR_UNSUPPORTED;
+      if (tile_rows != 64 && K % TBK == 0 && K >= 2 * TBK)
+        rc = launch_ring(g, dual, out_act, st);
+      else
+        rc = launch_tile<64, 2, 4>(g, dual, out_act, 1, st);
     } else if (tile_rows == 128) {     // experts with hundreds of rows each: the taller tile's rate for little padding
       if ((N + TBN - 1) / TBN > 65535 || M % 128) return TQ_ERR_UNSUPPORTED;
       // the gated pair as 2 x 4 waves of 64 x 32 outputs (and as many of w2): 3 to 4 % faster than 4 x 2 of 32 x 64

@@ -142,6 +142,7 @@ int product(Ctx& c, const Product& p, void** out, int* splits, int side = 0) {
   const bool grouped = p.tile_group != nullptr;
   const size_t esz = p.out_act ? TQ_ACT_BYTES : 4;
   const int tile_rows = p.tile_rows ? p.tile_rows : (p.M <= 32 ? 16 : 64);
+  const int unit_rows = tile_rows % TQ_TILE_PAIRS;      // pairs of units are the matrix-core product's alone
   *splits = 1;
   auto result = [&](size_t bytes) { return p.dest ? p.dest : c.arena.take(bytes); };
   if (!grouped && !p.a_rows && !p.bias.ptr && vendor_product(c, p)) {
@@ -181,7 +182,7 @@ int product(Ctx& c, const Product& p, void** out, int* splits, int side = 0) {
   }
 #else
   if (p.w.wtype == TQ_F32 && p.K % 4 == 0 && p.lda % 4 == 0 && p.gstride % 4 == 0 && ((uintptr_t)p.w.ptr & 15) == 0 &&
-      ((uintptr_t)p.w2 & 15) == 0 && (tile_rows == 16 || tile_rows == 64)) {
+      ((uintptr_t)p.w2 & 15) == 0 && (unit_rows == 16 || unit_rows == 64)) {
     const int runs = tq_gemm_f32_runs(p.M, p.N, p.K, grouped || p.a_rows != nullptr);
     if (p.partial) *splits = runs;
     *out = result((size_t)*splits * p.M * p.N * 4);
@@ -189,7 +190,7 @@ int product(Ctx& c, const Product& p, void** out, int* splits, int side = 0) {
     if (runs > 1 && !p.partial) scratch = c.arena.take((size_t)runs * (p.w2 ? 2 : 1) * p.M * p.N * 4);
     RUN(c, "gemm_f32",
         tq_gemm_f32(p.a, p.lda, p.a_rows, p.gather, p.w.ptr, p.w2, p.gstride, p.tile_group, p.n_tiles, p.bias.ptr,
-                    (int)p.bias.wtype, *out, p.N, p.M, p.N, p.K, tile_rows, p.gate, scratch, p.partial && runs > 1,
+                    (int)p.bias.wtype, *out, p.N, p.M, p.N, p.K, unit_rows, p.gate, scratch, p.partial && runs > 1,
                     c.stream));
     return 0;
   }
@@ -197,7 +198,7 @@ int product(Ctx& c, const Product& p, void** out, int* splits, int side = 0) {
   *out = result((size_t)p.M * p.N * esz);
   RUN(c, "gemm",
       tq_gemm_generic(p.a, p.lda, p.a_rows, p.gather, p.w.ptr, p.w2, (int)p.w.wtype, p.gstride, p.tile_group, p.n_tiles,
-                      p.bias.ptr, (int)p.bias.wtype, *out, p.N, p.out_act, p.M, p.N, p.K, tile_rows, p.gate, c.stream));
+                      p.bias.ptr, (int)p.bias.wtype, *out, p.N, p.out_act, p.M, p.N, p.K, unit_rows, p.gate, c.stream));
   return 0;
 }
 
@@ -352,7 +353,7 @@ int dense_ffn(Ctx& c, const tq_dense_ffn_desc& f, const void* normed, Pending* p
 int expert_tile_rows(const Ctx& c, int64_t n_pairs, int64_t E, bool mfma) {
   if (n_pairs <= (mfma ? 5 : 12) * E) return 16;
   if (mfma && n_pairs <= 10 * E) return 32;
-  if (mfma && n_pairs >= 256 * E) return n_pairs >= c.s->expert_256_from * E ? 256 : 128;
+  if (mfma && n_pairs >= c.s->expert_128_from * E) return n_pairs >= c.s->expert_256_from * E ? 256 : 128;
   return 64;
 }
 
@@ -374,21 +375,23 @@ int moe_ffn(Ctx& c, const tq_moe_ffn_desc& f, const void* normed, const float* n
   float* logits = (float*)c.arena.take((size_t)T * (E + (gated ? 1 : 0)) * 4);
   int* sorted_token = (int*)c.arena.take((size_t)cap * 4);
   int* pair_slot = (int*)c.arena.take((size_t)n_pairs * 4);
-  int* tile_expert = (int*)c.arena.take((size_t)(cap / unit) * 4);
-  int* n_tiles = (int*)c.arena.take(4);
+  int* tile_expert = (int*)c.arena.take((size_t)(cap / unit) * 2 * 4);      // row tiles, then items of two
+  int* n_tiles = (int*)c.arena.take(2 * 4);
   auto route = [&]() -> int {
     RUN(c, "route",
         tq_route(normed32, f.router.ptr, gated ? f.shared_scale.ptr : nullptr, (int)f.router.wtype, E, k, (int)f.renormalize,
                  ids, weights, gate, logits, unit, (int)cap, sorted_token, pair_slot, tile_expert, n_tiles, T, H, c.stream));
     return 0;
   };
+  // what the products are told: units of 64 two at a time where experts have that many rows (ops.expert_product_rows)
+  const int rows = unit == 64 && n_pairs >= s.expert_pairs_from * E ? 64 + TQ_TILE_PAIRS : unit;
   Product eg;       // the experts' gated pair over the gathered rows
   eg.a = normed, eg.lda = H, eg.a_rows = sorted_token, eg.w = f.expert_gate, eg.w2 = f.expert_up.ptr, eg.gstride = (int64_t)I * H,
-  eg.tile_group = tile_expert, eg.n_tiles = n_tiles, eg.out_act = 1, eg.M = (int)cap, eg.N = I, eg.K = H, eg.tile_rows = unit,
+  eg.tile_group = tile_expert, eg.n_tiles = n_tiles, eg.out_act = 1, eg.M = (int)cap, eg.N = I, eg.K = H, eg.tile_rows = rows,
   eg.gate = (int)f.gate;
   Product ed;       // their down product, row for row
   ed.lda = I, ed.a_rows = sorted_token, ed.gather = 0, ed.w = f.expert_down, ed.gstride = (int64_t)H * I, ed.tile_group = tile_expert,
-  ed.n_tiles = n_tiles, ed.M = (int)cap, ed.N = H, ed.K = I, ed.tile_rows = unit;
+  ed.n_tiles = n_tiles, ed.M = (int)cap, ed.N = H, ed.K = I, ed.tile_rows = rows;
   Product sg;       // the shared expert
   sg.a = normed, sg.lda = H, sg.w = f.shared_gate, sg.w2 = f.shared_up.ptr, sg.out_act = 1, sg.M = T, sg.N = Is, sg.K = H,
   sg.gate = (int)f.gate;

@@ -109,10 +109,10 @@ typedef struct {
   int64_t decode;         // every sequence brings one token
   int64_t capturing;      // the step is being recorded into a graph
   // tuning that the caller owns: plain products of vendor_min_rows rows and more may go to the vendor's matrix
-  // library (0: never); gated pairs go there vendor_gated_rows at a time; experts take units of 256 rows from
-  // expert_256_from rows per expert on average; an eager step of side_from tokens and more runs the shared expert
-  // on the side stream
-  int64_t vendor_min_rows, vendor_gated_rows, expert_256_from, side_from;
+  // library (0: never); gated pairs go there vendor_gated_rows at a time; experts take units of 128 rows from
+  // expert_128_from rows per expert on average, of 256 from expert_256_from, and units of 64 two at a time from
+  // expert_pairs_from; an eager step of side_from tokens and more runs the shared expert on the side stream
+  int64_t vendor_min_rows, vendor_gated_rows, expert_128_from, expert_256_from, expert_pairs_from, side_from;
   const int* tokens;          // [T]
   const int* positions;       // [T]
   const int* slot_of_token;   // [T]

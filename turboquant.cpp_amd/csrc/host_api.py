@@ -59,8 +59,8 @@ class ModelDesc(ctypes.Structure):
 
 class StepDesc(ctypes.Structure):
     _fields_ = [("T", i64), ("B", i64), ("n_want", i64), ("max_new", i64), ("max_end", i64), ("decode", i64),
-                ("capturing", i64), ("vendor_min_rows", i64), ("vendor_gated_rows", i64), ("expert_256_from", i64),
-                ("side_from", i64), ("tokens", ptr), ("positions", ptr), ("slot_of_token", ptr), ("cu_seqlens", ptr),
+                ("capturing", i64), ("vendor_min_rows", i64), ("vendor_gated_rows", i64), ("expert_128_from", i64),
+                ("expert_256_from", i64), ("expert_pairs_from", i64), ("side_from", i64), ("tokens", ptr), ("positions", ptr), ("slot_of_token", ptr), ("cu_seqlens", ptr),
                 ("slots", ptr), ("start", ptr), ("want_rows", ptr), ("workspace", ptr), ("workspace_bytes", i64),
                 ("logits", ptr), ("stream", ptr), ("side_stream", ptr)]
 

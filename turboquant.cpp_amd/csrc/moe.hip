@@ -270,6 +270,9 @@ TQ_API int tq_router_topk(const float* x, const void* wr, const void* shared_w, 
 //   sorted_token[r]  token whose activations feed row r, or -1
 //   pair_slot[i]     row of pair i
 //   tile_expert[j]   expert of row tile j (tiles of `unit` rows), n_tiles[0] tiles in all
+//   tile_expert[cap / unit + p]   first row tile of item p, n_tiles[1] items in all: an expert's row tiles two at a
+//                    time (its last one alone when their number is odd), for the product that takes two tiles of
+//                    one expert per workgroup; item p ends where item p + 1 begins, the last one at n_tiles[0]
 // One workgroup of 16 waves does all of it.  Wave w owns the w-th sixteenth of the pairs: it goes through
 // them 64 at a time, finds for every lane the lanes that hold the same expert (a ballot per bit of the expert's
 // number), gives it its rank among them in order of lane and adds their number to its count of the expert.
@@ -333,22 +336,36 @@ __device__ __forceinline__ void align_pairs(const int* ids, int n_pairs, int E, 
   if (wave == 0) {      // exclusive scan of the padded sizes: each lane a contiguous run of experts
     const int chunk = (E + TQ_WAVE - 1) / TQ_WAVE;
     const int e0 = lane * chunk, e1 = min(E, e0 + chunk);
-    int sum = 0;
-    for (int e = e0; e < e1; ++e) sum += starts[e];
-    int incl = sum;
+    int sum = 0, isum = 0;
+    for (int e = e0; e < e1; ++e) {
+      sum += starts[e];
+      isum += (starts[e] / unit + 1) / 2;
+    }
+    int incl = sum, iincl = isum;
 #pragma unroll
     for (int o = 1; o < TQ_WAVE; o <<= 1) {
       const int up = __shfl_up(incl, o, TQ_WAVE);
-      if (lane >= o) incl += up;
+      const int iup = __shfl_up(iincl, o, TQ_WAVE);
+      if (lane >= o) {
+        incl += up;
+        iincl += iup;
+      }
     }
-    int row = incl - sum;
+    int row = incl - sum, item = iincl - isum;
+    int* items = tile_expert + cap / unit;
     for (int e = e0; e < e1; ++e) {
       const int padded = starts[e];
       starts[e] = row;
-      for (int j = 0; j < padded / unit; ++j) tile_expert[row / unit + j] = e;
+      for (int j = 0; j < padded / unit; ++j) {
+        tile_expert[row / unit + j] = e;
+        if (j % 2 == 0) items[item++] = row / unit + j;
+      }
       row += padded;
     }
-    if (lane == TQ_WAVE - 1) n_tiles[0] = incl / unit;
+    if (lane == TQ_WAVE - 1) {
+      n_tiles[0] = incl / unit;
+      n_tiles[1] = iincl;
+    }
   }
   __syncthreads();
   if (one_batch) {
@@ -402,7 +419,7 @@ __global__ __launch_bounds__(64 * NW) void select_align_kernel(const float* __re
 }
 
 // cap: rows that sorted_token holds, a multiple of unit and at least n_pairs + min(E, n_pairs) * (unit - 1);
-// tile_expert holds cap / unit entries.
+// tile_expert holds 2 * cap / unit entries (row tiles, then items), n_tiles two.
 TQ_API int tq_moe_align(const int* ids, int n_pairs, int E, int topk, int unit, int cap, int* sorted_token,
                         int* pair_slot, int* tile_expert, int* n_tiles, hipStream_t st) {
   if (n_pairs <= 0) return 0;

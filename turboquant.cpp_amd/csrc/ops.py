@@ -457,8 +457,12 @@ def _use_mfma(act, a: torch.Tensor, w: torch.Tensor, K: int) -> bool:
             and has_kernel(act, "tq_gemm_mfma"))
 
 
-EXPERT_256_FROM = 1024
 EXPERT_16_UPTO, EXPERT_32_UPTO = 5, 10
+# Rows per expert on average from which the row order's unit is 128 and 256: never, since units of 64 taken two at a
+# time do better wherever the taller units did (see expert_tile_rows); tests lower them to run those kernels.
+EXPERT_128_FROM = EXPERT_256_FROM = 1 << 30
+TILE_PAIRS = 1024            # added to tile_rows 64: two units of one expert per workgroup (TQ_TILE_PAIRS)
+EXPERT_PAIRS_FROM = 64       # rows per expert on average from which units of 64 are taken two at a time
 
 
 def expert_tile_rows(n_pairs: int, num_experts: int, act, a: torch.Tensor, w: torch.Tensor) -> int:
@@ -472,17 +476,30 @@ def expert_tile_rows(n_pairs: int, num_experts: int, act, a: torch.Tensor, w: to
     to 6 rows per expert (64 experts, 8 per token: up to 12) and tiles of 64 rows win by 10 to 18 % from 12 on, since a
     crowded expert's matrices pass the streaming kernel once per unit.  The borders here lose at most 6 % either way (a replayed decode step of 64 sequences, 4.3 rows per expert, is 2 %
     faster with units of 16 than of 32).
-    Without the matrix-core product 16 up to 12.  From 256: 128 (the taller tile is 8 to 17 % faster there and slower
-    below; at 137 rows per expert it lost 35 %); from 1,024: 256 (the gated pair in tiles of 256 rows is 8 to 14 %
-    faster there, the second product keeps tiles of 128: both together 4 to 8 %)."""
+    Without the matrix-core product 16 up to 12.  Units of 128 and 256 rows (EXPERT_128_FROM, EXPERT_256_FROM) are
+    not chosen: they were 8 to 17 % faster than single tiles of 64 rows from 256 rows per expert on, but units of 64
+    taken two at a time (expert_product_rows) are faster than either (60 experts of 1,408 x 2,048, both products:
+    396 us against 448 at 205 rows per expert, 492 against 565 at 273, 841 against 949 at 546; 64 experts of
+    2,560 x 3,584 at 1,650 rows each: a prompt step of 425 ms against 436 with units of 256)."""
     mfma = _use_mfma(act, a, w, a.shape[1])
     if n_pairs <= (EXPERT_16_UPTO if mfma else 12) * num_experts:
         return 16
     if mfma and n_pairs <= EXPERT_32_UPTO * num_experts:
         return 32
-    if n_pairs >= 256 * num_experts and mfma:
+    if mfma and n_pairs >= EXPERT_128_FROM * num_experts:
         return 256 if n_pairs >= EXPERT_256_FROM * num_experts else 128
     return 64
+
+
+def expert_product_rows(unit: int, n_pairs: int, num_experts: int) -> int:
+    """The ``tile_rows`` that a product over experts is called with when the row order has units of ``unit`` rows: from
+    64 rows per expert on average, units of 64 two at a time (measured on 60 experts of 1,408 x 2,048, four per
+    token, both products together: 251 us against 286 at 68 rows per expert, 260 against 307 at 102, 346 against 360
+    at 137; level below; a prompt step of 24 layers: 10.3 ms against 10.9 at 1,024 tokens, 15.8 against 17.0 at
+    2,048, 22.3 against 23.7 at 3,072)."""
+    if unit == 64 and n_pairs >= EXPERT_PAIRS_FROM * num_experts:
+        return 64 + TILE_PAIRS
+    return unit
 
 
 def _gemm_problem(k: str, a, w, act, bias, w2, out_act, a_rows, tile_group, n_tiles, tile_rows, gather):
@@ -495,15 +512,19 @@ def _gemm_problem(k: str, a, w, act, bias, w2, out_act, a_rows, tile_group, n_ti
     grouped = tile_group is not None
     if grouped:
         _need(w.dim() == 3 and w.shape[2] == K, k, lambda: f"grouped w must be [G, N, {K}], is {tuple(w.shape)}")
-        _need(a_rows is not None and n_tiles is not None and tile_rows in (16, 32, 64, 128, 256), k,
+        _need(a_rows is not None and n_tiles is not None and tile_rows in (16, 32, 64, 128, 256, 64 + TILE_PAIRS), k,
               "grouped product needs a_rows, n_tiles and tile_rows of 16, 64, 128 or 256")
-        _need(tile_rows in (16, 64) or _use_mfma(act, a, w, a.shape[1]), k,
-              "tiles of 32, 128 and 256 rows are for the bfloat16 matrix-core product")
+        if not _use_mfma(act, a, w, a.shape[1]):
+            _need(tile_rows % TILE_PAIRS in (16, 64), k, "tiles of 32, 128 and 256 rows are for the bfloat16 matrix-core product")
+            tile_rows %= TILE_PAIRS      # pairs of units are that product's too: the others take unit by unit
         _check(a_rows, k, "a_rows", torch.int32)
         _check(tile_group, k, "tile_group", torch.int32)
         _check(n_tiles, k, "n_tiles", torch.int32)
         M = a_rows.numel()
-        _need(M % tile_rows == 0 and tile_group.numel() >= M // tile_rows, k, "a_rows must hold whole tiles, each with a group")
+        unit = tile_rows % TILE_PAIRS
+        _need(M % unit == 0 and tile_group.numel() >= M // unit, k, "a_rows must hold whole tiles, each with a group")
+        _need(tile_rows == unit or (tile_group.numel() >= 2 * (M // unit) and n_tiles.numel() >= 2), k,
+              "pairs of tiles need the items behind the row tiles (tile_group [2 M / 64], n_tiles [2])")
         N = w.shape[1]
         gstride = N * K
     else:
@@ -832,8 +853,8 @@ def _align_outputs(T: int, topk: int, num_experts: int, unit: int, dev):
     cap = (cap + unit - 1) // unit * unit
     sorted_token = torch.empty((cap,), dtype=torch.int32, device=dev)
     pair_slot = torch.empty((T, topk), dtype=torch.int32, device=dev)
-    tile_expert = torch.empty((cap // unit,), dtype=torch.int32, device=dev)
-    n_tiles = torch.empty((1,), dtype=torch.int32, device=dev)
+    tile_expert = torch.empty((2 * (cap // unit),), dtype=torch.int32, device=dev)      # row tiles, then items of two
+    n_tiles = torch.empty((2,), dtype=torch.int32, device=dev)
     return cap, sorted_token, pair_slot, tile_expert, n_tiles
 
 

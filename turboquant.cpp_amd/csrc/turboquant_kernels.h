@@ -14,6 +14,8 @@
 
 #define TQ_ERR_BAD_ARG (-1)
 #define TQ_ERR_UNSUPPORTED (-2)
+// added to a tile_rows of 64 of a product over experts: two units of one expert per workgroup (see tq_gemm_mfma)
+#define TQ_TILE_PAIRS 1024
 
 #ifdef __cplusplus
 extern "C" {

@@ -68,7 +68,8 @@ class NativeModel:
         side = ctx.side_stream
         step = host_api.StepDesc(
             b.n_tokens, b.n_seqs, b.n_want, b.max_new, b.max_end, int(b.is_decode), int(bool(ctx.capturing)),
-            ops.VENDOR_MIN_ROWS if ops._VENDOR else 0, ops.VENDOR_GATED_ROWS, ops.EXPERT_256_FROM, ffn_parts.SIDE_STREAM_FROM,
+            ops.VENDOR_MIN_ROWS if ops._VENDOR else 0, ops.VENDOR_GATED_ROWS, ops.EXPERT_128_FROM, ops.EXPERT_256_FROM, ops.EXPERT_PAIRS_FROM,
+            ffn_parts.SIDE_STREAM_FROM_IN_EXECUTOR,
             b.tokens.data_ptr(), b.positions.data_ptr(), b.slot_of_token.data_ptr(), b.cu_seqlens.data_ptr(),
             b.slots_dev.data_ptr(), b.start_dev.data_ptr(), b.want_rows.data_ptr() if b.n_want else None, None, 0,
             logits.data_ptr() if b.n_want else None, ops._stream(), side.cuda_stream if side is not None else None)
