@@ -24,7 +24,7 @@ SOURCES = {
     "float32": COMMON_SOURCES + ["gemm_f32.hip", "attention_f32.hip"],
     "bfloat16": COMMON_SOURCES + ["gemm_mfma.hip", "attention_mfma.hip", "probe.hip"],
 }
-HEADERS = ["common.h", "no_alloc.h", "gemm_mfma.h", "turboquant_kernels.h", "host/engine.h", "host/vendor.h",
+HEADERS = ["common.h", "gates.def", "no_alloc.h", "gemm_mfma.h", "turboquant_kernels.h", "host/engine.h", "host/vendor.h",
            "host/host_common.h"]
 DEFINES = {"float32": "-DTQ_ACT_F32", "bfloat16": "-DTQ_ACT_BF16"}
 FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-fno-gpu-rdc",
@@ -159,7 +159,7 @@ def build(dtype: str, force: bool = False, verbose: bool = True) -> str:
     return target
 
 
-RUNNER_SOURCES = ["host/quant_main.cpp", "host/engine.h"]
+RUNNER_SOURCES = ["host/quant_main.cpp", "host/engine.h", "gates.def"]
 
 
 def runner_name() -> str:

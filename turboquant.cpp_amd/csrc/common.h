@@ -92,18 +92,23 @@ __device__ __forceinline__ float block_max(float v, float* red) {
   return t;
 }
 
-// Activation of the gate in a gated pair act(a w^T) * (a w2^T); a parameter of the products' epilogues.
-// silu: x / (1 + exp(-x)) with an exact exponential (/root/reference/src/engine/tq_ops.c:1454-1478);
-// gelu_tanh: 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))) (tq_ops.c:1482-1484); relu2: max(x, 0)^2.
-#define TQ_GATE_SILU 0
-#define TQ_GATE_GELU_TANH 1
-#define TQ_GATE_RELU2 2
-#define TQ_GATE_COUNT 3
+// Activation of the gate in a gated pair act(a w^T) * (a w2^T); a parameter of the products' epilogues, numbered in
+// the order of the list in gates.def.
+enum {
+#define TQ_GATE(name, expr) TQ_GATE_##name,
+#include "gates.def"
+#undef TQ_GATE
+  TQ_GATE_COUNT
+};
 __device__ __forceinline__ float gate_fn(float x, int kind) {
-  if (kind == TQ_GATE_SILU) return x / (1.0f + expf(-x));
-  if (kind == TQ_GATE_GELU_TANH) return 0.5f * x * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
-  const float r = fmaxf(x, 0.f);
-  return r * r;
+  switch (kind) {
+#define TQ_GATE(name, expr) \
+  case TQ_GATE_##name:      \
+    return (expr);
+#include "gates.def"
+#undef TQ_GATE
+  }
+  return x;
 }
 
 #define TQ_LAUNCH_CHECK()                        \

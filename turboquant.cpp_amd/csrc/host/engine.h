@@ -44,7 +44,7 @@ typedef struct {
 
 typedef struct {
   int64_t hidden, inner;
-  int64_t gate;           // activation of the gate: 0 silu, 1 gelu_tanh, 2 relu2
+  int64_t gate;           // activation of the gate, numbered by its line in gates.def
   tq_weight gate_w, up_w; // [inner, hidden] each; up_w right behind gate_w in memory lets long prompts take one product
   tq_weight down_w;       // [hidden, inner]
 } tq_dense_ffn_desc;

@@ -446,10 +446,14 @@ std::vector<std::vector<int>> parse_prompts(const std::string& text) {
   return prompts;
 }
 
-int gate_code(const std::string& name) {
-  if (name == "silu") return 0;
-  if (name == "gelu_tanh") return 1;
-  if (name == "relu2") return 2;
+int gate_code(const std::string& name) {      // numbered by the lines of gates.def, as the kernels number them
+  static const char* const names[] = {
+#define TQ_GATE(gate, expr) #gate,
+#include "../gates.def"
+#undef TQ_GATE
+  };
+  for (size_t i = 0; i < sizeof(names) / sizeof(names[0]); ++i)
+    if (name == names[i]) return (int)i;
   die("plan: unknown activation " + name);
 }
 

@@ -11,6 +11,7 @@ import ctypes
 import dataclasses
 import math
 import os
+import re
 
 import torch
 
@@ -22,7 +23,9 @@ class KernelError(RuntimeError):
 
 
 ACT_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
-GATES = {"silu": 0, "gelu_tanh": 1, "relu2": 2}      # activations of the gate in a gated pair of products
+# activations of the gate in a gated pair of products: the lines of gates.def, numbered as the kernels number them
+with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "gates.def"), encoding="utf-8") as _f:
+    GATES = {name: i for i, name in enumerate(re.findall(r"^TQ_GATE\((\w+),", _f.read(), re.M))}
 _WTYPE = {torch.float32: 0, torch.bfloat16: 1}
 _LIBS: dict[str, ctypes.CDLL] = {}
 

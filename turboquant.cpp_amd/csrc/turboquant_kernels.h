@@ -6,7 +6,7 @@
 // comment in front of each definition in the .hip file named here says what the arguments mean; the Python face
 // (ops.py) checks shapes, types and strides before every call and is the reference for how to call them.
 // Weight types: TQ_F32 0, TQ_BF16 1.  Activations are bfloat16 in the bfloat16 library and float in the float32
-// library (written `void*` here).  Gate activations: 0 silu, 1 gelu_tanh, 2 relu2.
+// library (written `void*` here).  Gate activations: numbered by their lines in gates.def (0 silu, 1 gelu_tanh, 2 relu2).
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
