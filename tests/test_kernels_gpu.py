@@ -345,6 +345,39 @@ def test_the_height_of_expert_tiles(ops, monkeypatch):
     assert ops.expert_tile_rows(60 * 256, 60, "bfloat16", a16, w32) == 64      # float32 weights: the plain product
 
 
+@pytest.mark.parametrize("H,I", [(128, 256), (192, 1408), (256, 72)])
+def test_units_two_at_a_time_with_a_crowded_expert(ops, H, I):
+    """Units of 64 rows taken two at a time when the router sends nearly every token to one expert: that expert has
+    many items, its neighbours one row or none, an expert's last unit stands alone where their number is odd, and the
+    last column tile is not full (72 columns; a k of 72 falls back to the tile kernel).  Against sums in double, and
+    bit for bit what the same units give one by one."""
+    act, T, E, k = "bfloat16", 601, 5, 2
+    ids = torch.empty((T, k), dtype=torch.int32)
+    ids[:, 0] = 3                                  # the crowded expert: ten units, five items
+    ids[:, 1] = torch.where(torch.arange(T) % 150 == 0, 1, 4).to(torch.int32)      # expert 1: five rows; 4: the rest
+    ids[7, 1], ids[7, 0] = 0, 4                    # expert 0: one row; expert 2: none
+    x = rnd((T, H), adt(act), 45)
+    wg, wu, wd = rnd((E, I, H), adt(act), 46, 0.2), rnd((E, I, H), adt(act), 47, 0.2), rnd((E, H, I), adt(act), 48, 0.2)
+    st, slot, te, nt = ops.moe_align(ids.to(DEV), E, 64, act)
+    units, items = nt.tolist()
+    assert units == 1 + 1 + 10 + 10 and items == 1 + 1 + 5 + 5
+    out = {}
+    for rows in (64, 64 + 1024):
+        h = ops.gemm(x.to(DEV), wg.to(DEV), act, w2=wu.to(DEV), out_act=True, a_rows=st, tile_group=te, n_tiles=nt, tile_rows=rows)
+        y = ops.gemm(h, wd.to(DEV), act, a_rows=st, tile_group=te, n_tiles=nt, tile_rows=rows, gather=False)
+        out[rows] = (h.cpu(), y.cpu())
+    live = (st >= 0).cpu()
+    assert torch.equal(out[64][0][live], out[64 + 1024][0][live]) and torch.equal(out[64][1][live], out[64 + 1024][1][live])
+    hc, y = out[64 + 1024]
+    for t in (0, 7, 150, 300, 600):
+        for j in range(k):
+            e, r = int(ids[t, j]), int(slot[t, j])
+            href = ref_gemm(x[t:t + 1], wg[e], w2=wu[e])[0]
+            assert (hc[r].double() - href).abs().max() < tol(act, 2) * max(1.0, href.abs().max().item())
+            yref = hc[r:r + 1].double() @ wd[e].double().T
+            assert (y[r].double() - yref[0]).abs().max() < tol(act, 2) * max(1.0, yref.abs().max().item())
+
+
 @pytest.mark.parametrize("act", ACTS)
 @pytest.mark.parametrize("unit", [16, 32, 64, 128, 256, 64 + 1024])
 @pytest.mark.parametrize("T,E,k,H,I", [(1, 5, 2, 72, 40), (9, 7, 3, 136, 88), (150, 6, 2, 64, 200), (700, 3, 2, 64, 136),
