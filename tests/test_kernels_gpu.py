@@ -320,7 +320,7 @@ def test_gemm_rows_do_not_depend_on_the_batch(ops, act):
 
 def test_the_height_of_expert_tiles(ops, monkeypatch):
     """16 up to 5 pairs per expert and 32 up to 10 where the bfloat16 matrix-core product runs (else 16 up to 12), 64
-    beyond, which the products take two at a time from 64 rows per expert on; 128 and 256 only where their borders
+    beyond, which the products take two at a time from 48 rows per expert on; 128 and 256 only where their borders
     are lowered, and only for the bfloat16 matrix-core product."""
     a16, w16 = torch.zeros((1, 64), dtype=torch.bfloat16), torch.zeros((1, 8, 64), dtype=torch.bfloat16)
     a32, w32 = a16.float(), w16.float()
@@ -331,8 +331,8 @@ def test_the_height_of_expert_tiles(ops, monkeypatch):
     assert ops.expert_tile_rows(60 * 12, 60, "float32", a32, w32) == 16
     assert ops.expert_tile_rows(60 * 12 + 1, 60, "float32", a32, w32) == 64
     assert ops.expert_tile_rows(60 * 100000, 60, "bfloat16", a16, w16) == 64
-    assert ops.expert_product_rows(64, 60 * 64 - 1, 60) == 64
-    assert ops.expert_product_rows(64, 60 * 64, 60) == 64 + ops.TILE_PAIRS
+    assert ops.expert_product_rows(64, 60 * 48 - 1, 60) == 64
+    assert ops.expert_product_rows(64, 60 * 48, 60) == 64 + ops.TILE_PAIRS
     assert ops.expert_product_rows(16, 60 * 64, 60) == 16 and ops.expert_product_rows(256, 60 * 2000, 60) == 256
     monkeypatch.setattr(ops, "EXPERT_128_FROM", 256)
     monkeypatch.setattr(ops, "EXPERT_256_FROM", 1024)

@@ -671,7 +671,7 @@ int main(int argc, char** argv) {
     tq_step_desc step;
     memset(&step, 0, sizeof(step));
     step.T = T, step.B = B, step.n_want = B, step.max_new = max_new_here, step.max_end = max_end, step.decode = max_new_here == 1;
-    step.expert_128_from = step.expert_256_from = 1 << 30, step.expert_pairs_from = 64, step.side_from = 1 << 30;      // own kernels for every product, one stream
+    step.expert_128_from = step.expert_256_from = 1 << 30, step.expert_pairs_from = 48, step.side_from = 1 << 30;      // own kernels for every product, one stream
     step.tokens = ints, step.positions = ints + T, step.slot_of_token = ints + 2 * T, step.cu_seqlens = ints + 3 * T;
     step.slots = ints + 3 * T + B + 1, step.start = ints + 3 * T + 2 * B + 1, step.want_rows = ints + 3 * T + 3 * B + 1;
     step.logits = logits, step.stream = stream;

@@ -465,7 +465,7 @@ EXPERT_16_UPTO, EXPERT_32_UPTO = 5, 10
 # time do better wherever the taller units did (see expert_tile_rows); tests lower them to run those kernels.
 EXPERT_128_FROM = EXPERT_256_FROM = 1 << 30
 TILE_PAIRS = 1024            # added to tile_rows 64: two units of one expert per workgroup (TQ_TILE_PAIRS)
-EXPERT_PAIRS_FROM = 64       # rows per expert on average from which units of 64 are taken two at a time
+EXPERT_PAIRS_FROM = 48       # rows per expert on average from which units of 64 are taken two at a time
 
 
 def expert_tile_rows(n_pairs: int, num_experts: int, act, a: torch.Tensor, w: torch.Tensor) -> int:
@@ -496,10 +496,12 @@ def expert_tile_rows(n_pairs: int, num_experts: int, act, a: torch.Tensor, w: to
 
 def expert_product_rows(unit: int, n_pairs: int, num_experts: int) -> int:
     """The ``tile_rows`` that a product over experts is called with when the row order has units of ``unit`` rows: from
-    64 rows per expert on average, units of 64 two at a time (measured on 60 experts of 1,408 x 2,048, four per
+    48 rows per expert on average, units of 64 two at a time (measured on 60 experts of 1,408 x 2,048, four per
     token, both products together: 251 us against 286 at 68 rows per expert, 260 against 307 at 102, 346 against 360
     at 137; level below; a prompt step of 24 layers: 10.3 ms against 10.9 at 1,024 tokens, 15.8 against 17.0 at
-    2,048, 22.3 against 23.7 at 3,072)."""
+    2,048, 22.3 against 23.7 at 3,072; where the border lies, by such steps: 9.42 ms against 9.73 at 55 rows per
+    expert and 9.75 against 10.22 at 60, which already gives many experts a second unit, level at 43 and 47, 7.97
+    against 7.81 at 34)."""
     if unit == 64 and n_pairs >= EXPERT_PAIRS_FROM * num_experts:
         return 64 + TILE_PAIRS
     return unit
