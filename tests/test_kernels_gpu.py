@@ -621,6 +621,36 @@ def test_routing_in_one_call(ops, act, E, k, H, renorm, shared):
             assert torch.equal(got[5][:n], want[2][:n]) and torch.equal(got[5][half:half + items], want[2][half:half + items])
 
 
+@pytest.mark.parametrize("T,E,k,H,unit,skew", [(2048, 60, 4, 128, 64, False), (2500, 60, 4, 128, 64, True), (3000, 5, 3, 72, 16, False),
+                                                (1100, 130, 8, 64, 64, False), (40000, 64, 8, 64, 64, True)])
+def test_order_by_several_workgroups(ops, T, E, k, H, unit, skew):
+    """From 8,192 pairs on ``route`` orders the pairs with several workgroups (three launches, its table in the logits'
+    memory) where ``moe_align`` has one workgroup go through them: the same rows, tiles and items, also when most
+    tokens choose the same experts and when the last workgroup's waves have nothing left."""
+    act = "bfloat16"
+    x = rnd((T, H), torch.float32, 71)
+    if skew:
+        x[: T - T // 7] = x[0] + 0.01 * x[: T - T // 7]      # nearly the same logits for six tokens in seven
+    x = x.to(DEV)
+    wr = rnd((E, H), adt(act), 72).to(DEV)
+    sg = rnd((1, H), adt(act), 73, 0.1).to(DEV)
+    assert T * k >= 8192
+    ids, w, gate = ops.router_topk(x, wr, sg, k, False, act)
+    want = ops.moe_align(ids, E, unit, act)
+    got = ops.route(x, wr, sg, k, False, unit, act)
+    assert torch.equal(got[0], ids) and torch.equal(got[1], w) and torch.equal(got[2], gate)
+    n, items = want[3].tolist()
+    half = want[2].numel() // 2
+    assert torch.equal(got[3], want[0]) and torch.equal(got[4], want[1]) and torch.equal(got[6], want[3])
+    assert torch.equal(got[5][:n], want[2][:n]) and torch.equal(got[5][half:half + items], want[2][half:half + items])
+    # and the order is what it says: every pair's row holds its token, rows of an expert ascend with the pair
+    st, slot = got[3].cpu().long(), got[4].cpu().long().flatten()
+    assert torch.equal(st[slot], torch.arange(T * k) // k)
+    flat = ids.cpu().flatten().long()
+    order = torch.argsort(flat * (T * k) + torch.arange(T * k))
+    assert bool((slot[order][1:] > slot[order][:-1]).all())
+
+
 # ------------------------------------------------------------------------------------------------ rope + cache + attention
 def paged_setup(lens, page_size, nkv, hd, n_layers, act, seed):
     """Pages handed out in a scrambled order, so that a kernel that ignores the table fails."""
